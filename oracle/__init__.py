@@ -1,0 +1,296 @@
+"""ctypes front end of the CPU oracle (liboiloracle.so) and, when built, of the
+compiled reference (oracle/_ref/liboilref*.so).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, by the smoke check and by the
+cpu_baseline leg of bench.py.  The product package never imports this module.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+FORMATS = {
+    "OIL1": 0, "SPARK_Q0": 1, "OIL2": 2, "OIL4": 3, "OIL8": 4, "OIL16": 5, "OIL32": 6,
+    "OIL1_GRP": 7, "SPARK_Q0_GRP": 8, "OIL2_GRP": 9, "OIL4_GRP": 10, "OIL8_GRP": 11,
+    "OIL16_GRP": 12, "SPARK_SPARSE": 13, "SPARK_SPARSE_GRP": 14,
+}
+FORMAT_NAMES = {v: k for k, v in FORMATS.items()}
+
+# orc_block_t
+BLOCK_DTYPE = np.dtype(
+    [("cb_off", "<u8"), ("idx_off", "<u8"), ("cb_bytes", "<u4"), ("idx_bytes", "<u4"),
+     ("nw", "<u4"), ("fmt", "u1"), ("pad", "u1", (3,))], align=True)
+assert BLOCK_DTYPE.itemsize == 32
+
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+_u16p = C.POINTER(C.c_uint16)
+
+
+def _p(a, t):
+    return a.ctypes.data_as(t)
+
+
+def build(ref: bool = False) -> None:
+    """Compile the oracle (and the compiled reference when asked and present)."""
+    subprocess.run(["make", "-C", _HERE, "liboiloracle.so"], check=True, capture_output=True)
+    if ref and os.path.isdir("/root/reference/src"):
+        subprocess.run(["make", "-C", _HERE, "ref"], check=True, capture_output=True)
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        path = os.path.join(_HERE, "liboiloracle.so")
+        if not os.path.exists(path):
+            build()
+        L = C.CDLL(path)
+        L.orc_f32_to_f16.restype = C.c_uint16
+        L.orc_f32_to_f16.argtypes = [C.c_float]
+        L.orc_f16_to_f32.restype = C.c_float
+        L.orc_f16_to_f32.argtypes = [C.c_uint16]
+        L.orc_flat_fp16_to_float.restype = C.c_float
+        L.orc_flat_fp16_to_float.argtypes = [C.c_uint16]
+        L.orc_format_bpw.restype = C.c_float
+        L.orc_format_bpw.argtypes = [C.c_int]
+        L.orc_max_payload_bytes.restype = C.c_size_t
+        L.orc_max_payload_bytes.argtypes = [C.c_int, C.c_int]
+        L.orc_quantize_block.restype = C.c_int
+        L.orc_quantize_block.argtypes = [C.c_int, _f32p, C.c_int, _u8p, C.c_size_t,
+                                         C.POINTER(C.c_size_t), _u8p, C.c_size_t,
+                                         C.POINTER(C.c_size_t)]
+        L.orc_dequantize_block.restype = None
+        L.orc_dequantize_block.argtypes = [C.c_int, _u8p, C.c_size_t, _u8p, C.c_size_t,
+                                           C.c_uint32, _f32p]
+        L.orc_quantize_tensor.restype = C.c_uint64
+        L.orc_quantize_tensor.argtypes = [_u8p, C.c_uint32, _f32p, C.c_uint64, C.c_uint32,
+                                          _u8p, C.c_uint64, C.c_void_p, C.c_int]
+        L.orc_dequant_blocks.restype = None
+        L.orc_dequant_blocks.argtypes = [_u8p, C.c_void_p, C.c_uint32, _f32p]
+        for name in ("orc_block_gemm_f32", "orc_block_gemm_f64"):
+            f = getattr(L, name)
+            f.restype = None
+            f.argtypes = [_u8p, C.c_void_p, C.c_uint32, C.c_uint32, _f32p, _f32p, C.c_int, C.c_int]
+        L.orc_oil8_gemm.restype = None
+        L.orc_oil8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.orc_oil4_gemm.restype = None
+        L.orc_oil4_gemm.argtypes = [_u8p, _u16p, _f32p, _f32p, C.c_int, C.c_int, C.c_int, C.c_int]
+        L.orc_gemv_spark.restype = None
+        L.orc_gemv_spark.argtypes = [_u8p, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+        L.orc_gemv_oil4.restype = None
+        L.orc_gemv_oil4.argtypes = [_u8p, _u16p, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+        L.orc_gemv_oil8.restype = None
+        L.orc_gemv_oil8.argtypes = [_u8p, _f32p, C.c_float, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+        L.orc_engine_quant_gemm.restype = None
+        L.orc_engine_quant_gemm.argtypes = [C.c_int, _f32p, _u8p, _f32p, _f32p,
+                                            C.c_int64, C.c_int64, C.c_int64, C.c_int]
+        _lib = L
+    return _lib
+
+
+_ref = {}
+
+
+def ref(simd: bool = True):
+    """The compiled reference, or None where it has not been built."""
+    key = "liboilref.so" if simd else "liboilref_scalar.so"
+    if key not in _ref:
+        path = os.path.join(_HERE, "_ref", key)
+        if not os.path.exists(path):
+            _ref[key] = None
+        else:
+            R = C.CDLL(path)
+            R.ref_quantize_block.restype = C.c_int
+            R.ref_quantize_block.argtypes = lib().orc_quantize_block.argtypes
+            R.ref_dequantize_block.restype = None
+            R.ref_dequantize_block.argtypes = lib().orc_dequantize_block.argtypes
+            R.ref_format_bpw.restype = C.c_float
+            R.ref_format_bpw.argtypes = [C.c_int]
+            R.ref_oil8_gemm.restype = None
+            R.ref_oil8_gemm.argtypes = [_u8p, _f32p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+            R.ref_oil4_gemm.restype = None
+            R.ref_oil4_gemm.argtypes = [_u8p, _u16p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
+            R.ref_gemv_spark.restype = None
+            R.ref_gemv_spark.argtypes = [_u8p, C.c_float, _f32p, _f32p, C.c_int, C.c_int]
+            R.ref_gemv_oil4.restype = None
+            R.ref_gemv_oil4.argtypes = [_u8p, _u16p, C.c_float, _f32p, _f32p, C.c_int, C.c_int]
+            R.ref_gemv_oil8.restype = None
+            R.ref_gemv_oil8.argtypes = [_u8p, _f32p, C.c_float, _f32p, _f32p, C.c_int, C.c_int]
+            R.ref_engine_codebook.restype = C.c_int
+            R.ref_engine_codebook.argtypes = [C.c_int, _f32p]
+            R.ref_engine_quant_gemm.restype = None
+            R.ref_engine_quant_gemm.argtypes = [C.c_int, _f32p, _u8p, _f32p,
+                                                C.c_int64, C.c_int64, C.c_int64]
+            _ref[key] = R
+    return _ref[key]
+
+
+# --------------------------------------------------------------------------- codec
+def _quantize_block(fn, fmt: int, w: np.ndarray):
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    n = w.size
+    idx = np.zeros(max(16, 4 * n + 64), dtype=np.uint8)
+    cb = np.zeros(max(16, 2 * ((n + 31) // 32) + 16), dtype=np.uint8)
+    il, cl = C.c_size_t(0), C.c_size_t(0)
+    ok = fn(fmt, _p(w, _f32p), n, _p(idx, _u8p), idx.size, C.byref(il),
+            _p(cb, _u8p), cb.size, C.byref(cl))
+    if ok != 1:
+        raise RuntimeError(f"quantize_block failed for fmt={fmt} n={n} (rc={ok})")
+    return idx[: il.value].copy(), cb[: cl.value].copy()
+
+
+def quantize_block(fmt: int, w: np.ndarray):
+    """-> (index bytes, codebook bytes) of one block."""
+    return _quantize_block(lib().orc_quantize_block, fmt, w)
+
+
+def ref_quantize_block(fmt: int, w: np.ndarray, simd: bool = True):
+    return _quantize_block(ref(simd).ref_quantize_block, fmt, w)
+
+
+def _dequantize_block(fn, fmt, idx, cb, nw, prefill=None):
+    idx = np.ascontiguousarray(idx, dtype=np.uint8)
+    cb = np.ascontiguousarray(cb, dtype=np.uint8)
+    out = np.full(nw, np.nan if prefill is None else prefill, dtype=np.float32)
+    # numpy gives a valid pointer even for empty arrays
+    fn(fmt, _p(idx, _u8p), idx.size, _p(cb, _u8p), cb.size, nw, _p(out, _f32p))
+    return out
+
+
+def dequantize_block(fmt: int, idx, cb, nw: int) -> np.ndarray:
+    return _dequantize_block(lib().orc_dequantize_block, fmt, idx, cb, nw)
+
+
+def ref_dequantize_block(fmt: int, idx, cb, nw: int, simd: bool = True) -> np.ndarray:
+    return _dequantize_block(ref(simd).ref_dequantize_block, fmt, idx, cb, nw)
+
+
+def max_payload_bytes(fmt: int, n: int) -> int:
+    return int(lib().orc_max_payload_bytes(fmt, n))
+
+
+def quantize_tensor(w: np.ndarray, fmts, align: int = 16, threads: int = 0):
+    """Quantize a flat weight array block by block.
+
+    fmts: one format id, or an array of one id per 256-block.
+    -> (payload uint8[total], blocks BLOCK_DTYPE[nblocks])
+    """
+    w = np.ascontiguousarray(w, dtype=np.float32).reshape(-1)
+    nblocks = (w.size + 255) // 256
+    if np.isscalar(fmts):
+        fmts = np.full(nblocks, int(fmts), dtype=np.uint8)
+    fmts = np.ascontiguousarray(fmts, dtype=np.uint8)
+    assert fmts.size == nblocks
+    L = lib()
+    cap = L.orc_quantize_tensor(_p(fmts, _u8p), nblocks, _p(w, _f32p), w.size, align,
+                                None, 0, None, threads)
+    if cap == 0:
+        raise RuntimeError("orc_quantize_tensor: bad arguments")
+    payload = np.zeros(cap, dtype=np.uint8)
+    blocks = np.zeros(nblocks, dtype=BLOCK_DTYPE)
+    total = L.orc_quantize_tensor(_p(fmts, _u8p), nblocks, _p(w, _f32p), w.size, align,
+                                  _p(payload, _u8p), cap, blocks.ctypes.data, threads)
+    if total == 0:
+        raise RuntimeError("orc_quantize_tensor failed")
+    return payload[:total].copy(), blocks
+
+
+def dequant_blocks(payload: np.ndarray, blocks: np.ndarray) -> np.ndarray:
+    payload = np.ascontiguousarray(payload, dtype=np.uint8)
+    blocks = np.ascontiguousarray(blocks)
+    out = np.full(int(blocks["nw"].astype(np.int64).sum()), np.nan, dtype=np.float32)
+    lib().orc_dequant_blocks(_p(payload, _u8p), blocks.ctypes.data, blocks.size, _p(out, _f32p))
+    return out
+
+
+def block_gemm(payload, blocks, rows: int, cols: int, X: np.ndarray, wide: bool = True,
+               threads: int = 0) -> np.ndarray:
+    """Y[B][rows] = X[B][cols] . W^T from block payloads.  wide=True: double
+    accumulation (the tolerance yardstick); wide=False: the reference's FP32 order."""
+    payload = np.ascontiguousarray(payload, dtype=np.uint8)
+    blocks = np.ascontiguousarray(blocks)
+    X = np.ascontiguousarray(X, dtype=np.float32).reshape(-1, cols)
+    B = X.shape[0]
+    assert cols % 256 == 0 and blocks.size == rows * (cols // 256)
+    Y = np.zeros((B, rows), dtype=np.float32)
+    fn = lib().orc_block_gemm_f64 if wide else lib().orc_block_gemm_f32
+    fn(_p(payload, _u8p), blocks.ctypes.data, rows, cols, _p(X, _f32p), _p(Y, _f32p), B, threads)
+    return Y
+
+
+# ------------------------------------------------------------------- flat kernels
+def oil8_gemm(idx, cb, act, M, N, K, order=0):
+    idx = np.ascontiguousarray(idx, dtype=np.uint8)
+    cb = np.ascontiguousarray(cb, dtype=np.float32)
+    act = np.ascontiguousarray(act, dtype=np.float32)
+    out = np.zeros(M * N, dtype=np.float32)
+    lib().orc_oil8_gemm(_p(idx, _u8p), _p(cb, _f32p), _p(act, _f32p), _p(out, _f32p), M, N, K, order)
+    return out.reshape(M, N)
+
+
+def oil4_gemm(packed, cb16, act, M, N, K, order=0):
+    packed = np.ascontiguousarray(packed, dtype=np.uint8)
+    cb16 = np.ascontiguousarray(cb16, dtype=np.uint16)
+    act = np.ascontiguousarray(act, dtype=np.float32)
+    out = np.zeros(M * N, dtype=np.float32)
+    lib().orc_oil4_gemm(_p(packed, _u8p), _p(cb16, _u16p), _p(act, _f32p), _p(out, _f32p), M, N, K, order)
+    return out.reshape(M, N)
+
+
+def gemv_spark(w, scale, x, M, K, mode=0):
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.zeros(M, dtype=np.float32)
+    lib().orc_gemv_spark(_p(w, _u8p), scale, _p(x, _f32p), _p(y, _f32p), M, K, int(mode))
+    return y
+
+
+def gemv_oil4(w, cb16, scale, x, M, K, mode=0):
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    cb16 = np.ascontiguousarray(cb16, dtype=np.uint16)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.zeros(M, dtype=np.float32)
+    lib().orc_gemv_oil4(_p(w, _u8p), _p(cb16, _u16p), scale, _p(x, _f32p), _p(y, _f32p), M, K, int(mode))
+    return y
+
+
+def gemv_oil8(w, cb, scale, x, M, K, mode=0):
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    cb = np.ascontiguousarray(cb, dtype=np.float32)
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    y = np.zeros(M, dtype=np.float32)
+    lib().orc_gemv_oil8(_p(w, _u8p), _p(cb, _f32p), scale, _p(x, _f32p), _p(y, _f32p), M, K, int(mode))
+    return y
+
+
+def engine_quant_gemm(bits, A, b_idx, cb, M, N, K, as_double=False):
+    A = np.ascontiguousarray(A, dtype=np.float32)
+    b_idx = np.ascontiguousarray(b_idx, dtype=np.uint8)
+    cb = np.ascontiguousarray(cb, dtype=np.float32)
+    out = np.zeros(M * N, dtype=np.float32)
+    lib().orc_engine_quant_gemm(bits, _p(A, _f32p), _p(b_idx, _u8p), _p(cb, _f32p), _p(out, _f32p),
+                                M, N, K, int(as_double))
+    return out.reshape(M, N)
+
+
+# --------------------------------------------------------------- test generators
+def xorshift_fill(n: int, seed: int) -> np.ndarray:
+    """The reference codec test's deterministic generator
+    (tests/test_block_codec.cpp:49-55): uniform in [-1, 1]."""
+    state = (seed * 2654435761 + 12345) & 0xFFFFFFFF
+    out = np.empty(n, dtype=np.float32)
+    f = np.float32
+    for i in range(n):
+        state ^= (state << 13) & 0xFFFFFFFF
+        state ^= state >> 17
+        state ^= (state << 5) & 0xFFFFFFFF
+        out[i] = (f(state & 0xFFFF) / f(65535.0) - f(0.5)) * f(2.0)
+    return out

@@ -1,0 +1,142 @@
+/*
+ * oil_oracle.h -- CPU oracle for the OIL quantized-weight matmul path.
+ *
+ * TEST INFRASTRUCTURE ONLY.  This library is the checker that the HIP path is
+ * compared against (tests/, the smoke check and the cpu_baseline leg of the
+ * benchmark).  The product (innova_amd/, liboilhip.so) never links, loads or
+ * calls anything declared here.
+ *
+ * Every function restates, in plain C, the arithmetic of one reference routine
+ * (cited per function, paths relative to the reference tree).  The reference is
+ * built with -mfma and g++'s default -ffp-contract=fast, so expressions of the
+ * form a*b+c in it are fused; this file is compiled with -ffp-contract=off and
+ * spells each such fusion as an explicit fmaf()/fma() call.
+ */
+#ifndef OIL_ORACLE_H
+#define OIL_ORACLE_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Format ids: include/oil/types.h:19-35 */
+enum {
+    ORC_OIL1 = 0, ORC_SPARK_Q0 = 1, ORC_OIL2 = 2, ORC_OIL4 = 3, ORC_OIL8 = 4,
+    ORC_OIL16 = 5, ORC_OIL32 = 6, ORC_OIL1_GRP = 7, ORC_SPARK_Q0_GRP = 8,
+    ORC_OIL2_GRP = 9, ORC_OIL4_GRP = 10, ORC_OIL8_GRP = 11, ORC_OIL16_GRP = 12,
+    ORC_SPARK_SPARSE = 13, ORC_SPARK_SPARSE_GRP = 14, ORC_NUM_FORMATS = 15
+};
+
+/* src/block_codec.cpp:26-84 */
+uint16_t orc_f32_to_f16(float v);
+float    orc_f16_to_f32(uint16_t h);
+
+/* include/oil/types.h:57-82 (claimed bits per weight) */
+float orc_format_bpw(int fmt);
+
+/* Largest payload (indices + codebook bytes) quantize can emit for n weights. */
+size_t orc_max_payload_bytes(int fmt, int n);
+
+/* src/block_codec.cpp:368-574.  Returns 1 on success, 0 for bad arguments /
+ * unknown format / too-small output buffers.  *idx_len / *cb_len receive the
+ * byte counts written. */
+int orc_quantize_block(int fmt, const float* w, int n,
+                       uint8_t* idx, size_t idx_cap, size_t* idx_len,
+                       uint8_t* cb, size_t cb_cap, size_t* cb_len);
+
+/* src/block_codec.cpp:576-720.  Zero-fills out[0..nw) first; reads beyond the
+ * payload behave as zero bits. */
+void orc_dequantize_block(int fmt, const uint8_t* idx, size_t idx_bytes,
+                          const uint8_t* cb, size_t cb_bytes,
+                          uint32_t nw, float* out);
+
+/*
+ * A quantized matrix as the block-decode consumer sees it
+ * (src/adapters/tools/qwen35_engine.cpp:17-28,47-85): rows x cols weights,
+ * cols a multiple of 256, block id = row * (cols/256) + blk.  Each block is
+ * described by where its codebook bytes and index bytes start inside `payload`.
+ */
+typedef struct {
+    uint64_t cb_off;     /* byte offset of the codebook channel in payload */
+    uint64_t idx_off;    /* byte offset of the index channel in payload   */
+    uint32_t cb_bytes;
+    uint32_t idx_bytes;
+    uint32_t nw;         /* weights in this block                          */
+    uint8_t  fmt;
+    uint8_t  pad_[3];
+} orc_block_t;
+
+/* Tensor-level quantize: block b covers w[b*256 .. min(numel, b*256+256)) and is
+ * encoded with fmts[b]; each block's bytes (codebook channel, then index
+ * channel) are appended to `payload` at the next multiple of `align`
+ * (src/format_registry.cpp:158-197 is the same per-256 loop).  Fills
+ * blocks[0..nblocks) and returns the total byte count; with payload == NULL
+ * only returns an upper bound on the capacity needed.  Returns 0 on error. */
+uint64_t orc_quantize_tensor(const uint8_t* fmts, uint32_t nblocks,
+                             const float* w, uint64_t numel, uint32_t align,
+                             uint8_t* payload, uint64_t cap, orc_block_t* blocks,
+                             int threads);
+
+/* Dequantize blocks [0, nblocks) back to back into out (sum of nw floats).
+ * src/oil_format.cpp:464-477 (read_tensor's loop). */
+void orc_dequant_blocks(const uint8_t* payload, const orc_block_t* blocks,
+                        uint32_t nblocks, float* out);
+
+/* Y[b*rows + r] = sum over blocks of (sum_j W[r][blk*256+j] * X[b*cols + blk*256+j]).
+ * FP32 in the reference's own order: per block a sequential fused
+ * multiply-add chain from 0, then added to the row accumulator
+ * (qwen35_engine.cpp:66-80).  threads <= 0 means min(8, online cpus)
+ * (qwen35_engine.cpp:50-52); rows are split in contiguous chunks. */
+void orc_block_gemm_f32(const uint8_t* payload, const orc_block_t* blocks,
+                        uint32_t rows, uint32_t cols,
+                        const float* X, float* Y, int B, int threads);
+
+/* Same contraction with every product and sum in double, rounded once to float
+ * at the end: the yardstick the GEMV/GEMM tolerances are measured against. */
+void orc_block_gemm_f64(const uint8_t* payload, const orc_block_t* blocks,
+                        uint32_t rows, uint32_t cols,
+                        const float* X, float* Y, int B, int threads);
+
+/* Flat-codebook kernels.
+ * oil8: out[m*N+n] = sum_k cb[idx[n*K+k]] * act[m*K+k]   (src/kernel_oil8.cpp:14-32)
+ * oil4: out[m*N+n] = sum_k c16[nib((m*N+n)*K + k)] * act[n*K+k]
+ *       (src/kernel_oil4.cpp:31-60; weights are indexed per (m,n) pair and
+ *       activations per n, exactly as the reference does).
+ * order = 0: scalar left-to-right fused chain; order = 1: the AVX2 path's
+ * 8-lane accumulators + horizontal add + scalar tail
+ * (kernel_oil8.cpp:35-68, kernel_oil4.cpp:63-117); order = 2: double. */
+void orc_oil8_gemm(const uint8_t* idx, const float* cb, const float* act,
+                   float* out, int M, int N, int K, int order);
+void orc_oil4_gemm(const uint8_t* packed, const uint16_t* cb16, const float* act,
+                   float* out, int M, int N, int K, int order);
+/* src/kernel_oil4.cpp:15-29 */
+float orc_flat_fp16_to_float(uint16_t h);
+
+/* Production GEMVs, scalar bodies (src/kernel_production.cpp:79-128):
+ * y[m] = scale * sum_k dec(W[m][k]) * x[k].
+ * mode 0: FP32 chain with each multiply-add fused (a build with -mfma);
+ * mode 1: double accumulation; mode 2: FP32 chain with separately rounded
+ * multiply and add (a build without FMA flags). */
+void orc_gemv_spark(const uint8_t* w, float scale, const float* x, float* y,
+                    int M, int K, int mode);
+void orc_gemv_oil4(const uint8_t* w, const uint16_t* cb16, float scale,
+                   const float* x, float* y, int M, int K, int mode);
+void orc_gemv_oil8(const uint8_t* w, const float* cb, float scale,
+                   const float* x, float* y, int M, int K, int mode);
+
+/* Engine quant_gemm, [K][N] index layout:
+ * C[m*N+n] = sum_k A[m*K+k] * cb[code(k*N+n)], terms with A == 0 skipped,
+ * accumulation in k order (src/oil_engines_oil8.cpp:197-216,
+ * oil_engines_oil4.cpp:238-261, oil_engines_oil2.cpp:210-229).
+ * bits in {2,4,8}; as_double != 0 accumulates in double. */
+void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
+                           const float* cb, float* C,
+                           int64_t M, int64_t N, int64_t K, int as_double);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,182 @@
+#!/usr/bin/env python3
+"""Write tests/golden/*.npz from the COMPILED REFERENCE (oracle/_ref/liboilref*.so).
+
+Run in the build container only (the reference tree is needed to build
+oracle/_ref):   make -C oracle ref && python tests/golden/make_fixtures.py
+
+Inputs follow the reference codec test's deterministic generator
+(tests/test_block_codec.cpp:49-55, seeds 42 / 1337 / 1000+n, :176 tail sizes,
+:247-250 the dense*0.85+0.6 transform) plus a x0.02 variant in the spirit of the
+N(0,0.02) recipe; outputs are what the reference's quantize_block_all /
+dequantize_block_all / oil4_gemm / oil8_gemm / gemv_*_tiled / quant_gemm
+produced for them.  The fixtures hold data only: inputs, payload bytes and
+output bit patterns.
+"""
+import ctypes as C
+import os
+import sys
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+sys.path.insert(0, ROOT)
+import oracle as O  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+TAILS = [1, 7, 15, 16, 17, 20, 21, 25, 26, 31, 32, 33, 39, 40, 63, 100, 128, 200, 255]
+
+f32p = C.POINTER(C.c_float)
+u8p = C.POINTER(C.c_uint8)
+u16p = C.POINTER(C.c_uint16)
+
+
+def p(a, t):
+    return a.ctypes.data_as(t)
+
+
+def codec_inputs():
+    """(tag, weights) pairs."""
+    cases = []
+    w256 = O.xorshift_fill(256, 42) * np.float32(0.85) + np.float32(0.6)
+    w512 = O.xorshift_fill(512, 1337) * np.float32(0.85) + np.float32(0.6)
+    cases.append(("dense256", w256))
+    cases.append(("dense512", w512))
+    cases.append(("unit256", O.xorshift_fill(256, 99)))
+    cases.append(("small256", O.xorshift_fill(256, 7) * np.float32(0.02)))
+    cases.append(("zero256", np.zeros(256, dtype=np.float32)))
+    spike = O.xorshift_fill(256, 11) * np.float32(0.02)
+    spike[::37] *= np.float32(40.0)
+    cases.append(("spiky256", spike))
+    cases.append(("tiny256", O.xorshift_fill(256, 5) * np.float32(3e-8)))   # FP16 scale flushes
+    for n in TAILS:
+        cases.append((f"tail{n}", O.xorshift_fill(n, 1000 + n)))
+        cases.append((f"tail{n}s", O.xorshift_fill(n, 2000 + n) * np.float32(0.02)))
+    return cases
+
+
+def make_codec():
+    R = O.ref(True)
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    rec = {k: [] for k in ("fmt", "n", "w_off", "idx_off", "idx_len", "cb_off", "cb_len", "dec_off")}
+    tags, W, IDX, CB, DEC = [], [], [], [], []
+    w_off = idx_off = cb_off = dec_off = 0
+    for tag, w in codec_inputs():
+        for fmt in range(15):
+            idx, cb = O.ref_quantize_block(fmt, w)
+            dec = O.ref_dequantize_block(fmt, idx, cb, w.size)
+            tags.append(f"{tag}/{O.FORMAT_NAMES[fmt]}")
+            rec["fmt"].append(fmt); rec["n"].append(w.size)
+            rec["w_off"].append(w_off); rec["idx_off"].append(idx_off); rec["idx_len"].append(idx.size)
+            rec["cb_off"].append(cb_off); rec["cb_len"].append(cb.size); rec["dec_off"].append(dec_off)
+            IDX.append(idx); CB.append(cb); DEC.append(dec.view(np.uint32))
+            idx_off += idx.size; cb_off += cb.size; dec_off += dec.size
+        W.append(w.view(np.uint32)); w_off += w.size
+    out = {k: np.asarray(v, dtype=np.int64) for k, v in rec.items()}
+    out["tags"] = np.asarray(tags)
+    out["w_bits"] = np.concatenate(W)
+    out["idx"] = np.concatenate(IDX)
+    out["cb"] = np.concatenate(CB)
+    out["dec_bits"] = np.concatenate(DEC)
+    # all 65536 half patterns through the reference's OIL16 decode
+    hs = np.arange(65536, dtype=np.uint16)
+    out["f16_to_f32_bits"] = O.ref_dequantize_block(5, hs.view(np.uint8), np.zeros(0, np.uint8), 65536).view(np.uint32)
+    # float -> half: a spread of magnitudes, ties and specials through OIL16 encode
+    rng = np.random.default_rng(20260803)
+    f = np.concatenate([
+        (rng.standard_normal(4096) * 10.0 ** rng.integers(-9, 6, 4096)).astype(np.float32),
+        rng.integers(0, 1 << 32, 4096, dtype=np.uint64).astype(np.uint32).view(np.float32),
+        ((np.arange(0, 4096, dtype=np.uint32) << 13) | 0x38000000 | 0x1000).view(np.float32),
+        np.array([0.0, -0.0, np.inf, -np.inf, np.nan, 65504, 65520, 65519.99, 6.1e-5, 5.96e-8,
+                  2.98e-8, 2.9e-8, 3.1e-8, 1e-10], dtype=np.float32)])
+    h = np.concatenate([O.ref_quantize_block(5, f[s:s + 4096])[0] for s in range(0, f.size, 4096)])
+    out["f32_in_bits"] = f.view(np.uint32)
+    out["f32_to_f16"] = h.view(np.uint16)
+    np.savez_compressed(os.path.join(HERE, "codec.npz"), **out)
+    print("codec.npz:", len(tags), "cases")
+
+
+def make_gemv():
+    """Per format: a 32 x 768 matrix, reference payloads, reference decode,
+    double-precision X.W^T of the reference-decoded weights (B = 3)."""
+    R = O.ref(True)
+    rows, cols, B = 32, 768, 3
+    rng = np.random.default_rng(7)
+    Wm = (rng.standard_normal(rows * cols) * 0.02).astype(np.float32)
+    Wm[rng.integers(0, Wm.size, 200)] *= np.float32(8.0)
+    X = rng.standard_normal((B, cols)).astype(np.float32)
+    out = {"w_bits": Wm.view(np.uint32), "x_bits": X.view(np.uint32),
+           "shape": np.array([rows, cols, B])}
+    for fmt in range(15):
+        idxs, cbs, decs = [], [], []
+        for b in range(rows * cols // 256):
+            idx, cb = O.ref_quantize_block(fmt, Wm[b * 256:(b + 1) * 256])
+            idxs.append(idx); cbs.append(cb)
+            decs.append(O.ref_dequantize_block(fmt, idx, cb, 256))
+        Wd = np.concatenate(decs).reshape(rows, cols)
+        Y = (X.astype(np.float64) @ Wd.astype(np.float64).T).astype(np.float32)
+        name = O.FORMAT_NAMES[fmt]
+        out[f"{name}/idx"] = np.concatenate(idxs)
+        out[f"{name}/idx_len"] = np.array([a.size for a in idxs], dtype=np.int32)
+        out[f"{name}/cb"] = np.concatenate(cbs) if sum(a.size for a in cbs) else np.zeros(0, np.uint8)
+        out[f"{name}/cb_len"] = np.array([a.size for a in cbs], dtype=np.int32)
+        out[f"{name}/y_bits"] = Y.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "block_gemv.npz"), **out)
+    print("block_gemv.npz written")
+
+
+def make_flat():
+    R, RS = O.ref(True), O.ref(False)
+    rng = np.random.default_rng(11)
+    out = {}
+    # oil8_gemm / oil4_gemm (AVX2 build)
+    M, N, K = 3, 17, 300
+    idx8 = rng.integers(0, 256, N * K, dtype=np.uint8).astype(np.uint8)
+    cb8 = rng.standard_normal(256).astype(np.float32)
+    act8 = rng.standard_normal(M * K).astype(np.float32)
+    y8 = np.zeros(M * N, np.float32)
+    R.ref_oil8_gemm(p(idx8, u8p), p(cb8, f32p), p(act8, f32p), p(y8, f32p), M, N, K)
+    out.update({"oil8/idx": idx8, "oil8/cb_bits": cb8.view(np.uint32), "oil8/act_bits": act8.view(np.uint32),
+                "oil8/y_bits": y8.view(np.uint32), "oil8/mnk": np.array([M, N, K])})
+    pk = rng.integers(0, 256, M * N * K // 2 + 16, dtype=np.uint8).astype(np.uint8)
+    cb16 = rng.standard_normal(16).astype(np.float16).view(np.uint16).copy()
+    cb16[3] = 0x0001; cb16[5] = 0x83FF; cb16[9] = 0x0400
+    act4 = rng.standard_normal(N * K).astype(np.float32)
+    y4 = np.zeros(M * N, np.float32)
+    R.ref_oil4_gemm(p(pk, u8p), p(cb16, u16p), p(act4, f32p), p(y4, f32p), M, N, K)
+    out.update({"oil4/packed": pk, "oil4/cb16": cb16, "oil4/act_bits": act4.view(np.uint32),
+                "oil4/y_bits": y4.view(np.uint32), "oil4/mnk": np.array([M, N, K])})
+    # production GEMVs: scalar bodies (reference built without SIMD flags)
+    Mg, Kg = 9, 301
+    x = rng.standard_normal(Kg).astype(np.float32)
+    ws = rng.integers(0, 256, Mg * ((Kg + 3) // 4), dtype=np.uint8).astype(np.uint8)
+    w4 = rng.integers(0, 256, Mg * ((Kg + 1) // 2), dtype=np.uint8).astype(np.uint8)
+    w8 = rng.integers(0, 256, Mg * Kg, dtype=np.uint8).astype(np.uint8)
+    ys, yo4, yo8 = (np.zeros(Mg, np.float32) for _ in range(3))
+    RS.ref_gemv_spark(p(ws, u8p), 0.37, p(x, f32p), p(ys, f32p), Mg, Kg)
+    RS.ref_gemv_oil4(p(w4, u8p), p(cb16, u16p), 0.37, p(x, f32p), p(yo4, f32p), Mg, Kg)
+    RS.ref_gemv_oil8(p(w8, u8p), p(cb8, f32p), 0.37, p(x, f32p), p(yo8, f32p), Mg, Kg)
+    out.update({"prod/x_bits": x.view(np.uint32), "prod/mk": np.array([Mg, Kg]),
+                "prod/w_spark": ws, "prod/w_oil4": w4, "prod/w_oil8": w8,
+                "prod/y_spark_bits": ys.view(np.uint32), "prod/y_oil4_bits": yo4.view(np.uint32),
+                "prod/y_oil8_bits": yo8.view(np.uint32)})
+    # engines: default codebooks and quant_gemm
+    Me, Ne, Ke = 3, 24, 40
+    A = rng.standard_normal(Me * Ke).astype(np.float32)
+    A[::7] = 0
+    bq = rng.integers(0, 256, Ke * Ne, dtype=np.uint8).astype(np.uint8)
+    out.update({"eng/A_bits": A.view(np.uint32), "eng/b": bq, "eng/mnk": np.array([Me, Ne, Ke])})
+    for bits in (8, 4, 2):
+        cb = np.zeros(256, np.float32)
+        n = R.ref_engine_codebook(bits, p(cb, f32p))
+        Cc = np.zeros(Me * Ne, np.float32)
+        R.ref_engine_quant_gemm(bits, p(A, f32p), p(bq, u8p), p(Cc, f32p), Me, Ne, Ke)
+        out[f"eng/cb{bits}_bits"] = cb[:n].view(np.uint32).copy()
+        out[f"eng/c{bits}_bits"] = Cc.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "flat.npz"), **out)
+    print("flat.npz written")
+
+
+if __name__ == "__main__":
+    make_codec()
+    make_gemv()
+    make_flat()
