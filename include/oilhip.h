@@ -1,0 +1,148 @@
+/*
+ * oilhip.h -- C ABI of the MI355X (gfx950) OIL quantized-weight matmul library.
+ *
+ * Plain pointers and sizes only.  Every function returns 0 on success and a
+ * negative OILHIP_E_* code on failure; oilhip_last_error() then describes the
+ * failure for the calling thread.  Pointers named d_* are device (HBM)
+ * pointers, all others are host pointers.  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream); calls are asynchronous on that stream
+ * unless stated otherwise.
+ *
+ * Each entry point names the reference interface it stands in for
+ * (file:line relative to the reference tree).
+ */
+#ifndef OILHIP_H
+#define OILHIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define OILHIP_OK            0
+#define OILHIP_E_ARG        -1   /* bad argument / shape / unsupported combination */
+#define OILHIP_E_DEVICE     -2   /* a HIP call failed                              */
+#define OILHIP_E_NOGPU      -3   /* no gfx950 device visible                       */
+#define OILHIP_E_NOMEM      -4
+
+/* Wire formats, numbered as oil::Format (include/oil/types.h:19-35). */
+enum {
+    OILHIP_OIL1 = 0, OILHIP_SPARK_Q0 = 1, OILHIP_OIL2 = 2, OILHIP_OIL4 = 3, OILHIP_OIL8 = 4,
+    OILHIP_OIL16 = 5, OILHIP_OIL32 = 6, OILHIP_OIL1_GRP = 7, OILHIP_SPARK_Q0_GRP = 8,
+    OILHIP_OIL2_GRP = 9, OILHIP_OIL4_GRP = 10, OILHIP_OIL8_GRP = 11, OILHIP_OIL16_GRP = 12,
+    OILHIP_SPARK_SPARSE = 13, OILHIP_SPARK_SPARSE_GRP = 14, OILHIP_NUM_FORMATS = 15
+};
+
+const char* oilhip_last_error(void);
+
+/* Runtime probe of the device path: the counterpart of detect_cpu_isa()
+ * (include/oil/kernel_production.h:19) and probe_hardware()
+ * (include/oil/backend.h:98-139, src/backend.cpp:672-730).  Any out pointer
+ * may be NULL.  gfx receives 950 on MI355X.  Synchronous. */
+int oilhip_probe(int* gfx, uint64_t* hbm_bytes, int* compute_units, char* name, size_t name_cap);
+
+/* ---------------------------------------------------------------- host codec
+ * The reference quantizer runs on the CPU (it is the producer of .oil files,
+ * not part of the accelerated path); these are its host-side counterparts.
+ * oilhip_quantize_block  : quantize_block_all   (include/oil/block_codec.h:55-56)
+ * oilhip_payload_bound   : upper bound of idx+cb bytes for n weights
+ * oilhip_quantize_tensor : the per-256-block loop of FormatRegistry::quantize
+ *                          (src/format_registry.cpp:158-197)                    */
+typedef struct {
+    uint64_t cb_off;      /* byte offset of the block's codebook channel in the payload */
+    uint64_t idx_off;     /* byte offset of the block's index channel in the payload    */
+    uint32_t cb_bytes;
+    uint32_t idx_bytes;
+    uint32_t nw;          /* weights in the block */
+    uint8_t  fmt;         /* OILHIP_* format id   */
+    uint8_t  reserved[3];
+} oilhip_block_t;
+
+size_t oilhip_payload_bound(int fmt, int n);
+int oilhip_quantize_block(int fmt, const float* w, int n,
+                          uint8_t* idx, size_t idx_cap, size_t* idx_len,
+                          uint8_t* cb, size_t cb_cap, size_t* cb_len);
+/* Block b covers w[b*256 ..) and is encoded as fmts[b]; payloads are appended
+ * 16-byte aligned (codebook channel then index channel).  With payload == NULL
+ * returns only the capacity bound in *total.  threads <= 0: all host cores. */
+int oilhip_quantize_tensor(const uint8_t* fmts, uint32_t nblocks, const float* w, uint64_t numel,
+                           uint8_t* payload, uint64_t cap, oilhip_block_t* blocks,
+                           uint64_t* total, int threads);
+
+/* ------------------------------------------------------------- device weights
+ * A quantized tensor resident in HBM: block payloads byte-identical to the
+ * .oil file's, framing stripped into a descriptor table, uploaded once.
+ * Stands in for OILReader::block_ptr/format_entry + Qwen35Engine::Th{start,
+ * count,fmt,rows,cols} (src/oil_format.cpp:416-421, include/oil/oil_format.h:80-83,
+ * include/oil/qwen35_engine.h:29).  rows*cols must equal the sum of nw; for the
+ * matmul entry points cols must be a multiple of 256 and every block full.
+ * Synchronous (returns after the upload). */
+typedef struct oilhip_weights oilhip_weights;
+
+int oilhip_weights_create(const uint8_t* payload, uint64_t payload_bytes,
+                          const oilhip_block_t* blocks, uint32_t nblocks,
+                          uint64_t rows, uint64_t cols, oilhip_weights** out);
+
+/* Same, parsing on-disk block records [nw u32][cb_bytes u32][cb][idx_bytes u32][idx]
+ * (src/oil_format.cpp:219-233) laid end to end, with the per-block format ids
+ * from the file's format table (src/oil_format.cpp:329-350). */
+int oilhip_weights_create_from_records(const uint8_t* records, uint64_t record_bytes,
+                                       const uint8_t* fmts, uint32_t nblocks,
+                                       uint64_t rows, uint64_t cols, oilhip_weights** out);
+
+int oilhip_weights_destroy(oilhip_weights* w);
+
+/* Facts about an uploaded tensor.  payload_bytes = sum of cb_bytes + idx_bytes
+ * (the algorithmic weight bytes); uniform_fmt = the single format id or -1 for a
+ * mixed tensor.  Any out pointer may be NULL. */
+int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols,
+                        uint32_t* nblocks, uint64_t* payload_bytes, int* uniform_fmt);
+
+/* dequantize_block_all over every block, back to back (include/oil/block_codec.h:60-63,
+ * OILReader::read_tensor src/oil_format.cpp:464-477).  d_out holds rows*cols
+ * floats.  Bit-exact with the reference decode. */
+int oilhip_dequant_f32(const oilhip_weights* w, float* d_out, void* stream);
+
+/* Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:47-85):
+ * d_y[b*rows + r] = sum_c W[r][c] * d_x[b*cols + c], FP32 in, FP32 out,
+ * FP32 accumulation, 1 <= M (the reference caps a call at 512). */
+int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream);
+
+/* Prefill form of the same contraction: activations as bf16 bit patterns,
+ * weights dequantized to bf16 in LDS, MFMA with FP32 accumulation, FP32 out.
+ * (The reference has no bf16 path; its FP32 prefill loop is
+ * qwen35_engine.cpp:630-753 over the same gemm.) */
+int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x_bf16, float* d_y, int M, void* stream);
+
+/* ---------------------------------------------------- flat-codebook kernels
+ * oil::kernel::oil8_gemm (include/oil/kernel.h:24-26, src/kernel_oil8.cpp:71-79):
+ *   out[m*N+n] = sum_k cb[idx[n*K+k]] * act[m*K+k]
+ * oil::kernel::oil4_gemm (include/oil/kernel.h:30-32, src/kernel_oil4.cpp:120-128):
+ *   out[m*N+n] = sum_k f16(cb[nib((m*N+n)*K+k)]) * act[n*K+k]                   */
+int oilhip_flat_oil8_gemm(const uint8_t* d_idx, const float* d_cb256, const float* d_act,
+                          float* d_out, int M, int N, int K, void* stream);
+int oilhip_flat_oil4_gemm(const uint8_t* d_packed, const uint16_t* d_cb16, const float* d_act,
+                          float* d_out, int M, int N, int K, void* stream);
+
+/* oil::adapters::prod::gemv_{spark,oil4,oil8}_tiled / _batch
+ * (include/oil/kernel_production.h:25-52; scalar bodies src/kernel_production.cpp:79-128):
+ *   Y[n*M + m] = scale * sum_k dec(W[m][k]) * X[n*K + k],  n < batch            */
+int oilhip_prod_gemv_spark(const uint8_t* d_w, float scale, const float* d_x, float* d_y,
+                           int M, int K, int batch, void* stream);
+int oilhip_prod_gemv_oil4(const uint8_t* d_w, const uint16_t* d_cb16, float scale, const float* d_x,
+                          float* d_y, int M, int K, int batch, void* stream);
+int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb256, float scale, const float* d_x,
+                          float* d_y, int M, int K, int batch, void* stream);
+
+/* oil::engines::OIL{8,4,2}Engine::quant_gemm (include/oil/oil_engines.h:49,78,151;
+ * src/oil_engines_oil8.cpp:197-216, oil4.cpp:238-261, oil2.cpp:210-229):
+ *   C[m*N+n] = sum_k A[m*K+k] * cb[code(k*N+n)],  [K][N] packed codes, bits in {2,4,8} */
+int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b_idx, const float* d_cb,
+                             float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

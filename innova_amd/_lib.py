@@ -1,0 +1,92 @@
+"""ctypes binding of liboilhip.so.  There is no fallback: if the library has not
+been built the import of a kernel entry point fails loudly."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "liboilhip.so")
+
+u8p = C.POINTER(C.c_uint8)
+f32p = C.POINTER(C.c_float)
+vp = C.c_void_p
+
+# oilhip_block_t
+BLOCK_DTYPE = np.dtype(
+    [("cb_off", "<u8"), ("idx_off", "<u8"), ("cb_bytes", "<u4"), ("idx_bytes", "<u4"),
+     ("nw", "<u4"), ("fmt", "u1"), ("reserved", "u1", (3,))], align=True)
+assert BLOCK_DTYPE.itemsize == 32
+
+
+class OilHipError(RuntimeError):
+    """A liboilhip call failed (the counterpart of oil::Error, include/oil/types.h:184-190)."""
+
+
+_lib = None
+
+_SIGNATURES = {
+    "oilhip_last_error": (C.c_char_p, []),
+    "oilhip_probe": (C.c_int, [C.POINTER(C.c_int), C.POINTER(C.c_uint64), C.POINTER(C.c_int), C.c_char_p, C.c_size_t]),
+    "oilhip_payload_bound": (C.c_size_t, [C.c_int, C.c_int]),
+    "oilhip_quantize_block": (C.c_int, [C.c_int, vp, C.c_int, vp, C.c_size_t, C.POINTER(C.c_size_t),
+                                        vp, C.c_size_t, C.POINTER(C.c_size_t)]),
+    "oilhip_quantize_tensor": (C.c_int, [vp, C.c_uint32, vp, C.c_uint64, vp, C.c_uint64, vp,
+                                         C.POINTER(C.c_uint64), C.c_int]),
+    "oilhip_weights_create": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
+    "oilhip_weights_create_from_records": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
+    "oilhip_weights_destroy": (C.c_int, [vp]),
+    "oilhip_weights_info": (C.c_int, [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint32),
+                                      C.POINTER(C.c_uint64), C.POINTER(C.c_int)]),
+    "oilhip_dequant_f32": (C.c_int, [vp, vp, vp]),
+    "oilhip_gemv_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_gemv_f32_general": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_gemm_bf16": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_flat_oil8_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_flat_oil4_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_prod_gemv_spark": (C.c_int, [vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_prod_gemv_oil4": (C.c_int, [vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_prod_gemv_oil8": (C.c_int, [vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_engine_quant_gemm": (C.c_int, [C.c_int, vp, vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
+}
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise OilHipError(
+                f"{LIB_PATH} is missing: build it first (make -C innova_amd/csrc, or "
+                "python -c 'import __graft_entry__ as g; g.build()'); there is no CPU fallback")
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = L
+    return _lib
+
+
+def exported_symbols():
+    return list(_SIGNATURES)
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        raise OilHipError(f"liboilhip error {rc}: {lib().oilhip_last_error().decode(errors='replace')}")
+
+
+def probe() -> dict:
+    """Runtime probe of the device path (cf. detect_cpu_isa / probe_hardware)."""
+    gfx, hbm, cus = C.c_int(0), C.c_uint64(0), C.c_int(0)
+    name = C.create_string_buffer(256)
+    check(lib().oilhip_probe(C.byref(gfx), C.byref(hbm), C.byref(cus), name, 256))
+    return {"gfx": gfx.value, "hbm_bytes": hbm.value, "compute_units": cus.value, "name": name.value.decode()}
+
+
+def current_stream() -> int:
+    import torch
+    return torch.cuda.current_stream().cuda_stream

@@ -1,0 +1,255 @@
+// api.hip -- C ABI of liboilhip: error text, device probe, weight upload, dispatch.
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "common.h"
+
+namespace oilhip {
+
+static thread_local std::string g_err;
+
+void set_error(const std::string& msg) { g_err = msg; }
+int fail(int code, const std::string& msg) {
+    g_err = msg;
+    return code;
+}
+
+// ---- decode tables: the reference's expressions evaluated once on the host ----
+static std::mutex g_mu;
+static const DecodeTables* g_tables[64] = {};
+static int g_cus[64] = {};
+
+int get_tables(const DecodeTables** out) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_mu);
+    if (!g_tables[dev]) {
+        DecodeTables h;
+        for (int q = 0; q < 256; ++q) {
+            volatile float num = 16.0f * (float)q;          // block_codec.cpp:131: mul, div, add
+            volatile float quo = num / 255.0f;
+            h.lv8[q] = -8.0f + quo;
+            volatile float t = (float)q / 255.0f;           // :326
+            h.t255[q] = t;
+            volatile float u = (float)q / 127.5f;           // :338
+            h.t1275[q] = u - 1.0f;
+            volatile float s = (float)(int8_t)(uint8_t)q / 127.0f;   // :690
+            h.q127[q] = s;
+        }
+        DecodeTables* d = nullptr;
+        OILHIP_HIP(hipMalloc(&d, sizeof(DecodeTables)));
+        OILHIP_HIP(hipMemcpy(d, &h, sizeof(DecodeTables), hipMemcpyHostToDevice));
+        g_tables[dev] = d;
+    }
+    *out = g_tables[dev];
+    return OILHIP_OK;
+}
+
+int device_cu_count() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    if (!g_cus[dev]) {
+        hipDeviceProp_t p;
+        g_cus[dev] = (hipGetDeviceProperties(&p, dev) == hipSuccess && p.multiProcessorCount > 0)
+                         ? p.multiProcessorCount : 256;
+    }
+    return g_cus[dev];
+}
+
+static int check_matmul_shape(const oilhip_weights* w, const void* x, const void* y, int M) {
+    if (!w || !x || !y) return fail(OILHIP_E_ARG, "null argument");
+    if (M < 1) return fail(OILHIP_E_ARG, "M must be >= 1");
+    if (!w->all_full || (w->cols % 256) != 0 || w->cols == 0 || w->rows == 0)
+        return fail(OILHIP_E_ARG, "matmul needs cols a positive multiple of 256 and only full 256-weight blocks");
+    if ((uint64_t)w->nblocks != w->rows * (w->cols / 256))
+        return fail(OILHIP_E_ARG, "block count does not match rows * cols / 256");
+    if (w->rows > 0xFFFFFFFFull || w->cols > 0xFFFFFFFFull)
+        return fail(OILHIP_E_ARG, "rows/cols exceed 32 bits");
+    return OILHIP_OK;
+}
+
+}  // namespace oilhip
+
+using namespace oilhip;
+
+extern "C" {
+
+const char* oilhip_last_error(void) { return g_err.c_str(); }
+
+int oilhip_probe(int* gfx, uint64_t* hbm_bytes, int* compute_units, char* name, size_t name_cap) {
+    int n = 0;
+    if (hipGetDeviceCount(&n) != hipSuccess || n < 1) return fail(OILHIP_E_NOGPU, "no HIP device visible");
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    hipDeviceProp_t p;
+    OILHIP_HIP(hipGetDeviceProperties(&p, dev));
+    int arch = 0;
+    if (const char* g = std::strstr(p.gcnArchName, "gfx")) arch = (int)std::strtol(g + 3, nullptr, 10);
+    if (gfx) *gfx = arch;
+    if (hbm_bytes) *hbm_bytes = (uint64_t)p.totalGlobalMem;
+    if (compute_units) *compute_units = p.multiProcessorCount;
+    if (name && name_cap) {
+        std::strncpy(name, p.name, name_cap - 1);
+        name[name_cap - 1] = 0;
+    }
+    if (arch != 950) return fail(OILHIP_E_NOGPU, std::string("device is ") + p.gcnArchName + ", this library is built for gfx950 only");
+    return OILHIP_OK;
+}
+
+static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vector<uint64_t>& out_off,
+                  uint64_t algo_bytes, uint64_t rows, uint64_t cols, oilhip_weights** out) {
+    const uint32_t nblocks = (uint32_t)db.size();
+    bool all_full = true, uniform = true, regular = nblocks > 0;
+    uint64_t total_nw = 0;
+    for (uint32_t b = 0; b < nblocks; ++b) {
+        total_nw += db[b].nw;
+        all_full &= db[b].nw == 256;
+        uniform &= db[b].fmt == db[0].fmt;
+        if (b > 0) regular &= (db[b].off16 - db[b - 1].off16) == (db[1].off16 - db[0].off16) &&
+                              db[b].idx_bytes == db[0].idx_bytes && db[b].cb_bytes == db[0].cb_bytes;
+    }
+    if (total_nw != rows * cols) return fail(OILHIP_E_ARG, "rows*cols does not equal the number of weights in the blocks");
+    auto* w = new (std::nothrow) oilhip_weights();
+    if (!w) return fail(OILHIP_E_NOMEM, "host allocation failed");
+    auto bail = [&](hipError_t e, const char* what) {
+        oilhip_weights_destroy(w);
+        return fail(e == hipErrorOutOfMemory ? OILHIP_E_NOMEM : OILHIP_E_DEVICE, std::string(what) + ": " + hipGetErrorString(e));
+    };
+    hipError_t e;
+    if ((e = hipGetDevice(&w->device)) != hipSuccess) return bail(e, "hipGetDevice");
+    // 64 spare bytes so vector loads that straddle the end of the last block stay in bounds
+    w->alloc_bytes = pay.size() + 64;
+    if ((e = hipMalloc(&w->d_payload, w->alloc_bytes)) != hipSuccess) return bail(e, "hipMalloc(payload)");
+    if ((e = hipMemset(w->d_payload, 0, w->alloc_bytes)) != hipSuccess) return bail(e, "hipMemset");
+    if (!pay.empty() && (e = hipMemcpy(w->d_payload, pay.data(), pay.size(), hipMemcpyHostToDevice)) != hipSuccess)
+        return bail(e, "hipMemcpy(payload)");
+    if (nblocks) {
+        if ((e = hipMalloc(&w->d_blocks, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(blocks)");
+        if ((e = hipMemcpy(w->d_blocks, db.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
+            return bail(e, "hipMemcpy(blocks)");
+        if (!all_full) {
+            if ((e = hipMalloc(&w->d_out_off, 8 * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(out_off)");
+            if ((e = hipMemcpy(w->d_out_off, out_off.data(), 8 * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
+                return bail(e, "hipMemcpy(out_off)");
+        }
+    }
+    w->payload_bytes = algo_bytes;
+    w->rows = rows;
+    w->cols = cols;
+    w->nblocks = nblocks;
+    w->uniform_fmt = (uniform && nblocks) ? db[0].fmt : -1;
+    w->all_full = all_full && nblocks > 0;
+    if (regular && uniform && nblocks)
+        w->uniform_stride = nblocks > 1 ? (db[1].off16 - db[0].off16) * 16u
+                                        : (uint32_t)((db[0].cb_bytes + db[0].idx_bytes + 15u) & ~15u);
+    *out = w;
+    return OILHIP_OK;
+}
+
+int oilhip_weights_create(const uint8_t* payload, uint64_t payload_bytes, const oilhip_block_t* blocks,
+                          uint32_t nblocks, uint64_t rows, uint64_t cols, oilhip_weights** out) {
+    if (!out) return fail(OILHIP_E_ARG, "out is null");
+    *out = nullptr;
+    if ((!payload && payload_bytes) || (!blocks && nblocks)) return fail(OILHIP_E_ARG, "null payload/blocks");
+    std::vector<uint8_t> pay;
+    std::vector<DevBlock> db(nblocks);
+    std::vector<uint64_t> off(nblocks);
+    pay.reserve(payload_bytes + 16ull * nblocks);
+    uint64_t nw_sum = 0, algo = 0;
+    for (uint32_t b = 0; b < nblocks; ++b) {
+        const oilhip_block_t& s = blocks[b];
+        if (s.fmt >= OILHIP_NUM_FORMATS) return fail(OILHIP_E_ARG, "block " + std::to_string(b) + ": unknown format id");
+        if (s.cb_off + s.cb_bytes > payload_bytes || s.idx_off + s.idx_bytes > payload_bytes)
+            return fail(OILHIP_E_ARG, "block " + std::to_string(b) + ": payload range out of bounds");
+        if (s.cb_bytes > 0xFFFFu) return fail(OILHIP_E_ARG, "block " + std::to_string(b) + ": codebook channel too large");
+        if (s.nw == 0 || s.nw > (1u << 24)) return fail(OILHIP_E_ARG, "block " + std::to_string(b) + ": bad weight count");
+        pay.resize((pay.size() + 15) & ~(size_t)15, 0);
+        if ((pay.size() >> 4) > 0xFFFFFFFFull) return fail(OILHIP_E_ARG, "payload exceeds 64 GiB");
+        db[b].off16 = (uint32_t)(pay.size() >> 4);
+        db[b].idx_bytes = s.idx_bytes;
+        db[b].nw = s.nw;
+        db[b].cb_bytes = (uint16_t)s.cb_bytes;
+        db[b].fmt = s.fmt;
+        db[b].pad = 0;
+        pay.insert(pay.end(), payload + s.cb_off, payload + s.cb_off + s.cb_bytes);
+        pay.insert(pay.end(), payload + s.idx_off, payload + s.idx_off + s.idx_bytes);
+        off[b] = nw_sum;
+        nw_sum += s.nw;
+        algo += (uint64_t)s.cb_bytes + s.idx_bytes;
+    }
+    return upload(pay, db, off, algo, rows, cols, out);
+}
+
+int oilhip_weights_create_from_records(const uint8_t* rec, uint64_t bytes, const uint8_t* fmts,
+                                       uint32_t nblocks, uint64_t rows, uint64_t cols, oilhip_weights** out) {
+    if (!out) return fail(OILHIP_E_ARG, "out is null");
+    *out = nullptr;
+    if (!rec || !fmts) return fail(OILHIP_E_ARG, "null records/fmts");
+    std::vector<oilhip_block_t> blocks(nblocks);
+    uint64_t at = 0;
+    auto rd32 = [&](uint64_t o) { uint32_t v; std::memcpy(&v, rec + o, 4); return v; };
+    for (uint32_t b = 0; b < nblocks; ++b) {
+        if (at + 8 > bytes) return fail(OILHIP_E_ARG, "record " + std::to_string(b) + " truncated");
+        const uint32_t nw = rd32(at), cbb = rd32(at + 4);
+        if (at + 8 + cbb + 4 > bytes) return fail(OILHIP_E_ARG, "record " + std::to_string(b) + " truncated");
+        const uint32_t ib = rd32(at + 8 + cbb);
+        if (at + 12 + cbb + (uint64_t)ib > bytes) return fail(OILHIP_E_ARG, "record " + std::to_string(b) + " truncated");
+        blocks[b] = oilhip_block_t{at + 8, at + 12 + cbb, cbb, ib, nw, fmts[b] <= 14 ? fmts[b] : (uint8_t)OILHIP_OIL32, {0, 0, 0}};
+        at += 12ull + cbb + ib;
+    }
+    return oilhip_weights_create(rec, bytes, blocks.data(), nblocks, rows, cols, out);
+}
+
+int oilhip_weights_destroy(oilhip_weights* w) {
+    if (!w) return OILHIP_OK;
+    if (w->d_payload) (void)hipFree(w->d_payload);
+    if (w->d_blocks) (void)hipFree(w->d_blocks);
+    if (w->d_out_off) (void)hipFree(w->d_out_off);
+    delete w;
+    return OILHIP_OK;
+}
+
+int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols, uint32_t* nblocks,
+                        uint64_t* payload_bytes, int* uniform_fmt) {
+    if (!w) return fail(OILHIP_E_ARG, "null weights");
+    if (rows) *rows = w->rows;
+    if (cols) *cols = w->cols;
+    if (nblocks) *nblocks = w->nblocks;
+    if (payload_bytes) *payload_bytes = w->payload_bytes;
+    if (uniform_fmt) *uniform_fmt = w->uniform_fmt;
+    return OILHIP_OK;
+}
+
+int oilhip_dequant_f32(const oilhip_weights* w, float* d_out, void* stream) {
+    if (!w || !d_out) return fail(OILHIP_E_ARG, "null argument");
+    return launch_dequant(*w, d_out, (hipStream_t)stream);
+}
+
+int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
+    if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
+    if (w->uniform_fmt == OILHIP_OIL4 && w->uniform_stride == 128) {
+        const int rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
+    return launch_gemv_generic(*w, d_x, d_y, M, (hipStream_t)stream);
+}
+
+// Test hook: the all-format kernel regardless of shape (the specialised kernels
+// are checked against it as well as against the CPU oracle).
+int oilhip_gemv_f32_general(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
+    if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
+    return launch_gemv_generic(*w, d_x, d_y, M, (hipStream_t)stream);
+}
+
+int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x, float* d_y, int M, void* stream) {
+    if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
+    if (w->uniform_fmt != OILHIP_OIL4 || w->uniform_stride != 128)
+        return fail(OILHIP_E_ARG, "bf16 prefill GEMM is implemented for uniform OIL4 tensors");
+    return launch_gemm_oil4_bf16(*w, d_x, d_y, M, (hipStream_t)stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,52 @@
+// common.h -- shared host-side declarations of liboilhip (not part of the C ABI).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
+
+#include "../../include/oilhip.h"
+#include "block_decode.h"
+
+namespace oilhip {
+
+// Thread-local text behind oilhip_last_error().
+void set_error(const std::string& msg);
+int fail(int code, const std::string& msg);
+
+#define OILHIP_HIP(call)                                                                  \
+    do {                                                                                  \
+        hipError_t e_ = (call);                                                           \
+        if (e_ != hipSuccess)                                                             \
+            return ::oilhip::fail(OILHIP_E_DEVICE, std::string(#call) + ": " + hipGetErrorString(e_)); \
+    } while (0)
+
+// Per-device decode tables (device pointer), created on first use.
+int get_tables(const DecodeTables** out);
+int device_cu_count();
+
+}  // namespace oilhip
+
+// The handle behind oilhip_weights*.
+struct oilhip_weights {
+    int device = 0;
+    uint8_t* d_payload = nullptr;           // block payloads, each 16-byte aligned
+    oilhip::DevBlock* d_blocks = nullptr;   // one descriptor per block
+    uint64_t* d_out_off = nullptr;          // first output index per block (only when nw varies)
+    uint64_t alloc_bytes = 0;               // size of d_payload
+    uint64_t payload_bytes = 0;             // sum of cb_bytes + idx_bytes
+    uint64_t rows = 0, cols = 0;
+    uint32_t nblocks = 0;
+    int uniform_fmt = -1;                   // single format id, or -1
+    uint32_t uniform_stride = 0;            // bytes between consecutive blocks when regular, else 0
+    bool all_full = false;                  // every block holds exactly 256 weights
+};
+
+namespace oilhip {
+// kernels (each returns an OILHIP_* code and sets the error text)
+int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
+int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+// fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
+int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
+}  // namespace oilhip

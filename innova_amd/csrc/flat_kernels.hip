@@ -1,0 +1,219 @@
+// flat_kernels.hip -- the reference's flat-codebook matmul entry points on the
+// device: one caller-supplied codebook, plain row-major index matrices.
+//   oil::kernel::oil8_gemm / oil4_gemm          src/kernel_oil8.cpp, src/kernel_oil4.cpp
+//   oil::adapters::prod::gemv_{spark,oil4,oil8} src/kernel_production.cpp:79-128,345-364
+//   oil::engines::OIL{8,4,2}Engine::quant_gemm  src/oil_engines_oil{8,4,2}.cpp
+// One workgroup of 256 threads per output row; the codebook sits in LDS; thread t
+// walks k = t, t+256, ... so index bytes are read coalesced.
+#include "common.h"
+
+namespace oilhip {
+namespace {
+
+constexpr int MBF = 4;   // activation rows per pass
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// Sum acc[0..MBF) over the 256 threads; thread b < MBF returns the total of acc[b].
+__device__ __forceinline__ float block_sums(const float (&acc)[MBF], float (*part)[4]) {
+    const uint32_t t = threadIdx.x;
+#pragma unroll
+    for (int b = 0; b < MBF; ++b) {
+        const float s = wave_sum(acc[b]);
+        if ((t & 63) == 0) part[b][t >> 6] = s;
+    }
+    __syncthreads();
+    float r = 0.0f;
+    if (t < MBF) r = (part[t][0] + part[t][1]) + (part[t][2] + part[t][3]);
+    __syncthreads();
+    return r;
+}
+
+// FP16 codebook entry exactly as fp16_to_float (src/kernel_oil4.cpp:15-29).
+__device__ __forceinline__ float flat_half(uint16_t h) {
+    const uint32_t e = (h >> 10) & 31u, m = h & 0x3FFu;
+    if (e == 31u && m != 0u) return __uint_as_float(0x7FC00000u);
+    return half_bits_to_float(h);
+}
+
+// mode 0: oil8_gemm  -- weights row n (K bytes),        activations row m, out[m*N+n]
+// mode 1: prod oil8  -- weights row n (K bytes),        activations row m, out[m*N+n] * scale
+__global__ void __launch_bounds__(256)
+flat8_kernel(const uint8_t* __restrict__ idx, const float* __restrict__ cb, const float* __restrict__ act,
+             float* __restrict__ out, int M, int N, int K, float scale) {
+    __shared__ float c[256];
+    __shared__ float part[MBF][4];
+    const uint32_t t = threadIdx.x, n = blockIdx.x;
+    c[t] = cb[t];
+    __syncthreads();
+    const uint8_t* w = idx + (size_t)n * K;
+    for (int m0 = 0; m0 < M; m0 += MBF) {
+        float acc[MBF] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int k = t; k < K; k += 256) {
+            const float v = c[w[k]];
+#pragma unroll
+            for (int b = 0; b < MBF; ++b)
+                if (m0 + b < M) acc[b] = __fmaf_rn(v, act[(size_t)(m0 + b) * K + k], acc[b]);
+        }
+        const float r = block_sums(acc, part);
+        if (t < MBF && m0 + (int)t < M) out[(size_t)(m0 + t) * N + n] = r * scale;
+    }
+}
+
+// oil4_gemm: one workgroup per (m, n) pair; the pair's K nibbles start at nibble
+// (m*N+n)*K rounded down to a byte, activations are row n (src/kernel_oil4.cpp:38-56).
+__global__ void __launch_bounds__(256)
+flat4_pair_kernel(const uint8_t* __restrict__ packed, const uint16_t* __restrict__ cb16,
+                  const float* __restrict__ act, float* __restrict__ out, int N, int K) {
+    __shared__ float c[16];
+    __shared__ float part[MBF][4];
+    const uint32_t t = threadIdx.x;
+    const uint64_t pair = blockIdx.x;
+    if (t < 16) c[t] = flat_half(cb16[t]);
+    __syncthreads();
+    const uint8_t* w = packed + (pair * (uint64_t)K) / 2;
+    const float* a = act + (pair % (uint64_t)N) * (uint64_t)K;
+    float acc[MBF] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int k = t; k < K; k += 256) {
+        const uint32_t byte = w[k >> 1];
+        acc[0] = __fmaf_rn(c[(k & 1) ? (byte >> 4) : (byte & 15u)], a[k], acc[0]);
+    }
+    const float r = block_sums(acc, part);
+    if (t == 0) out[pair] = r;
+}
+
+// prod gemv over packed rows: BITS = 4 (two codes per byte, FP16 codebook) or
+// BITS = 2 (SPARK ternary: 0 -> -1, 1 -> 0, 2 and 3 -> +1).  Row m of W against
+// activation row b; Y[b*M + m] = scale * dot.
+template <int BITS>
+__global__ void __launch_bounds__(256)
+prod_packed_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ cb16, float scale,
+                   const float* __restrict__ x, float* __restrict__ y, int M, int K, int batch) {
+    __shared__ float c[16];
+    __shared__ float part[MBF][4];
+    const uint32_t t = threadIdx.x, m = blockIdx.x;
+    if (BITS == 4 && t < 16) c[t] = flat_half(cb16[t]);
+    __syncthreads();
+    constexpr int PER = 8 / BITS;
+    const uint8_t* row = wq + (size_t)m * ((K + PER - 1) / PER);
+    for (int b0 = 0; b0 < batch; b0 += MBF) {
+        float acc[MBF] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int k = t; k < K; k += 256) {
+            const uint32_t code = (row[k / PER] >> ((k % PER) * BITS)) & ((1u << BITS) - 1u);
+            const float v = BITS == 4 ? c[code] : (code == 0 ? -1.0f : (code == 1 ? 0.0f : 1.0f));
+#pragma unroll
+            for (int b = 0; b < MBF; ++b)
+                if (b0 + b < batch) acc[b] = __fmaf_rn(v, x[(size_t)(b0 + b) * K + k], acc[b]);
+        }
+        const float r = block_sums(acc, part);
+        if (t < MBF && b0 + (int)t < batch) y[(size_t)(b0 + t) * M + m] = r * scale;
+    }
+}
+
+// Engine layout: codes packed along the flat [K][N] index; thread per output column
+// n, sequential in k like the reference loop (terms with A == 0 are skipped).
+template <int BITS>
+__global__ void __launch_bounds__(256)
+engine_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const float* __restrict__ cb,
+              float* __restrict__ C, long long M, long long N, long long K) {
+    __shared__ float c[1 << BITS];
+    for (int i = threadIdx.x; i < (1 << BITS); i += 256) c[i] = cb[i];
+    __syncthreads();
+    const long long n = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long m = blockIdx.y;
+    if (n >= N) return;
+    constexpr int PER = 8 / BITS;
+    float acc = 0.0f;
+    for (long long k = 0; k < K; ++k) {
+        const float a = A[m * K + k];
+        if (a == 0.0f) continue;
+        const long long flat = k * N + n;
+        const uint32_t code = (bq[flat / PER] >> ((flat % PER) * BITS)) & ((1u << BITS) - 1u);
+        acc = __fmaf_rn(a, c[code], acc);
+    }
+    C[m * N + n] = acc;
+}
+
+int check(const void* a, const void* b, const void* c, const void* d, long long M, long long N, long long K) {
+    if (!a || !b || !c || !d) return fail(OILHIP_E_ARG, "null argument");
+    if (M < 0 || N < 0 || K < 0) return fail(OILHIP_E_ARG, "negative dimension");
+    return OILHIP_OK;
+}
+
+}  // namespace
+}  // namespace oilhip
+
+using namespace oilhip;
+
+extern "C" {
+
+int oilhip_flat_oil8_gemm(const uint8_t* d_idx, const float* d_cb, const float* d_act, float* d_out,
+                          int M, int N, int K, void* stream) {
+    if (int rc = check(d_idx, d_cb, d_act, d_out, M, N, K)) return rc;
+    if (M == 0 || N == 0) return OILHIP_OK;
+    hipLaunchKernelGGL(flat8_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, d_idx, d_cb, d_act, d_out, M, N, K, 1.0f);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_flat_oil4_gemm(const uint8_t* d_packed, const uint16_t* d_cb16, const float* d_act, float* d_out,
+                          int M, int N, int K, void* stream) {
+    if (int rc = check(d_packed, d_cb16, d_act, d_out, M, N, K)) return rc;
+    if (M == 0 || N == 0) return OILHIP_OK;
+    if ((long long)M * N > 0x7FFFFFFFll) return fail(OILHIP_E_ARG, "M*N exceeds the grid limit");
+    hipLaunchKernelGGL(flat4_pair_kernel, dim3((uint32_t)((long long)M * N)), dim3(256), 0, (hipStream_t)stream,
+                       d_packed, d_cb16, d_act, d_out, N, K);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_prod_gemv_spark(const uint8_t* d_w, float scale, const float* d_x, float* d_y,
+                           int M, int K, int batch, void* stream) {
+    if (int rc = check(d_w, d_x, d_y, d_y, M, batch, K)) return rc;
+    if (M == 0 || batch == 0) return OILHIP_OK;
+    hipLaunchKernelGGL(prod_packed_kernel<2>, dim3(M), dim3(256), 0, (hipStream_t)stream, d_w,
+                       (const uint16_t*)nullptr, scale, d_x, d_y, M, K, batch);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_prod_gemv_oil4(const uint8_t* d_w, const uint16_t* d_cb16, float scale, const float* d_x,
+                          float* d_y, int M, int K, int batch, void* stream) {
+    if (int rc = check(d_w, d_cb16, d_x, d_y, M, batch, K)) return rc;
+    if (M == 0 || batch == 0) return OILHIP_OK;
+    hipLaunchKernelGGL(prod_packed_kernel<4>, dim3(M), dim3(256), 0, (hipStream_t)stream, d_w, d_cb16, scale,
+                       d_x, d_y, M, K, batch);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+// Y[b*M + m]: the flat OIL8 kernel with (rows = M weight rows, batch = activation rows).
+int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb, float scale, const float* d_x, float* d_y,
+                          int M, int K, int batch, void* stream) {
+    if (int rc = check(d_w, d_cb, d_x, d_y, M, batch, K)) return rc;
+    if (M == 0 || batch == 0) return OILHIP_OK;
+    hipLaunchKernelGGL(flat8_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, d_w, d_cb, d_x, d_y, batch, M, K, scale);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b, const float* d_cb, float* d_c,
+                             int64_t M, int64_t N, int64_t K, void* stream) {
+    if (int rc = check(d_a, d_b, d_cb, d_c, M, N, K)) return rc;
+    if (bits != 2 && bits != 4 && bits != 8) return fail(OILHIP_E_ARG, "bits must be 2, 4 or 8");
+    if (M == 0 || N == 0) return OILHIP_OK;
+    if (M > 65535) return fail(OILHIP_E_ARG, "M exceeds the grid limit");
+    const dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)M);
+    hipStream_t s = (hipStream_t)stream;
+    if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    else if (bits == 4) hipLaunchKernelGGL(engine_kernel<4>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    else hipLaunchKernelGGL(engine_kernel<2>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+"""Host mirror of the reference's flat-codebook kernel entry points
+(include/oil/kernel.h:24-32, include/oil/kernel_production.h:25-52,
+include/oil/oil_engines.h quant_gemm).  Arguments may be numpy arrays (uploaded
+per call, as the reference's host-pointer signatures imply) or cuda tensors
+(used in place); results come back in the same kind."""
+from __future__ import annotations
+
+import numpy as np
+
+from . import _lib
+
+
+def _dev(a, np_dtype):
+    import torch
+    if isinstance(a, torch.Tensor):
+        assert a.is_cuda and a.is_contiguous()
+        return a, True
+    t = torch.from_numpy(np.ascontiguousarray(a, dtype=np_dtype).reshape(-1).view(
+        np.int16 if np_dtype == np.uint16 else np_dtype)).cuda()
+    return t, False
+
+
+def _ret(out, on_device):
+    return out if on_device else out.cpu().numpy()
+
+
+def oil8_gemm(indices, codebook, activations, M: int, N: int, K: int):
+    """out[m*N+n] = sum_k codebook[indices[n*K+k]] * activations[m*K+k]  (kernel.h:24-26)."""
+    import torch
+    i, d1 = _dev(indices, np.uint8)
+    c, _ = _dev(codebook, np.float32)
+    a, d2 = _dev(activations, np.float32)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_flat_oil8_gemm(i.data_ptr(), c.data_ptr(), a.data_ptr(), out.data_ptr(),
+                                                M, N, K, _lib.current_stream()))
+    return _ret(out, d1 and d2)
+
+
+def oil4_gemm(packed_indices, codebook, activations, M: int, N: int, K: int):
+    """out[m*N+n] = sum_k f16(codebook[nib((m*N+n)*K+k)]) * activations[n*K+k]  (kernel.h:30-32)."""
+    import torch
+    i, d1 = _dev(packed_indices, np.uint8)
+    c, _ = _dev(codebook, np.uint16)
+    a, d2 = _dev(activations, np.float32)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_flat_oil4_gemm(i.data_ptr(), c.data_ptr(), a.data_ptr(), out.data_ptr(),
+                                                M, N, K, _lib.current_stream()))
+    return _ret(out, d1 and d2)
+
+
+def _prod(fn, w, cb, cb_dtype, scale, X, M, N, K):
+    import torch
+    wd, d1 = _dev(w, np.uint8)
+    xd, d2 = _dev(X, np.float32)
+    Y = torch.empty((N, M), dtype=torch.float32, device="cuda")
+    if cb is None:
+        _lib.check(fn(wd.data_ptr(), float(scale), xd.data_ptr(), Y.data_ptr(), M, K, N, _lib.current_stream()))
+    else:
+        cd, _ = _dev(cb, cb_dtype)
+        _lib.check(fn(wd.data_ptr(), cd.data_ptr(), float(scale), xd.data_ptr(), Y.data_ptr(), M, K, N,
+                      _lib.current_stream()))
+    return _ret(Y, d1 and d2)
+
+
+def gemv_spark_batch(packed_w, scale, X, M: int, N: int, K: int):
+    """Y[n*M+m] = scale * sum_k tern(W[m][k]) * X[n*K+k]  (kernel_production.h:40-42)."""
+    return _prod(_lib.lib().oilhip_prod_gemv_spark, packed_w, None, None, scale, X, M, N, K)
+
+
+def gemv_oil4_batch(packed_indices, codebook, scale, X, M: int, N: int, K: int):
+    return _prod(_lib.lib().oilhip_prod_gemv_oil4, packed_indices, codebook, np.uint16, scale, X, M, N, K)
+
+
+def gemv_oil8_batch(indices, codebook, scale, X, M: int, N: int, K: int):
+    return _prod(_lib.lib().oilhip_prod_gemv_oil8, indices, codebook, np.float32, scale, X, M, N, K)
+
+
+def gemv_spark_tiled(packed_w, scale, x, M: int, K: int, tile_m: int = 32):
+    """y = scale * (W @ x)  (kernel_production.h:25-27); tile_m is a CPU cache hint, unused here."""
+    return gemv_spark_batch(packed_w, scale, x, M, 1, K).reshape(-1)
+
+
+def gemv_oil4_tiled(packed_indices, codebook, scale, x, M: int, K: int, tile_m: int = 32):
+    return gemv_oil4_batch(packed_indices, codebook, scale, x, M, 1, K).reshape(-1)
+
+
+def gemv_oil8_tiled(indices, codebook, scale, x, M: int, K: int, tile_m: int = 32):
+    return gemv_oil8_batch(indices, codebook, scale, x, M, 1, K).reshape(-1)
+
+
+def engine_quant_gemm(bits: int, a, b_idx, codebook, M: int, N: int, K: int):
+    """C[m*N+n] = sum_k A[m*K+k] * codebook[code(k*N+n)]: OIL{8,4,2}Engine::quant_gemm
+    (include/oil/oil_engines.h:49,78,151)."""
+    import torch
+    ad, d1 = _dev(a, np.float32)
+    bd, d2 = _dev(b_idx, np.uint8)
+    cd, _ = _dev(codebook, np.float32)
+    if cd.numel() < (1 << bits):
+        raise _lib.OilHipError("engine_quant_gemm: codebook has fewer than 2^bits entries")
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_engine_quant_gemm(bits, ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), out.data_ptr(),
+                                                   M, N, K, _lib.current_stream()))
+    return _ret(out, d1 and d2)

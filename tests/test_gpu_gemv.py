@@ -1,0 +1,132 @@
+"""Decode GEMV through the C ABI (oilhip_gemv_f32) against the CPU oracle.
+
+Tolerance (north star): relative L2 error <= 1e-5 against the double-precision
+dot of the bit-exact decoded weights.  The reference's own FP32 summation order
+is measured against the same yardstick for comparison."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import innova_amd as ia
+import oracle as O
+from gpu_util import gaussian_weights, rel_l2, to_orc_blocks
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+GV = np.load(os.path.join(os.path.dirname(__file__), "golden", "block_gemv.npz"))
+
+
+def run_case(fmts, rows, cols, M, seed, general=False, outlier_every=13):
+    w = gaussian_weights(rows * cols, seed, outlier_every=outlier_every)
+    payload, blocks = ia.block_codec.quantize_tensor(w, fmts)
+    X = np.random.default_rng(seed + 1).standard_normal((M, cols)).astype(np.float32)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        got = dw.gemv(torch.from_numpy(X).cuda(), general=general).cpu().numpy()
+    want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+    assert got.shape == (M, rows)
+    return rel_l2(got, want), payload, blocks, X, want
+
+
+@pytest.mark.parametrize("name", list(O.FORMATS))
+def test_golden_gemv_every_format(name):
+    """Reference payloads + double-precision outputs of the reference-decoded weights."""
+    rows, cols, B = (int(v) for v in GV["shape"])
+    il, cl = GV[f"{name}/idx_len"], GV[f"{name}/cb_len"]
+    payload = np.concatenate([GV[f"{name}/idx"], GV[f"{name}/cb"], np.zeros(16, np.uint8)])
+    blocks = np.zeros(il.size, dtype=ia._lib.BLOCK_DTYPE)
+    blocks["idx_off"] = np.concatenate([[0], np.cumsum(il)[:-1]])
+    blocks["idx_bytes"] = il
+    blocks["cb_off"] = GV[f"{name}/idx"].size + np.concatenate([[0], np.cumsum(cl)[:-1]])
+    blocks["cb_bytes"] = cl
+    blocks["nw"], blocks["fmt"] = 256, O.FORMATS[name]
+    X = GV["x_bits"].view(np.float32).reshape(B, cols)
+    want = GV[f"{name}/y_bits"].view(np.float32).reshape(B, rows)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        got = dw.gemv(torch.from_numpy(X.copy()).cuda()).cpu().numpy()
+        gen = dw.gemv(torch.from_numpy(X.copy()).cuda(), general=True).cpu().numpy()
+    assert rel_l2(got, want) <= TOL, name
+    assert rel_l2(gen, want) <= TOL, name
+
+
+@pytest.mark.parametrize("fmt", list(ia.Format))
+@pytest.mark.parametrize("M", [1, 3])
+def test_uniform_format_gemv(fmt, M):
+    err, *_ = run_case(fmt, rows=70, cols=1280, M=M, seed=20 + int(fmt))
+    assert err <= TOL
+
+
+def test_mixed_format_rows():
+    rng = np.random.default_rng(3)
+    rows, cols = 48, 2048
+    fmts = rng.integers(0, 15, rows * cols // 256).astype(np.uint8)
+    err, *_ = run_case(fmts, rows, cols, M=2, seed=31)
+    assert err <= TOL
+
+
+# the fast OIL4 kernel: every slab width (cols/256 = 16 -> 8 blocks per slab, 43 -> 4,
+# 6 -> 2, 3 -> 1, 56 -> 8), ragged row counts, chunked rows, M up to 16
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (1000, 4096), (37, 11008), (300, 11008),
+                                        (129, 1536), (50, 768), (77, 14336), (1, 256), (5, 512),
+                                        (3000, 2048)])
+@pytest.mark.parametrize("M", [1, 2, 4, 16])
+def test_oil4_fast_kernel_shapes(rows, cols, M):
+    if M > 2 and rows * cols > 2_000_000:
+        pytest.skip("large-M cases are covered at the smaller shapes")
+    err, payload, blocks, X, want = run_case(ia.Format.OIL4, rows, cols, M, seed=rows + cols + M)
+    assert err <= TOL
+    ref32 = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=False)
+    # the reference's own FP32 order sits at a comparable distance from the yardstick
+    assert rel_l2(ref32, want) <= TOL
+
+
+def test_oil4_special_blocks():
+    """Zero blocks (-0.0 levels), underflowing scales, huge outliers, zero activations."""
+    rows, cols = 96, 4096
+    w = gaussian_weights(rows * cols, 77)
+    w[0:256] = 0.0
+    w[256 * 20: 256 * 21] *= np.float32(1e-7)
+    w[256 * 40: 256 * 41] *= np.float32(1e4)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    X = np.random.default_rng(78).standard_normal((1, cols)).astype(np.float32)
+    X[0, ::5] = 0.0
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        got = dw.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
+        gen = dw.gemv(torch.from_numpy(X).cuda(), general=True).cpu().numpy()
+    want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+    assert rel_l2(got, want) <= TOL and rel_l2(gen, want) <= TOL
+
+
+@pytest.mark.parametrize("rows,cols", [(11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("M", [1, 4, 16])
+def test_oil4_llama_mlp_shapes_full_size(rows, cols, M):
+    """Config sizes.  The oracle runs on a row sample; all rows are covered by
+    linearity: y(x1 + x2) = y(x1) + y(x2) and y(2x) = 2 y(x) within tolerance."""
+    w = gaussian_weights(rows * cols, seed=rows)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    assert payload.size == 22544384
+    rng = np.random.default_rng(cols + M)
+    X = rng.standard_normal((M, cols)).astype(np.float32)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        xd = torch.from_numpy(X).cuda()
+        y = dw.gemv(xd).cpu().numpy()
+        y2 = dw.gemv(xd * 2.0).cpu().numpy()
+        perm = torch.from_numpy(rng.permutation(M)).cuda()
+        ysum = dw.gemv(xd + xd[perm]).cpu().numpy()
+    assert rel_l2(y2, 2.0 * y) <= 1e-6
+    assert rel_l2(ysum, y + y[perm.cpu().numpy()]) <= TOL
+    # oracle on every 64th row and the last rows
+    sel = np.unique(np.concatenate([np.arange(0, rows, 64), np.arange(rows - 8, rows)]))
+    bpr = cols // 256
+    ob = to_orc_blocks(blocks).reshape(rows, bpr)[sel].reshape(-1)
+    want = O.block_gemm(payload, ob, sel.size, cols, X, wide=True)
+    assert rel_l2(y[:, sel], want) <= TOL
+
+
+def test_shape_errors():
+    w = gaussian_weights(256 * 3 + 10, 1)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    with ia.DeviceWeights.from_blocks(payload, blocks, 1, w.size) as dw:
+        with pytest.raises(ia.OilHipError):
+            dw.gemv(torch.zeros(1, w.size, device="cuda"))        # ragged block: matmul refuses
