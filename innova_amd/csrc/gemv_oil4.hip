@@ -8,21 +8,28 @@
 // zero, own no bits).  In nibble units: nibbles 0..3 hold the scale, nibble
 // p >= 4 holds weight i(p) = (p-4) + (p-4)/63.
 //
-// Mapping.  Work is cut into "slabs" of SB consecutive blocks of a row.  A
-// wavefront owns one slab position and walks down rows: 8 lanes cover one
-// 128-byte block with one 16-byte load each (32 nibbles per lane), so a wave
-// load covers RW = 8/SB rows x SB blocks.  Because a lane sees the same 32
-// nibble positions in every row, its 32 activations live in registers for the
-// whole kernel, pre-permuted into nibble order (scale nibbles and out-of-range
-// blocks get activation 0).  Per packed byte the two level values come from one
-// LDS read of a 256-entry pair table (address built with a single v_perm_b32),
-// followed by two FP32 FMAs.  The per-block FP16 scale is applied once per
-// block after an 8-lane DPP reduction; slab partials meet in LDS.
+// Mapping.  8 lanes cover one 128-byte block with one 16-byte load each (32
+// nibbles per lane), so one wave-load covers 8 consecutive blocks of a row (a
+// "column set", 1 KB).  A wavefront owns CS consecutive column sets (a slab of
+// the row) and walks down rows.  A lane sees the same 32*CS nibble positions in
+// every row, so its activations live in registers for the whole kernel,
+// gathered once from an LDS copy of x (scale nibbles and blocks past the end of
+// the row get activation 0).  Per packed byte the two level values come from
+// one LDS read of a 256-entry pair table whose address is built by a single
+// v_perm_b32, followed by two FP32 FMAs.  The block's FP16 scale is applied to
+// the lane's 32-nibble partial sum; one 6-step DPP reduction per row and slab
+// finishes the dot product.  The kernel is issue-bound on the vector ALU, so
+// everything outside the per-byte perm + 2 FMAs is kept to a handful of
+// instructions per row.
 #include <hip/hip_fp16.h>
 
 #include <cstdlib>
 
 #include "common.h"
+
+#ifndef OILHIP_OIL4_PREFETCH
+#define OILHIP_OIL4_PREFETCH 6
+#endif
 
 namespace oilhip {
 namespace {
@@ -42,27 +49,54 @@ __device__ __forceinline__ float dpp_half_mirror(float v) {
 __device__ __forceinline__ float dpp_row_ror8(float v) {
     return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));  // row_ror:8
 }
-__device__ __forceinline__ float lane_value(float v, int lane) {
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+__device__ __forceinline__ float dpp_row_mirror(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
+}
+// lane 15 of rows 0 and 2 into every lane of rows 1 and 3 (other rows receive 0)
+__device__ __forceinline__ float dpp_row_bcast15(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));
+}
+// lane 31 into every lane of rows 2 and 3 (other rows receive 0)
+__device__ __forceinline__ float dpp_row_bcast31(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));
+}
+// value of the first lane of each group of 8 lanes, in all 8 lanes
+__device__ __forceinline__ uint32_t dpp_bcast8(uint32_t v) {
+    const int q = __builtin_amdgcn_update_dpp(0, (int)v, 0x00, 0xF, 0xF, true);      // quad_perm [0,0,0,0]
+    return (uint32_t)__builtin_amdgcn_update_dpp(q, q, 0x114, 0xF, 0xA, false);     // row_shr:4 into quads 1 and 3
 }
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) const float lds_cfloat;
 
 constexpr uint32_t kOobOffset = 0xFFFFFF00u;   // beyond any buffer range: the load returns zeros, no fetch
 
 // The two level values of one packed byte: (low nibble, high nibble).
 struct LevelPair { float lo, hi; };
 
-template <int J>
-__device__ __forceinline__ LevelPair lookup(uint32_t word, uint32_t lanebase) {
-    // byte J of the dword -> address bits 8..15, this lane's table copy -> bits 0..7
-    const uint32_t addr = __builtin_amdgcn_perm(word, lanebase, 0x0C0C0000u | ((4u + J) << 8));
-    lds_cfloat* tp = (lds_cfloat*)(uintptr_t)addr;
-    return LevelPair{tp[0], tp[32]};
+// kOIL4Levels (src/block_codec.cpp:18-23) selected by compares on literals: no memory access.
+__device__ __forceinline__ float level_literal(uint32_t i) {
+    const float mag = (i == 7 || i == 8) ? 0.1260f : (i == 6 || i == 9) ? 0.3976f : (i == 5 || i == 10) ? 0.6508f
+                    : (i == 4 || i == 11) ? 0.9275f : (i == 3 || i == 12) ? 1.2392f : (i == 2 || i == 13) ? 1.5995f
+                    : (i == 1 || i == 14) ? 2.0522f : 2.7178f;
+    return i < 8 ? -mag : mag;
 }
 
-__device__ __forceinline__ void lookup_row(const u32x4& w, uint32_t lanebase, LevelPair (&t)[16]) {
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const f32x2 lds_cfloat2;
+typedef __attribute__((address_space(3))) const float lds_cfloat;
+
+// Pair table, 64 KB at LDS offset 0: entry of byte value v and lane copy c at
+// byte v*256 + c*8 = (level[v & 15], level[v >> 4]).  32 lane-private copies:
+// lanes of a half-wave never meet in a bank at different addresses.
+template <int J>
+__device__ __forceinline__ LevelPair lookup(uint32_t word, uint32_t lanebase) {
+    // byte J of the dword -> address bits 8..15, this lane's copy -> bits 0..7
+    const uint32_t addr = __builtin_amdgcn_perm(word, lanebase, 0x0C0C0000u | ((4u + J) << 8));
+    const f32x2 t = *(lds_cfloat2*)(uintptr_t)addr;
+    return LevelPair{t.x, t.y};
+}
+
+__device__ __forceinline__ void lookup_load(const u32x4& w, uint32_t lanebase, LevelPair (&t)[16]) {
     const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
@@ -73,164 +107,226 @@ __device__ __forceinline__ void lookup_row(const u32x4& w, uint32_t lanebase, Le
     }
 }
 
-// SB: blocks per slab (8, 4, 2 or 1); RPW: wave-loads per chunk (all in flight
-// at once); MB: activation rows handled together; MAXT: workgroup size bound.
-template <int SB, int RPW, int MB, int MAXT>
-__global__ void __launch_bounds__(MAXT)
+constexpr int kPrefetch = OILHIP_OIL4_PREFETCH;   // wave-loads in flight per wavefront
+constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 32 so that neighbouring blocks start 32 banks apart
+
+// CS: column sets (wave-loads) per row and wave; RPW: rows per chunk, all loads of
+// a chunk in flight at once; MB: activation rows handled together; MAXT: workgroup size bound.
+template <int CS, int RPW, int MB, int MAXT>
+__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y,
-                 uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M) {
-    constexpr int LS = 8 * SB;        // lanes across one slab row
-    constexpr int RW = 64 / LS;       // rows per wave-load
-    constexpr int CH = RPW * RW;      // rows per chunk and row group
+                 uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M,
+                 uint32_t rg_base, uint32_t rg_rem) {
+    constexpr int NL = CS * RPW;      // wave-loads per chunk
     extern __shared__ __align__(16) uint8_t lds[];
-    float* tab = reinterpret_cast<float*>(lds);                        // LDS byte offset 0
-    float* xs = reinterpret_cast<float*>(lds + kTabBytes);             // [MB][S*SB*256] nibble-ordered
-    const uint32_t kpad = S * SB * 256;
-    float* red = xs + (size_t)MB * kpad;                               // [G][CH][MB][S]
+    float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
+    const uint32_t nblk = S * CS * 8;                                         // blocks covered by all slabs (>= cols/256)
+    const uint32_t xstride = nblk * kXsBlock;                                 // floats per activation row in LDS
+    float* xs = reinterpret_cast<float*>(lds + kTabBytes);                    // [MB][nblk][8 c][8 lp][4 e] (+32 pad), nibble order
+    float* red = xs + (size_t)MB * xstride;                                   // [G][RPW][MB][S]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t slab = wave % S, grp = wave / S;
     const uint32_t bpr = cols >> 8;
-    const uint32_t sub = lane / LS, l = lane % LS, lp = l & 7u;
-    const uint32_t kb = slab * SB + (l >> 3);
-    const bool col_ok = kb < bpr;
+    const uint32_t lp = lane & 7u;
 
-    const uint32_t J = gridDim.x * G, jg = blockIdx.x * G + grp;
-    const uint32_t r0 = (uint32_t)(((uint64_t)rows * jg) / J);
-    const uint32_t r1 = (uint32_t)(((uint64_t)rows * (jg + 1)) / J);
+    // row group j owns rows [j*rg_base + min(j, rg_rem), ...): rows split evenly over gridDim.x * G groups
+    auto group_begin = [&](uint32_t j) { return j * rg_base + (j < rg_rem ? j : rg_rem); };
+    const uint32_t jg = blockIdx.x * G + grp;
+    const bool working = wave < S * G;                                        // spare wavefronts only help with the prologue
+    const uint32_t r0 = working ? group_begin(jg) : 0u, r1 = working ? group_begin(jg + 1) : 0u;
     const uint32_t row_bytes = bpr * 128u;
     // buffer resource over this workgroup's rows (offsets stay below 2^31)
-    const uint32_t wg_r0 = (uint32_t)(((uint64_t)rows * (blockIdx.x * G)) / J);
+    const uint32_t wg_r0 = group_begin(blockIdx.x * G);
     const uint64_t remain = (uint64_t)(rows - wg_r0) * row_bytes;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(W + (size_t)wg_r0 * row_bytes), 0, (int)(remain < 0x80000000ull ? remain : 0x80000000ull), 0x00020000);
-    const uint32_t lane_off = kb * 128u + lp * 16u;
 
-    // ---- activations first (they are needed soonest), then the first chunk of weights ----
-    // xs[m][b*256 + c*32 + q8*4 + e] = x'(p = 32*q8 + 4c + e): nibble order, 0 under the scale
-    // nibbles and beyond the last block.  XPT elements per thread are fetched up front so the
-    // table build and these loads overlap the weight loads that follow them in the queue.
-    constexpr int XPT = 8;
+    // ---- x first (needed soonest), then every weight load of the first chunk ----------
+    // Nothing that waits on vector memory may follow the weight loads before their use:
+    // loads return in order, so it would wait for every weight byte.
+    constexpr int XPT = 4;            // float4 pieces of x fetched up front per thread
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(x + (size_t)m0 * cols), 0, (int)((uint64_t)(M - m0 < MB ? M - m0 : MB) * cols * 4u), 0x00020000);
-    auto x_offset = [&](uint32_t d) -> uint32_t {          // byte offset of x' element d, or out of range
-        const uint32_t b = d >> 8, rem = d & 255u;
-        const uint32_t c = rem >> 5, q8 = (rem >> 2) & 7u, e = rem & 3u;
-        const uint32_t p = 32 * q8 + 4 * c + e;
-        const uint32_t q = p - 4;
-        const uint32_t i = q + (q >= 63) + (q >= 126) + (q >= 189);
-        return (p >= 4 && b < bpr && d < kpad) ? (b * 256u + i) * 4u : kOobOffset;
-    };
-    float xpre[MB][XPT];
+        (void*)(x + (size_t)m0 * cols), 0, (int)((uint32_t)(M - m0 < MB ? M - m0 : MB) * cols * 4u), 0x00020000);
+    u32x4 xpre[MB][XPT];
 #pragma unroll
     for (int u = 0; u < XPT; ++u) {
-        const uint32_t off = x_offset(tid + u * blockDim.x);
+        const uint32_t d4 = tid + u * 512u;                             // float4 index into the padded row
 #pragma unroll
         for (int m = 0; m < MB; ++m)
-            xpre[m][u] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
-                xrsrc, off == kOobOffset ? off : off + m * cols * 4u, 0, 0));
+            xpre[m][u] = __builtin_amdgcn_raw_buffer_load_b128(
+                xrsrc, (d4 * 4u < cols && m0 + m < M) ? d4 * 16u + m * cols * 4u : kOobOffset, 0, 0);
     }
-    u32x4 wv[RPW];
+    const uint32_t lane_off = (slab * CS * 8u + (lane >> 3)) * 128u + lp * 16u;   // first column set of this lane
+    // The 64 KB pair table is written while the weight loads queue up: float4 number e of the
+    // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + 512*k,
+    // k = 0..7, so its low nibble (tid >> 4) & 15 is fixed and its high nibble is (tid >> 8) + 2k,
+    // uniform across the wavefront.  Levels come from literals: no memory access, no barrier.
+    const float lv_lane = level_literal(lane & 15u);                          // lane i holds level[i & 15]
+    const float lo_fix = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+    auto table_chunk = [&](int k) {
+        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
+        reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
+    };
+    // Wave-load n of a chunk: row cbase + n / CS, column set n % CS.  Only PF loads are queued up
+    // front (the memory pipeline of a CU holds a limited number of outstanding lines; queueing
+    // more only stalls the wavefront in front of its prologue); the rest follow once the
+    // prologue is done, while the first PF are being consumed.
+    constexpr int PF = NL < kPrefetch ? NL : kPrefetch;
+    u32x4 wv[NL];
+    auto issue_load = [&](int n, uint32_t cbase) {
+        const int it = n / CS, cs = n % CS;
+        const uint32_t r = cbase + it;
+        const bool ok = (slab * CS + cs) * 8u + (lane >> 3) < bpr && r < r1;
+        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(
+            rsrc, ok ? (r - wg_r0) * row_bytes + lane_off + cs * 1024u : kOobOffset, 0, 0);
+    };
 #pragma unroll
-    for (int it = 0; it < RPW; ++it) {
-        const uint32_t r = r0 + it * RW + sub;
-        const uint32_t off = (col_ok && r < r1) ? (r - wg_r0) * row_bytes + lane_off : kOobOffset;
-        wv[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
-    }
+    for (int n = 0; n < PF; ++n) issue_load(n, r0);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) table_chunk(k);
 
-    // ---- pair table: tab[v*64 + h*32 + c] = level[h ? v>>4 : v&15] ----------------
-    for (uint32_t e = tid; e < 256 * 64 / 4; e += blockDim.x) {
-        const uint32_t rowi = e >> 3;                 // (v, h) pair: 8 float4 hold its 32 copies
-        const uint32_t v = rowi >> 1, h = rowi & 1u;
-        const float lv = kLv4[h ? (v >> 4) : (v & 15u)];
-        reinterpret_cast<float4*>(tab)[e] = make_float4(lv, lv, lv, lv);
-    }
+    // ---- x into LDS in nibble order -------------------------------------------------------------
+    // Weight i of a block sits at nibble p = i - i/64 + 4 (slots i % 64 == 63 own no nibble); lane
+    // lp of the block holds nibbles 32*lp .. 32*lp+31 and reads them as 8 float4 (c = 0..7), so
+    // x[i] goes to xs[blk*288 + c*32 + lp*4 + e] with p = 32*lp + 4*c + e.  The four scale
+    // nibbles (p < 4) and blocks past the end of the row hold zeros.
+    // A thread's float4 number d4 = tid + u*blockDim keeps the same position inside its block for
+    // every u when blockDim is a multiple of 64, so the four target offsets are computed once.
+    uint32_t xoff[4];
+    bool xlast_ok;
+    {
+        const uint32_t w = (tid * 4u) & 255u;
+        xlast_ok = (w & 63u) != 60u;                                          // i % 64 == 63 is a slot
 #pragma unroll
-    for (int u = 0; u < XPT; ++u) {
-        const uint32_t d = tid + u * blockDim.x;
-        if (d < kpad) {
-#pragma unroll
-            for (int m = 0; m < MB; ++m) xs[(size_t)m * kpad + d] = xpre[m][u];
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t pnib = w + k - (w >> 6) + 4u;
+            xoff[k] = ((pnib >> 2) & 7u) * 32u + (pnib >> 5) * 4u + (pnib & 3u);
         }
     }
-    for (uint32_t d = tid + XPT * blockDim.x; d < kpad; d += blockDim.x) {     // rows wider than XPT * workgroup
-        const uint32_t off = x_offset(d);
+    auto scatter4 = [&](uint32_t d4, const u32x4& v, int m) {
+        float* dst = xs + (size_t)m * xstride + (d4 >> 6) * kXsBlock;
+        dst[xoff[0]] = __uint_as_float(v.x);
+        dst[xoff[1]] = __uint_as_float(v.y);
+        dst[xoff[2]] = __uint_as_float(v.z);
+        if (xlast_ok) dst[xoff[3]] = __uint_as_float(v.w);
+    };
+    for (uint32_t bz = tid; bz < nblk * MB; bz += 512u) {                     // scale nibbles of every block
+        const uint32_t m = bz / nblk, b = bz % nblk;
+        *reinterpret_cast<float4*>(xs + (size_t)m * xstride + b * kXsBlock) = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    for (uint32_t z = bpr * 64u + tid; z < nblk * 64u; z += 512u) {           // blocks past the end of the row
 #pragma unroll
         for (int m = 0; m < MB; ++m)
-            xs[(size_t)m * kpad + d] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(
-                xrsrc, off == kOobOffset ? off : off + m * cols * 4u, 0, 0));
+            reinterpret_cast<float4*>(xs + (size_t)m * xstride + (z >> 6) * kXsBlock)[z & 63u] = make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int u = 0; u < XPT; ++u) {
+        const uint32_t d4 = tid + u * 512u;
+        if (d4 * 4u < cols) {
+#pragma unroll
+            for (int m = 0; m < MB; ++m) scatter4(d4, xpre[m][u], m);
+        }
+    }
+    for (uint32_t d4 = tid + XPT * 512u; d4 * 4u < cols; d4 += 512u) {    // rows wider than XPT*4*workgroup
+#pragma unroll
+        for (int m = 0; m < MB; ++m)
+            scatter4(d4, __builtin_amdgcn_raw_buffer_load_b128(
+                xrsrc, (m0 + m < M) ? d4 * 16u + m * cols * 4u : kOobOffset, 0, 0), m);
     }
     __syncthreads();
 
-    float xr[MB][32];
+    // ---- this lane's activations: 8 float4 per column set ------------------------------------
+    float xr[MB][CS][32];
 #pragma unroll
-    for (int m = 0; m < MB; ++m)
+    for (int cs = 0; cs < CS; ++cs) {
+        const uint32_t blk = (slab * CS + cs) * 8u + (lane >> 3);
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
-            const float4 t = *reinterpret_cast<const float4*>(xs + (size_t)m * kpad + (size_t)(slab * SB + (l >> 3)) * 256 + c * 32 + lp * 4);
-            xr[m][4 * c + 0] = t.x; xr[m][4 * c + 1] = t.y; xr[m][4 * c + 2] = t.z; xr[m][4 * c + 3] = t.w;
-        }
+        for (int m = 0; m < MB; ++m)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) {
+                const float4 t = *reinterpret_cast<const float4*>(xs + (size_t)m * xstride + blk * kXsBlock + c * 32 + lp * 4);
+                xr[m][cs][4 * c + 0] = t.x; xr[m][cs][4 * c + 1] = t.y; xr[m][cs][4 * c + 2] = t.z; xr[m][cs][4 * c + 3] = t.w;
+            }
+    }
 
-    const uint32_t lanebase = (lane & 31u) * 4u;      // byte offset of this lane's table copy
+    const uint32_t lanebase = (lane & 31u) * 8u;          // byte offset of this lane's table copy
 
     for (uint32_t ch = 0; ch < nchunks; ++ch) {
-        const uint32_t cbase = r0 + ch * CH;
+        const uint32_t cbase = r0 + ch * RPW;
         if (ch > 0) {
 #pragma unroll
-            for (int it = 0; it < RPW; ++it) {
-                const uint32_t r = cbase + it * RW + sub;
-                const uint32_t off = (col_ok && r < r1) ? (r - wg_r0) * row_bytes + lane_off : kOobOffset;
-                wv[it] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, off, 0, 0);
-            }
+            for (int n = 0; n < PF; ++n) issue_load(n, cbase);
         }
+#pragma unroll
+        for (int n = PF; n < NL; ++n) issue_load(n, cbase);
+        float part[MB][RPW];                              // per-lane partial of each row, block scales applied
         LevelPair cur[16];
-        lookup_row(wv[0], lanebase, cur);
+        lookup_load(wv[0], lanebase, cur);
 #pragma unroll
-        for (int it = 0; it < RPW; ++it) {
+        for (int n = 0; n < NL; ++n) {
+            const int it = n / CS, cs = n % CS;
             LevelPair nxt[16];
-            if (it + 1 < RPW) lookup_row(wv[it + 1], lanebase, nxt);      // next row's table reads fly during this row's FMAs
-            float acc[MB][4];
-#pragma unroll
-            for (int m = 0; m < MB; ++m) acc[m][0] = acc[m][1] = acc[m][2] = acc[m][3] = 0.0f;
-#pragma unroll
-            for (int k = 0; k < 16; ++k)
-#pragma unroll
-                for (int m = 0; m < MB; ++m) {
-                    acc[m][k & 3] = __fmaf_rn(cur[k].lo, xr[m][2 * k], acc[m][k & 3]);
-                    acc[m][k & 3] = __fmaf_rn(cur[k].hi, xr[m][2 * k + 1], acc[m][k & 3]);
-                }
-            const float scale = __half2float(__ushort_as_half((unsigned short)(wv[it].x & 0xFFFFu)));
-            float tot[MB];
+            if (n + 1 < NL) lookup_load(wv[n + 1], lanebase, nxt);    // next load's table reads fly during these FMAs
+            __builtin_amdgcn_sched_barrier(0);                        // keep them above the FMAs
+            // the block's FP16 scale sits in the low half of its first lane's first dword
+            const float scale = __half2float(__ushort_as_half((unsigned short)(dpp_bcast8(wv[n].x) & 0xFFFFu)));
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
-                float s = (acc[m][0] + acc[m][1]) + (acc[m][2] + acc[m][3]);
-                s += dpp_quad_xor1(s);
-                s += dpp_quad_xor2(s);
-                s += dpp_half_mirror(s);                       // all 8 lanes of the block: block sum
-                float v = (lp == 0) ? s * scale : 0.0f;        // one scaled value per block
-                if (SB >= 2) v += dpp_row_ror8(v);             // lanes 0 and 8 of each row of 16
-                if (SB == 8) tot[m] = (lane_value(v, 0) + lane_value(v, 16)) + (lane_value(v, 32) + lane_value(v, 48));
-                else if (SB == 4) tot[m] = sub == 0 ? lane_value(v, 0) + lane_value(v, 16) : lane_value(v, 32) + lane_value(v, 48);
-                else tot[m] = v;                               // SB <= 2: lane l == 0 of each slab row holds it
-            }
-            if (l == 0) {
+                float a0 = 0.0f, a1 = 0.0f;
 #pragma unroll
-                for (int m = 0; m < MB; ++m)
-                    red[(((size_t)grp * CH + it * RW + sub) * MB + m) * S + slab] = tot[m];
+                for (int k = 0; k < 16; k += 2) {
+                    a0 = __fmaf_rn(cur[k].lo, xr[m][cs][2 * k], a0);
+                    a0 = __fmaf_rn(cur[k].hi, xr[m][cs][2 * k + 1], a0);
+                    a1 = __fmaf_rn(cur[k + 1].lo, xr[m][cs][2 * k + 2], a1);
+                    a1 = __fmaf_rn(cur[k + 1].hi, xr[m][cs][2 * k + 3], a1);
+                }
+                part[m][it] = cs == 0 ? (a0 + a1) * scale : __fmaf_rn(a0 + a1, scale, part[m][it]);
             }
-            if (it + 1 < RPW) {
+            if (n + 1 < NL) {
 #pragma unroll
                 for (int k = 0; k < 16; ++k) cur[k] = nxt[k];
             }
+            __builtin_amdgcn_sched_barrier(0);                        // one scheduling region per wave-load
+        }
+        // ---- all rows of the chunk reduced over the 64 lanes together (independent chains) ----
+#pragma unroll
+        for (int it = 0; it < RPW; ++it)
+#pragma unroll
+            for (int m = 0; m < MB; ++m) {
+                float v = part[m][it];
+                v += dpp_quad_xor1(v);
+                v += dpp_quad_xor2(v);
+                v += dpp_half_mirror(v);
+                v += dpp_row_mirror(v);
+                v += dpp_row_bcast15(v);
+                v += dpp_row_bcast31(v);
+                part[m][it] = v;                          // lane 63 holds the slab's dot product
+            }
+        if (S == 1) {                                     // a wave covers whole rows: lane 63 stores y
+            if (lane == 63) {
+#pragma unroll
+                for (int it = 0; it < RPW; ++it)
+#pragma unroll
+                    for (int m = 0; m < MB; ++m)
+                        if (cbase + it < r1 && m0 + m < M) y[(size_t)(m0 + m) * rows + cbase + it] = part[m][it];
+            }
+            continue;
+        }
+        if (lane == 63 && working) {
+#pragma unroll
+            for (int it = 0; it < RPW; ++it)
+#pragma unroll
+                for (int m = 0; m < MB; ++m)
+                    red[(((size_t)grp * RPW + it) * MB + m) * S + slab] = part[m][it];
         }
         __syncthreads();
         // ---- slab partials -> y -------------------------------------------------
-        for (uint32_t o = tid; o < G * CH * MB; o += blockDim.x) {
-            const uint32_t g2 = o / (CH * MB), rem = o % (CH * MB), slot = rem / MB, m = rem % MB;
+        for (uint32_t o = tid; o < G * RPW * MB; o += 512u) {
+            const uint32_t g2 = o / (RPW * MB), rem = o % (RPW * MB), slot = rem / MB, m = rem % MB;
             const uint32_t jg2 = blockIdx.x * G + g2;
-            const uint32_t q0 = (uint32_t)(((uint64_t)rows * jg2) / J);
-            const uint32_t q1 = (uint32_t)(((uint64_t)rows * (jg2 + 1)) / J);
-            const uint32_t r = q0 + ch * CH + slot;
+            const uint32_t q0 = group_begin(jg2), q1 = group_begin(jg2 + 1);
+            const uint32_t r = q0 + ch * RPW + slot;
             if (r < q1 && m0 + (int)m < M) {
                 const float* pr = red + (size_t)o * S;
                 float s = 0.0f;
@@ -244,72 +340,71 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
 
 // One launch configuration of the kernel above.
 struct Oil4Plan {
-    int sb, rpw, maxt;     // template choice
+    int cs, rpw, maxt;     // template choice
     uint32_t S, G, grid, nchunks;
     size_t lds_bytes;
 };
 
-template <int SB, int RPW, int MB, int MAXT>
+template <int CS, int RPW, int MB, int MAXT>
 int launch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
     static bool attr_done = false;
-    auto kern = gemv_oil4_kernel<SB, RPW, MB, MAXT>;
+    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT>;
     if (!attr_done) {
         OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
+    const uint32_t J = p.grid * p.G;
     for (int m0 = 0; m0 < M; m0 += MB) {
-        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(p.S * p.G * 64), p.lds_bytes, s, w.d_payload, d_x, d_y,
-                           (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M);
+        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_y,
+                           (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M,
+                           (uint32_t)w.rows / J, (uint32_t)w.rows % J);
         OILHIP_HIP(hipGetLastError());
     }
     return OILHIP_OK;
 }
 
-// Chooses slab width, waves per workgroup and chunking for a shape.
-// waves_target: 8 (two waves per SIMD, deep per-wave pipelining) or 16.
+// Chooses column sets per wave, slabs, waves per workgroup and chunking for a shape.
 bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan* p) {
-    const uint32_t bpr = cols >> 8;
-    int sb = 1;
-    for (int cand : {8, 4, 2}) {       // widest slab that wastes <= ~3 % of lanes on the ragged last slab
-        const uint32_t slabs = (bpr + cand - 1) / cand;
-        if ((double)(slabs * cand - bpr) / (double)(slabs * cand) <= 0.03) { sb = cand; break; }
+    const uint32_t sets = ((cols >> 8) + 7) / 8;                  // column sets (1 KB wave-loads) per row
+    const int cs_max = MB == 1 ? 3 : 1;                           // register budget: 32*CS*MB activations per lane
+    // fewest slabs first (less cross-wave reduction), then least padding
+    int best_cs = 1; uint32_t best_S = sets; double best_cost = 1e30;
+    for (int cs = 1; cs <= cs_max; ++cs) {
+        const uint32_t S = (sets + cs - 1) / cs;
+        if (S > (uint32_t)waves_target) continue;
+        const double waste = (double)(S * cs) / (double)sets;      // >= 1: padded column sets cost ALU time
+        const double cost = waste + 0.04 * (S > 1 ? S : 0);
+        if (cost < best_cost) { best_cost = cost; best_cs = cs; best_S = S; }
     }
-    uint32_t S = (bpr + sb - 1) / sb;
-    while (S > 16 && sb < 8) { sb *= 2; S = (bpr + sb - 1) / sb; }
-    if (S > 16) return false;
+    if (best_cost > 1e29) return false;
+    const uint32_t S = best_S;
     uint32_t G = (uint32_t)waves_target / S;
     if (G == 0) G = 1;
-    const int RW = 64 / (8 * sb);
     uint32_t grid = (uint32_t)device_cu_count();
-    const uint32_t max_groups = (rows + RW - 1) / RW;
-    if (grid * G > max_groups) grid = (max_groups + G - 1) / G;
+    if (grid * G > rows) grid = (rows + G - 1) / G;
     if (grid == 0) grid = 1;
     const uint32_t Jn = grid * G;
-    const uint32_t max_rows = (rows + Jn - 1) / Jn;                 // rows of the largest row group
-    const uint32_t loads = (max_rows + RW - 1) / RW;                // wave-loads it needs
-    const int rpw = loads <= 4 ? 4 : (loads <= 6 ? 6 : (loads <= 8 ? 8 : 12));
-    const uint32_t CH = (uint32_t)rpw * RW;
-    p->sb = sb; p->rpw = rpw; p->maxt = (S * G > 12) ? 1024 : ((S * G > 8) ? 768 : 512);
+    const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
+    const int budget = 12 / best_cs;                               // <= 12 wave-loads in flight per wave
+    int rpw = 1;
+    for (int cand : {1, 2, 3, 4, 6, 12}) if (cand <= budget) { rpw = cand; if ((uint32_t)cand >= max_rows) break; }
+    p->cs = best_cs; p->rpw = rpw; p->maxt = 512;
     p->S = S; p->G = G; p->grid = grid;
-    p->nchunks = (max_rows + CH - 1) / CH;
+    p->nchunks = (max_rows + rpw - 1) / rpw;
     if (p->nchunks == 0) p->nchunks = 1;
-    p->lds_bytes = (size_t)kTabBytes + 4ull * MB * S * sb * 256 + 4ull * G * CH * MB * S;
-    return p->lds_bytes <= (size_t)kMaxLds;
+    p->lds_bytes = (size_t)kTabBytes + 4ull * MB * (S * best_cs * 8 * kXsBlock) + 4ull * G * rpw * MB * S + 64;
+    return p->lds_bytes <= (size_t)kMaxLds && S * G <= 8;
 }
 
 template <int MB>
 int dispatch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
-#define OIL4_CASE(SB_, RPW_, MAXT_) \
-    if (p.sb == SB_ && p.rpw == RPW_ && p.maxt == MAXT_) return launch<SB_, RPW_, MB, MAXT_>(w, d_x, d_y, M, s, p);
-    OIL4_CASE(8, 4, 512) OIL4_CASE(8, 6, 512) OIL4_CASE(8, 8, 512) OIL4_CASE(8, 12, 512)
-    OIL4_CASE(4, 4, 512) OIL4_CASE(4, 6, 512) OIL4_CASE(4, 8, 512) OIL4_CASE(4, 12, 512)
-    OIL4_CASE(2, 4, 512) OIL4_CASE(2, 6, 512) OIL4_CASE(2, 8, 512) OIL4_CASE(2, 12, 512)
-    OIL4_CASE(1, 4, 512) OIL4_CASE(1, 6, 512) OIL4_CASE(1, 8, 512) OIL4_CASE(1, 12, 512)
-    OIL4_CASE(8, 4, 768) OIL4_CASE(8, 8, 768) OIL4_CASE(4, 4, 768) OIL4_CASE(4, 8, 768)
-    OIL4_CASE(2, 4, 768) OIL4_CASE(2, 8, 768) OIL4_CASE(1, 4, 768) OIL4_CASE(1, 8, 768)
+#define OIL4_CASE(CS_, RPW_) \
+    if (p.cs == CS_ && p.rpw == RPW_) return launch<CS_, RPW_, MB, 512>(w, d_x, d_y, M, s, p);
+    OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
     if constexpr (MB == 1) {
-        OIL4_CASE(8, 4, 1024) OIL4_CASE(4, 4, 1024) OIL4_CASE(2, 4, 1024) OIL4_CASE(1, 4, 1024)
+        OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)
+        OIL4_CASE(3, 1) OIL4_CASE(3, 2) OIL4_CASE(3, 3) OIL4_CASE(3, 4)
     }
 #undef OIL4_CASE
     return 1;
@@ -317,35 +412,11 @@ int dispatch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipSt
 
 }  // namespace
 
-// OILHIP_OIL4_WAVES=8|16 overrides the waves-per-workgroup target (tuning aid).
-static int waves_target_default() {
-    static int v = [] {
-        const char* e = getenv("OILHIP_OIL4_WAVES");
-        const int n = e ? atoi(e) : 0;
-        return (n == 8 || n == 16) ? n : 8;
-    }();
-    return v;
-}
-
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || M > 16) return 1;
     Oil4Plan p;
     const int MB = M == 1 ? 1 : 2;
-    int wt = waves_target_default();
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, wt, &p)) return 1;
-    // register budget: 12 waves leave 170 VGPRs (chunks of <= 8 loads), 16 waves 128 (chunks of 4, M = 1 only)
-    const int cap = p.maxt == 1024 ? 4 : (p.maxt == 768 ? (MB == 1 ? 8 : 4) : 12);
-    if (p.maxt == 1024 && MB != 1) return 1;
-    if (p.maxt == 768 && p.rpw == 6) p.rpw = 8;
-    if (p.rpw > cap) p.rpw = cap;
-    {
-        const uint32_t RW = 64u / (8u * p.sb), Jn = p.grid * p.G;
-        const uint32_t max_rows = ((uint32_t)w.rows + Jn - 1) / Jn, CH = (uint32_t)p.rpw * RW;
-        p.nchunks = (max_rows + CH - 1) / CH;
-        if (p.nchunks == 0) p.nchunks = 1;
-        p.lds_bytes = (size_t)kTabBytes + 4ull * MB * p.S * p.sb * 256 + 4ull * p.G * CH * MB * p.S;
-        if (p.lds_bytes > (size_t)kMaxLds) return 1;
-    }
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) return 1;
     return MB == 1 ? dispatch<1>(w, d_x, d_y, M, s, p) : dispatch<2>(w, d_x, d_y, M, s, p);
 }
 
