@@ -1,8 +1,244 @@
-// gemm_oil4_mfma.hip -- prefill GEMM over uniform OIL4 tensors (placeholder until the MFMA kernel lands).
+// gemm_oil4_mfma.hip -- prefill GEMM over uniform OIL4 tensors on the matrix cores:
+// Y[M][N] = X[M][K] . W^T with X in bf16, W dequantized tile by tile to bf16 in LDS,
+// v_mfma_f32_32x32x16_bf16, FP32 accumulation, FP32 output.  Same contraction as the
+// reference's FP32 prefill (Qwen35Engine::gemm with B up to 512,
+// src/adapters/tools/qwen35_engine.cpp:47-85,630-753) over dequant_lattice blocks
+// (src/block_codec.cpp:173-182).
+//
+// The contraction runs in nibble order: inside a 256-weight block the 4-bit index of
+// weight i sits at nibble p = 4 + i - i/64 (nibbles 0..3 are the FP16 scale, weights
+// 63,127,191,255 are slots that decode to zero and own no nibble).  A small pre-pass
+// writes X' with X'[m][blk*256 + p] = X[m][blk*256 + i(p)] and zeros at p < 4, so the
+// main kernel multiplies consecutive nibbles with consecutive X' columns and never
+// needs a shift across bytes; the scale nibbles meet zeros.
+//
+// Main kernel: workgroup = 2 x 2 wavefronts, each wavefront owns WBM x WBN blocks of
+// 32 x 32 outputs.  Per 64-column step the workgroup stages an X' tile and a weight tile
+// in LDS; the weight tile goes through the same byte -> (level, level) pair table as the
+// decode GEMV (one v_perm_b32 + one LDS read per packed byte), is multiplied by the
+// block's FP16 scale in FP32 and rounded once to bf16.
+#include <hip/hip_fp16.h>
+
+#include <cstdlib>
+#include <mutex>
+
 #include "common.h"
 
 namespace oilhip {
-int launch_gemm_oil4_bf16(const oilhip_weights&, const uint16_t*, float*, int, hipStream_t) {
-    return fail(OILHIP_E_ARG, "bf16 prefill GEMM kernel is not built into this library yet");
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const f32x2 lds_cfloat2;
+
+constexpr int kTabBytes = 256 * 64 * 4;     // pair table: byte v, lane copy c at v*256 + c*8
+constexpr int BK = 64;                      // columns per step (a quarter of a block)
+constexpr int LDK = BK + 8;                 // LDS row pitch in bf16: 144 bytes keeps 16-byte reads of 16 rows on distinct banks
+
+__device__ __forceinline__ float level_literal(uint32_t i) {      // kOIL4Levels, src/block_codec.cpp:18-23
+    const float mag = (i == 7 || i == 8) ? 0.1260f : (i == 6 || i == 9) ? 0.3976f : (i == 5 || i == 10) ? 0.6508f
+                    : (i == 4 || i == 11) ? 0.9275f : (i == 3 || i == 12) ? 1.2392f : (i == 2 || i == 13) ? 1.5995f
+                    : (i == 1 || i == 14) ? 2.0522f : 2.7178f;
+    return i < 8 ? -mag : mag;
 }
+
+// X (bf16 bit patterns, [M][K]) -> X' ([Mpad][K], rows >= M zero), columns in nibble order.
+__global__ void __launch_bounds__(256)
+permute_x_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ xp, uint32_t M, uint32_t K, uint32_t Mpad) {
+    const uint32_t row = blockIdx.y;
+    for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < K; c += gridDim.x * 256) {
+        const uint32_t p = c & 255u;
+        uint16_t v = 0;
+        if (p >= 4 && row < M) {
+            const uint32_t q = p - 4;
+            v = x[(size_t)row * K + (c - p) + q + (q >= 63) + (q >= 126) + (q >= 189)];
+        }
+        xp[(size_t)row * K + c] = v;
+    }
+}
+
+template <int WBM, int WBN>
+__global__ void __launch_bounds__(256)
+gemm_oil4_bf16_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
+                      uint32_t M, uint32_t N, uint32_t K, uint32_t Mpad) {
+    constexpr int BM = 64 * WBM, BN = 64 * WBN;
+    constexpr int A_CHUNKS = BM * 8 / 256;          // 16-byte pieces of the X' tile per thread
+    constexpr int B_CHUNKS = BN * 2 / 256;          // 16-byte pieces (32 nibbles) of the weight tile per thread
+    static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1, "tile too small for 256 threads");
+    extern __shared__ __align__(16) uint8_t lds[];
+    float* tab = reinterpret_cast<float*>(lds);                                   // LDS byte offset 0
+    __bf16* As = reinterpret_cast<__bf16*>(lds + kTabBytes);                      // [BM][LDK]
+    __bf16* Bs = As + BM * LDK;                                                   // [BN][LDK]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+    const uint32_t bpr = K >> 8, KT = K / BK;
+
+    {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 256*k
+        const float lv_lane = level_literal(lane & 15u);
+        const float lo = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const float hi = level_literal(k);
+            reinterpret_cast<float4*>(tab)[tid + 256u * k] = make_float4(lo, hi, lo, hi);
+        }
+    }
+
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(W + (size_t)n0 * bpr * 128u), 0,
+        (int)((uint64_t)(N - n0 < (uint32_t)BN ? N - n0 : (uint32_t)BN) * bpr * 128u), 0x00020000);
+    const uint16_t* xa = Xp + (size_t)m0 * K;
+
+    u32x4 ar[A_CHUNKS], br[B_CHUNKS];
+    uint32_t sr[B_CHUNKS];
+    auto load_tiles = [&](uint32_t kt) {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const uint32_t id = tid + c * 256u, row = id >> 3, kc = id & 7u;
+            ar[c] = *reinterpret_cast<const u32x4*>(xa + (size_t)row * K + kt * BK + kc * 8u);
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; ++c) {
+            const uint32_t id = tid + c * 256u, row = id >> 1, half = id & 1u;
+            const uint32_t blk_off = (row * bpr + (kt >> 2)) * 128u;
+            br[c] = __builtin_amdgcn_raw_buffer_load_b128(wrs, blk_off + (kt & 3u) * 32u + half * 16u, 0, 0);
+            sr[c] = __builtin_amdgcn_raw_buffer_load_b16(wrs, blk_off, 0, 0);     // the block's FP16 scale
+        }
+    };
+    const uint32_t lanebase = (lane & 31u) * 8u;
+    auto store_tiles = [&]() {
+#pragma unroll
+        for (int c = 0; c < A_CHUNKS; ++c) {
+            const uint32_t id = tid + c * 256u, row = id >> 3, kc = id & 7u;
+            *reinterpret_cast<u32x4*>(As + row * LDK + kc * 8u) = ar[c];
+        }
+#pragma unroll
+        for (int c = 0; c < B_CHUNKS; ++c) {
+            const uint32_t id = tid + c * 256u, row = id >> 1, half = id & 1u;
+            const float scale = __half2float(__ushort_as_half((unsigned short)sr[c]));
+            const uint32_t wd[4] = {br[c].x, br[c].y, br[c].z, br[c].w};
+            uint32_t packed[16];
+#pragma unroll
+            for (int d = 0; d < 4; ++d)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t addr = __builtin_amdgcn_perm(wd[d], lanebase, 0x0C0C0000u | ((4u + j) << 8));
+                    const f32x2 t = *(lds_cfloat2*)(uintptr_t)addr;
+                    const bf16x2 pr = bf16x2{(__bf16)(t.x * scale), (__bf16)(t.y * scale)};
+                    packed[d * 4 + j] = *reinterpret_cast<const uint32_t*>(&pr);
+                }
+            u32x4* dst = reinterpret_cast<u32x4*>(Bs + row * LDK + half * 32u);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) dst[q] = u32x4{packed[4 * q], packed[4 * q + 1], packed[4 * q + 2], packed[4 * q + 3]};
+        }
+    };
+
+    f32x16 acc[WBM][WBN];
+#pragma unroll
+    for (int i = 0; i < WBM; ++i)
+#pragma unroll
+        for (int j = 0; j < WBN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    load_tiles(0);
+    __syncthreads();                                   // table complete
+    for (uint32_t kt = 0; kt < KT; ++kt) {
+        store_tiles();
+        __syncthreads();
+        if (kt + 1 < KT) load_tiles(kt + 1);           // next tile's global loads fly during the MFMAs
+        const __bf16* ap = As + (wm * WBM * 32u + (lane & 31u)) * LDK + (lane >> 5) * 8u;
+        const __bf16* bp = Bs + (wn * WBN * 32u + (lane & 31u)) * LDK + (lane >> 5) * 8u;
+#pragma unroll
+        for (int kk = 0; kk < BK / 16; ++kk) {
+            bf16x8 a[WBM], b[WBN];
+#pragma unroll
+            for (int i = 0; i < WBM; ++i) a[i] = *reinterpret_cast<const bf16x8*>(ap + i * 32 * LDK + kk * 16);
+#pragma unroll
+            for (int j = 0; j < WBN; ++j) b[j] = *reinterpret_cast<const bf16x8*>(bp + j * 32 * LDK + kk * 16);
+#pragma unroll
+            for (int i = 0; i < WBM; ++i)
+#pragma unroll
+                for (int j = 0; j < WBN; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+
+    // C layout of the 32x32 MFMA: lane l holds column l % 32; register v holds row 8*(v/4) + 4*(l/32) + v%4
+#pragma unroll
+    for (int i = 0; i < WBM; ++i)
+#pragma unroll
+        for (int j = 0; j < WBN; ++j) {
+            const uint32_t col = n0 + (wn * WBN + j) * 32u + (lane & 31u);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t row = m0 + (wm * WBM + i) * 32u + 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u);
+                if (row < M && col < N) Y[(size_t)row * N + col] = acc[i][j][v];
+            }
+        }
+}
+
+// grow-only device scratch for X' (one per process and device; calls that overlap on one device race on it)
+std::mutex g_scratch_mu;
+uint16_t* g_scratch[64] = {};
+size_t g_scratch_bytes[64] = {};
+
+int get_scratch(size_t bytes, uint16_t** out) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_bytes[dev] < bytes) {
+        if (g_scratch[dev]) {
+            OILHIP_HIP(hipDeviceSynchronize());
+            OILHIP_HIP(hipFree(g_scratch[dev]));
+            g_scratch[dev] = nullptr;
+            g_scratch_bytes[dev] = 0;
+        }
+        OILHIP_HIP(hipMalloc(&g_scratch[dev], bytes));
+        g_scratch_bytes[dev] = bytes;
+    }
+    *out = g_scratch[dev];
+    return OILHIP_OK;
+}
+
+template <int WBM, int WBN>
+int launch(const oilhip_weights& w, const uint16_t* xp, float* d_y, uint32_t M, uint32_t Mpad, hipStream_t s) {
+    constexpr int BM = 64 * WBM, BN = 64 * WBN;
+    const size_t lds_bytes = (size_t)kTabBytes + (size_t)(BM + BN) * LDK * 2;
+    static bool attr_done = false;
+    auto kern = gemm_oil4_bf16_kernel<WBM, WBN>;
+    if (!attr_done) {
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        attr_done = true;
+    }
+    const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols;
+    hipLaunchKernelGGL(kern, dim3((N + BN - 1) / BN, Mpad / BM), dim3(256), lds_bytes, s, w.d_payload, xp, d_y, M, N, K, Mpad);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+}  // namespace
+
+int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s) {
+    if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
+    const uint32_t K = (uint32_t)w.cols;
+    static const int tile = [] { const char* e = getenv("OILHIP_GEMM_TILE"); return e ? atoi(e) : 0; }();
+    const bool big = tile ? tile == 256 : M > 256;
+    const uint32_t BM = big ? 256 : 128;
+    const uint32_t Mpad = ((uint32_t)M + BM - 1) / BM * BM;
+    uint16_t* xp = nullptr;
+    if (int rc = get_scratch((size_t)Mpad * K * 2, &xp)) return rc;
+    uint32_t gx = (K + 255) / 256;
+    if (gx > 64) gx = 64;
+    hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
+    OILHIP_HIP(hipGetLastError());
+    return big ? launch<4, 4>(w, xp, d_y, (uint32_t)M, Mpad, s) : launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
+}
+
 }  // namespace oilhip
