@@ -1,0 +1,101 @@
+// oilhip_shims.hpp -- C++20 drop-in layer over the C ABI (oilhip.h): the reference's own
+// entry points for this path, same namespaces, names, argument meaning and error
+// behaviour, taking host pointers like the reference does.  Each shim uploads its
+// operands, runs the HIP kernel and copies the result back; there is no CPU fallback
+// (a missing GPU or a failed launch throws oil::Error).
+//
+// Built inside the reference tree the shim sources include the reference's own headers
+// (oil/types.h ...) so the signatures are the reference's by construction; built
+// stand-alone they use the minimal declarations below.
+#pragma once
+#include <cstddef>
+#include <cstdint>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#if __has_include("oil/types.h")
+#include "oil/types.h"
+#else
+namespace oil {
+// include/oil/types.h:19-35 (values pinned by tests/test_format.cpp:183-186)
+enum class Format : uint8_t {
+    OIL1 = 0, SPARK_Q0 = 1, OIL2 = 2, OIL4 = 3, OIL8 = 4, OIL16 = 5, OIL32 = 6, OIL1_GRP = 7,
+    SPARK_Q0_GRP = 8, OIL2_GRP = 9, OIL4_GRP = 10, OIL8_GRP = 11, OIL16_GRP = 12,
+    SPARK_SPARSE = 13, SPARK_SPARSE_GRP = 14,
+};
+// include/oil/types.h:184-187
+class Error : public std::runtime_error {
+public:
+    explicit Error(const std::string& msg) : std::runtime_error(msg) {}
+};
+}  // namespace oil
+#endif
+
+namespace oil {
+
+// include/oil/block_codec.h:55-63
+bool quantize_block_all(Format fmt, const float* w, int n, std::vector<uint8_t>& indices, std::vector<uint8_t>& codebook);
+void dequantize_block_all(Format fmt, const uint8_t* indices, size_t idx_bytes, const uint8_t* codebook,
+                          size_t cb_bytes, uint32_t nw, float* out);
+
+namespace kernel {
+// include/oil/kernel.h:24-32
+void oil8_gemm(const uint8_t* indices, const float* codebook, const float* activations, float* output, int M, int N, int K);
+void oil4_gemm(const uint8_t* packed_indices, const uint16_t* codebook, const float* activations, float* output, int M, int N, int K);
+}  // namespace kernel
+
+namespace adapters::prod {
+// include/oil/kernel_production.h:19-52; detect_cpu_isa() keeps its name, 950 = the gfx950 device path
+int detect_cpu_isa();
+void gemv_spark_tiled(const uint8_t* packed_w, float scale, const float* x, float* y, int M, int K, int tile_m = 32);
+void gemv_oil4_tiled(const uint8_t* packed_indices, const uint16_t* codebook, float scale, const float* x, float* y, int M, int K, int tile_m = 32);
+void gemv_oil8_tiled(const uint8_t* indices, const float* codebook, float scale, const float* x, float* y, int M, int K, int tile_m = 32);
+void gemv_spark_batch(const uint8_t* packed_w, float scale, const float* X, float* Y, int M, int N, int K);
+void gemv_oil4_batch(const uint8_t* packed_indices, const uint16_t* codebook, float scale, const float* X, float* Y, int M, int N, int K);
+void gemv_oil8_batch(const uint8_t* indices, const float* codebook, float scale, const float* X, float* Y, int M, int N, int K);
+}  // namespace adapters::prod
+
+namespace gfx950 {
+
+// Body of OIL{8,4,2}Engine::quant_gemm (include/oil/oil_engines.h:49,78,151) on host pointers:
+// C[m*N+n] = sum_k A[m*K+k] * codebook[code(k*N+n)].
+void engine_quant_gemm(int bits, const float* a, const uint8_t* b_idx, const float* codebook, float* c,
+                       int64_t M, int64_t N, int64_t K);
+
+// One block as the .oil file stores it (OILWriter::write_block, src/oil_format.cpp:219-233).
+struct BlockRef {
+    Format format;
+    const uint8_t* codebook; uint32_t cb_bytes;
+    const uint8_t* indices;  uint32_t idx_bytes;
+    uint32_t num_weights;
+};
+
+// A tensor of .oil blocks resident in HBM: what Qwen35Engine::Th + OILReader give the
+// reference's gemm (include/oil/qwen35_engine.h:29,38).  gemm() is that function:
+// Y[b*rows + r] = sum_c W[r][c] * X[b*cols + c], host pointers, FP32, any B >= 1.
+class DeviceTensor {
+public:
+    DeviceTensor(const std::vector<BlockRef>& blocks, uint64_t rows, uint64_t cols);
+    // raw block records [nw][cb_bytes][cb][idx_bytes][idx] back to back + one format id per block
+    DeviceTensor(const uint8_t* records, uint64_t record_bytes, const uint8_t* formats, uint32_t nblocks,
+                 uint64_t rows, uint64_t cols);
+    ~DeviceTensor();
+    DeviceTensor(const DeviceTensor&) = delete;
+    DeviceTensor& operator=(const DeviceTensor&) = delete;
+    void gemm(const float* X, float* Y, int B) const;
+    void dequantize(float* out) const;                    // rows*cols floats, bit-exact with dequantize_block_all
+    uint64_t rows() const { return rows_; }
+    uint64_t cols() const { return cols_; }
+    uint64_t payload_bytes() const;
+private:
+    void* handle_ = nullptr;
+    uint64_t rows_ = 0, cols_ = 0;
+};
+
+// backend::probe_hardware / select_optimal_backend hook (include/oil/backend.h:98-139):
+// true when a gfx950 device is usable; fills name and HBM size when given.
+bool probe(std::string* name = nullptr, uint64_t* hbm_bytes = nullptr, int* compute_units = nullptr);
+
+}  // namespace gfx950
+}  // namespace oil

@@ -1,0 +1,201 @@
+// oil_shims.cpp -- host-pointer C++ shims over the C ABI (see include/oilhip_shims.hpp).
+#include "../../../include/oilhip_shims.hpp"
+
+#include <hip/hip_runtime.h>
+
+#include <cstring>
+
+#include "../../../include/oilhip.h"
+
+namespace {
+
+[[noreturn]] void raise(const char* what) {
+    throw oil::Error(std::string(what) + ": " + oilhip_last_error());
+}
+void ok(int rc, const char* what) {
+    if (rc != OILHIP_OK) raise(what);
+}
+void hip_ok(hipError_t e, const char* what) {
+    if (e != hipSuccess) throw oil::Error(std::string(what) + ": " + hipGetErrorString(e));
+}
+
+// Device buffer holding a copy of a host range (or an output range).
+template <class T>
+class Dev {
+public:
+    Dev(const T* host, size_t n) : n_(n) {
+        if (n_ == 0) return;
+        hip_ok(hipMalloc(&p_, n_ * sizeof(T)), "hipMalloc");
+        if (host) hip_ok(hipMemcpy(p_, host, n_ * sizeof(T), hipMemcpyHostToDevice), "hipMemcpy H2D");
+    }
+    ~Dev() { if (p_) (void)hipFree(p_); }
+    Dev(const Dev&) = delete;
+    Dev& operator=(const Dev&) = delete;
+    T* get() const { return p_; }
+    void to_host(T* host) const {
+        if (n_) hip_ok(hipMemcpy(host, p_, n_ * sizeof(T), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    }
+private:
+    T* p_ = nullptr;
+    size_t n_;
+};
+
+size_t sz(long long v) { return v < 0 ? 0 : (size_t)v; }
+
+}  // namespace
+
+namespace oil {
+
+bool quantize_block_all(Format fmt, const float* w, int n, std::vector<uint8_t>& indices, std::vector<uint8_t>& codebook) {
+    indices.clear();
+    codebook.clear();
+    if (!w || n <= 0 || (int)fmt > 14) return false;                  // block_codec.cpp:370,571-572
+    const size_t bound = oilhip_payload_bound((int)fmt, n);
+    indices.resize(bound ? bound : 1);
+    codebook.resize(2 * (((size_t)n + 31) / 32) + 2);
+    size_t il = 0, cl = 0;
+    if (oilhip_quantize_block((int)fmt, w, n, indices.data(), indices.size(), &il, codebook.data(), codebook.size(), &cl) != OILHIP_OK)
+        return false;
+    indices.resize(il);
+    codebook.resize(cl);
+    return true;
+}
+
+void dequantize_block_all(Format fmt, const uint8_t* indices, size_t idx_bytes, const uint8_t* codebook,
+                          size_t cb_bytes, uint32_t nw, float* out) {
+    if (!out || nw == 0) return;                                       // block_codec.cpp:580
+    if ((int)fmt > 14 || nw > (1u << 24) || cb_bytes > 0xFFFF) {       // unhandled input decodes to zeros (:717-718)
+        std::memset(out, 0, sizeof(float) * nw);
+        return;
+    }
+    const gfx950::BlockRef b{fmt, codebook, (uint32_t)cb_bytes, indices, (uint32_t)idx_bytes, nw};
+    gfx950::DeviceTensor t(std::vector<gfx950::BlockRef>{b}, 1, nw);
+    t.dequantize(out);
+}
+
+namespace kernel {
+
+void oil8_gemm(const uint8_t* indices, const float* codebook, const float* activations, float* output, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    Dev<uint8_t> i(indices, sz(N) * sz(K));
+    Dev<float> c(codebook, 256), a(activations, sz(M) * sz(K)), o(nullptr, sz(M) * sz(N));
+    ok(oilhip_flat_oil8_gemm(i.get(), c.get(), a.get(), o.get(), M, N, K, nullptr), "oil8_gemm");
+    o.to_host(output);
+}
+
+void oil4_gemm(const uint8_t* packed, const uint16_t* codebook, const float* activations, float* output, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    Dev<uint8_t> i(packed, (sz(M) * sz(N) * sz(K) + 1) / 2);
+    Dev<uint16_t> c(codebook, 16);
+    Dev<float> a(activations, sz(N) * sz(K)), o(nullptr, sz(M) * sz(N));
+    ok(oilhip_flat_oil4_gemm(i.get(), c.get(), a.get(), o.get(), M, N, K, nullptr), "oil4_gemm");
+    o.to_host(output);
+}
+
+}  // namespace kernel
+
+namespace adapters::prod {
+
+int detect_cpu_isa() {
+    int gfx = 0;
+    return oilhip_probe(&gfx, nullptr, nullptr, nullptr, 0) == OILHIP_OK ? gfx : 0;
+}
+
+void gemv_spark_batch(const uint8_t* w, float scale, const float* X, float* Y, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    Dev<uint8_t> dw(w, sz(M) * ((sz(K) + 3) / 4));
+    Dev<float> x(X, sz(N) * sz(K)), y(nullptr, sz(N) * sz(M));
+    ok(oilhip_prod_gemv_spark(dw.get(), scale, x.get(), y.get(), M, K, N, nullptr), "gemv_spark");
+    y.to_host(Y);
+}
+void gemv_oil4_batch(const uint8_t* w, const uint16_t* cb, float scale, const float* X, float* Y, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    Dev<uint8_t> dw(w, sz(M) * ((sz(K) + 1) / 2));
+    Dev<uint16_t> c(cb, 16);
+    Dev<float> x(X, sz(N) * sz(K)), y(nullptr, sz(N) * sz(M));
+    ok(oilhip_prod_gemv_oil4(dw.get(), c.get(), scale, x.get(), y.get(), M, K, N, nullptr), "gemv_oil4");
+    y.to_host(Y);
+}
+void gemv_oil8_batch(const uint8_t* w, const float* cb, float scale, const float* X, float* Y, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    Dev<uint8_t> dw(w, sz(M) * sz(K));
+    Dev<float> c(cb, 256), x(X, sz(N) * sz(K)), y(nullptr, sz(N) * sz(M));
+    ok(oilhip_prod_gemv_oil8(dw.get(), c.get(), scale, x.get(), y.get(), M, K, N, nullptr), "gemv_oil8");
+    y.to_host(Y);
+}
+void gemv_spark_tiled(const uint8_t* w, float scale, const float* x, float* y, int M, int K, int) {
+    gemv_spark_batch(w, scale, x, y, M, 1, K);
+}
+void gemv_oil4_tiled(const uint8_t* w, const uint16_t* cb, float scale, const float* x, float* y, int M, int K, int) {
+    gemv_oil4_batch(w, cb, scale, x, y, M, 1, K);
+}
+void gemv_oil8_tiled(const uint8_t* w, const float* cb, float scale, const float* x, float* y, int M, int K, int) {
+    gemv_oil8_batch(w, cb, scale, x, y, M, 1, K);
+}
+
+}  // namespace adapters::prod
+
+namespace gfx950 {
+
+void engine_quant_gemm(int bits, const float* a, const uint8_t* b_idx, const float* codebook, float* c,
+                       int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0) return;
+    if (bits != 2 && bits != 4 && bits != 8) throw Error("engine_quant_gemm: bits must be 2, 4 or 8");
+    Dev<float> da(a, sz(M) * sz(K)), dc(codebook, (size_t)1 << bits), out(nullptr, sz(M) * sz(N));
+    Dev<uint8_t> db(b_idx, (sz(K) * sz(N) * (size_t)bits + 7) / 8);
+    ok(oilhip_engine_quant_gemm(bits, da.get(), db.get(), dc.get(), out.get(), M, N, K, nullptr), "quant_gemm");
+    out.to_host(c);
+}
+
+DeviceTensor::DeviceTensor(const std::vector<BlockRef>& blocks, uint64_t rows, uint64_t cols) : rows_(rows), cols_(cols) {
+    std::vector<uint8_t> pay;
+    std::vector<oilhip_block_t> desc(blocks.size());
+    for (size_t b = 0; b < blocks.size(); ++b) {
+        const BlockRef& s = blocks[b];
+        desc[b] = oilhip_block_t{pay.size(), pay.size() + s.cb_bytes, s.cb_bytes, s.idx_bytes, s.num_weights, (uint8_t)s.format, {0, 0, 0}};
+        if (s.cb_bytes) pay.insert(pay.end(), s.codebook, s.codebook + s.cb_bytes);
+        if (s.idx_bytes) pay.insert(pay.end(), s.indices, s.indices + s.idx_bytes);
+    }
+    oilhip_weights* h = nullptr;
+    ok(oilhip_weights_create(pay.data(), pay.size(), desc.data(), (uint32_t)desc.size(), rows, cols, &h), "DeviceTensor");
+    handle_ = h;
+}
+
+DeviceTensor::DeviceTensor(const uint8_t* records, uint64_t record_bytes, const uint8_t* formats, uint32_t nblocks,
+                           uint64_t rows, uint64_t cols) : rows_(rows), cols_(cols) {
+    oilhip_weights* h = nullptr;
+    ok(oilhip_weights_create_from_records(records, record_bytes, formats, nblocks, rows, cols, &h), "DeviceTensor");
+    handle_ = h;
+}
+
+DeviceTensor::~DeviceTensor() { oilhip_weights_destroy(static_cast<oilhip_weights*>(handle_)); }
+
+void DeviceTensor::gemm(const float* X, float* Y, int B) const {
+    if (B <= 0) return;
+    Dev<float> x(X, (size_t)B * cols_), y(nullptr, (size_t)B * rows_);
+    ok(oilhip_gemv_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm");
+    y.to_host(Y);
+}
+
+void DeviceTensor::dequantize(float* out) const {
+    Dev<float> o(nullptr, (size_t)rows_ * cols_);
+    ok(oilhip_dequant_f32(static_cast<oilhip_weights*>(handle_), o.get(), nullptr), "dequantize");
+    o.to_host(out);
+}
+
+uint64_t DeviceTensor::payload_bytes() const {
+    uint64_t v = 0;
+    ok(oilhip_weights_info(static_cast<oilhip_weights*>(handle_), nullptr, nullptr, nullptr, &v, nullptr), "info");
+    return v;
+}
+
+bool probe(std::string* name, uint64_t* hbm_bytes, int* compute_units) {
+    char buf[256] = {0};
+    int gfx = 0;
+    if (oilhip_probe(&gfx, hbm_bytes, compute_units, buf, sizeof buf) != OILHIP_OK) return false;
+    if (name) *name = buf;
+    return gfx == 950;
+}
+
+}  // namespace gfx950
+}  // namespace oil
