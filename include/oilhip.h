@@ -71,6 +71,30 @@ int oilhip_quantize_tensor(const uint8_t* fmts, uint32_t nblocks, const float* w
                            uint8_t* payload, uint64_t cap, oilhip_block_t* blocks,
                            uint64_t* total, int threads);
 
+/* --------------------------------------------------------------- format routing
+ * Which wire format each 256-weight block gets (host side, like the reference).
+ * oilhip_score_importance : FormatPlanner::score_importance (fisher = 0: mean |w|*|a| per block,
+ *                           a = aux or 1) / score_importance_fisher (fisher = 1: aux = gradients)
+ *                           (src/format_planner.cpp:12-61)
+ * oilhip_plan_formats     : FormatPlanner::allocate (src/format_planner.cpp:133-315): fmts[b] for a
+ *                           target bits-per-weight; scores may be NULL (blocks keep their order).
+ *                           counts7 = blocks counted as {OIL32, OIL16, OIL8, OIL4, OIL2, SPARK, OIL1}
+ *                           the way the reference's plan counts them (:236-249).
+ * oilhip_mix_allocate     : FormatRegistry::allocate_mix_blocks (src/format_registry.cpp:477-599):
+ *                           adaptive mix under a hard byte budget ceil(effective_bpw*n/8); tier_fmts are
+ *                           the mix's member formats (SPARK_MIX_Q0 = {OIL8_GRP, OIL4_GRP, OIL2_GRP,
+ *                           OIL1_GRP} at 1.925; QUAD_SPARK_Q1 = {OIL32, OIL8_GRP, OIL2_GRP, OIL1_GRP} at
+ *                           2.075).  rows/cols: tensor shape or 0 (one block per row when cols <
+ *                           block_size).  The per-candidate reconstruction errors are measured on the
+ *                           GPU.  With fmts_out == NULL only *nblocks_out is set.  Synchronous. */
+int oilhip_score_importance(const float* w, const float* aux, int64_t n, int block_size, int fisher,
+                            float* scores, int64_t nblocks);
+int oilhip_plan_formats(float target_bpw, const float* scores, int64_t nscores, int num_blocks,
+                        uint8_t* fmts, float* achieved_bpw, int* uses_mix, int* counts7);
+int oilhip_mix_allocate(const uint8_t* tier_fmts, int num_tiers, float effective_bpw, const float* data, int64_t n,
+                        int block_size, int64_t rows, int64_t cols, uint8_t* fmts_out, int64_t* starts_out,
+                        int64_t* lens_out, int64_t cap, int64_t* nblocks_out);
+
 /* ------------------------------------------------------------- device weights
  * A quantized tensor resident in HBM: block payloads byte-identical to the
  * .oil file's, framing stripped into a descriptor table, uploaded once.

@@ -35,6 +35,10 @@ _SIGNATURES = {
                                         vp, C.c_size_t, C.POINTER(C.c_size_t)]),
     "oilhip_quantize_tensor": (C.c_int, [vp, C.c_uint32, vp, C.c_uint64, vp, C.c_uint64, vp,
                                          C.POINTER(C.c_uint64), C.c_int]),
+    "oilhip_score_importance": (C.c_int, [vp, vp, C.c_int64, C.c_int, C.c_int, vp, C.c_int64]),
+    "oilhip_plan_formats": (C.c_int, [C.c_float, vp, C.c_int64, C.c_int, vp, C.POINTER(C.c_float), C.POINTER(C.c_int), vp]),
+    "oilhip_mix_allocate": (C.c_int, [vp, C.c_int, C.c_float, vp, C.c_int64, C.c_int, C.c_int64, C.c_int64, vp, vp, vp,
+                                      C.c_int64, C.POINTER(C.c_int64)]),
     "oilhip_weights_create": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
     "oilhip_weights_create_from_records": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
     "oilhip_weights_destroy": (C.c_int, [vp]),

@@ -61,7 +61,38 @@ gemv_generic_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restr
         y[(size_t)(m0 + t) * rows + row] = (part[t][0] + part[t][1]) + (part[t][2] + part[t][3]);
 }
 
+// Mean squared error of one decoded block against the original weights it encodes:
+// FormatRegistry::measure_mse (src/format_registry.cpp:281-289) over dequantize_block_all,
+// one thread per block, double accumulation in index order with the fused multiply-add the
+// reference build uses, rounded to float at the end.
+__global__ void __launch_bounds__(64)
+block_mse_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__ blocks,
+                 const DecodeTables* __restrict__ T, const float* __restrict__ orig,
+                 const uint64_t* __restrict__ start, float* __restrict__ out, uint32_t nblocks) {
+    const uint32_t b = blockIdx.x * 64 + threadIdx.x;
+    if (b >= nblocks) return;
+    const DevBlock d = blocks[b];
+    const uint8_t* cb = payload + (size_t)d.off16 * 16;
+    const float* o = orig + start[b];
+    double s = 0.0;
+    for (uint32_t i = 0; i < d.nw; ++i) {
+        const double diff = (double)o[i] - (double)decode_weight(d.fmt, cb, d.cb_bytes, cb + d.cb_bytes, d.idx_bytes, d.nw, i, T);
+        s = fma(diff, diff, s);
+    }
+    out[b] = (float)(s / (double)d.nw);
+}
+
 }  // namespace
+
+int launch_block_mse(const oilhip_weights& w, const float* d_orig, const uint64_t* d_start, float* d_out, hipStream_t s) {
+    const DecodeTables* T = nullptr;
+    if (int rc = get_tables(&T)) return rc;
+    if (w.nblocks == 0) return OILHIP_OK;
+    hipLaunchKernelGGL(block_mse_kernel, dim3((w.nblocks + 63) / 64), dim3(64), 0, s, w.d_payload, w.d_blocks, T,
+                       d_orig, d_start, d_out, w.nblocks);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
 
 int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s) {
     const DecodeTables* T = nullptr;

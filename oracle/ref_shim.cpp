@@ -6,12 +6,15 @@
 // linked only into oracle/_ref/liboilref*.so, which is built only where the
 // reference tree is present, and is never part of the product.
 #include "oil/block_codec.h"
+#include "oil/format_planner.h"
+#include "oil/format_registry.h"
 #include "oil/kernel.h"
 #include "oil/kernel_production.h"
 #include "oil/oil_engines.h"
 #include "oil/types.h"
 
 #include <cstdint>
+#include <cstdio>
 #include <cstring>
 #include <vector>
 
@@ -89,6 +92,83 @@ void ref_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx, float
     else if (bits == 4) { oil::engines::OIL4Engine e; c = e.quant_gemm(a, b_idx, M, N, K); }
     else { oil::engines::OIL2Engine e; c = e.quant_gemm(a, b_idx, M, N, K); }
     std::memcpy(C, c.data<float>(), (size_t)(M * N) * 4);
+}
+
+// include/oil/format_planner.h:44-78.  aux = calibration activations (fisher 0, may be null)
+// or gradients (fisher 1).
+void ref_score_importance(const float* w, const float* aux, int64_t n, int block_size, int fisher, float* scores) {
+    oil::Tensor wt({n}), at;
+    std::memcpy(wt.data<float>(), w, (size_t)n * 4);
+    if (aux) { at = oil::Tensor({n}); std::memcpy(at.data<float>(), aux, (size_t)n * 4); }
+    oil::FormatPlanner pl(1.5f);
+    pl.score_importance(wt, at, block_size, fisher ? oil::ImportanceMetric::FISHER_DIAG : oil::ImportanceMetric::MAGNITUDE);
+    std::memcpy(scores, pl.importance_scores().data(), pl.importance_scores().size() * 4);
+}
+
+// FormatPlanner::allocate with scores planted through score_importance on |w| = score, a = null
+// (mean of one weight per block reproduces the score exactly with block_size 1).
+void ref_plan_allocate(float target, const float* scores, int64_t nscores, int nb, uint8_t* fmts,
+                       float* achieved, float* estimated, int* uses_mix, int* counts7) {
+    oil::FormatPlanner pl(target);
+    if (scores && nscores > 0) {
+        oil::Tensor wt({nscores}), at;
+        std::memcpy(wt.data<float>(), scores, (size_t)nscores * 4);
+        pl.score_importance(wt, at, 1, oil::ImportanceMetric::MAGNITUDE);
+    }
+    oil::FormatPlan plan = pl.allocate(nb, 256);
+    for (int i = 0; i < nb; ++i) fmts[i] = (uint8_t)plan.blocks[(size_t)i].assigned_format;
+    *achieved = plan.achieved_bpw;
+    *estimated = oil::FormatPlanner::estimate_bpw(plan);
+    *uses_mix = plan.uses_mix ? 1 : 0;
+    counts7[0] = plan.num_oil32_blocks; counts7[1] = plan.num_oil16_blocks; counts7[2] = plan.num_oil8_blocks;
+    counts7[3] = plan.num_oil4_blocks; counts7[4] = plan.num_oil2_blocks; counts7[5] = plan.num_spark_blocks;
+    counts7[6] = plan.num_oil1_blocks;
+}
+
+// FormatRegistry::allocate_mix_blocks for a registry mix selected by name
+// ("SPARK_MIX_Q0", "QUAD_SPARK_Q1", ...).  Returns the block count, -1 for an unknown name.
+int64_t ref_mix_allocate(const char* mix_name, const float* data, int64_t n, int block_size, int64_t rows, int64_t cols,
+                         uint8_t* fmts, int64_t* starts, int64_t* lens, int64_t cap, float* eff_bpw, uint8_t* tiers4, int* ntiers) {
+    const oil::MixDescriptor* m = nullptr;
+    for (const auto& x : oil::FormatRegistry::get_all_twi_mixes()) if (x.name == mix_name) m = &x;
+    for (const auto& x : oil::FormatRegistry::get_all_four_mixes()) if (x.name == mix_name) m = &x;
+    if (!m) return -1;
+    if (eff_bpw) *eff_bpw = m->effective_bpw;
+    if (ntiers) *ntiers = m->num_tiers;
+    if (tiers4) {
+        const oil::RegFormat t[4] = {m->tier1_fmt, m->tier2_fmt, m->tier3_fmt, m->tier4_fmt};
+        for (int i = 0; i < 4; ++i) tiers4[i] = (uint8_t)oil::regformat_to_format(t[i]);
+    }
+    std::vector<int64_t> shape = {rows, cols};
+    auto plan = oil::FormatRegistry::allocate_mix_blocks(*m, data, n, block_size, rows > 0 ? &shape : nullptr);
+    const int64_t nb = (int64_t)plan.formats.size();
+    for (int64_t b = 0; b < nb && b < cap; ++b) {
+        fmts[b] = (uint8_t)plan.formats[(size_t)b];
+        starts[b] = plan.block_starts[(size_t)b];
+        lens[b] = plan.block_lens[(size_t)b];
+    }
+    return nb;
+}
+
+// registry tables, for checking the product's copies: kind 0 singles, 1 two-tier mixes, 2 four-tier mixes
+int ref_registry_row(int kind, int i, char* name, int cap, float* bpw, uint8_t* tiers4, float* ratios4, int* ntiers) {
+    if (kind == 0) {
+        const auto& v = oil::FormatRegistry::get_all_singles();
+        if (i >= (int)v.size()) return 0;
+        std::snprintf(name, (size_t)cap, "%s", v[(size_t)i].name.c_str());
+        *bpw = v[(size_t)i].bpw; *ntiers = 1;
+        tiers4[0] = (uint8_t)oil::regformat_to_format(v[(size_t)i].id);
+        return 1;
+    }
+    const auto& v = kind == 1 ? oil::FormatRegistry::get_all_twi_mixes() : oil::FormatRegistry::get_all_four_mixes();
+    if (i >= (int)v.size()) return 0;
+    const auto& m = v[(size_t)i];
+    std::snprintf(name, (size_t)cap, "%s", m.name.c_str());
+    *bpw = m.effective_bpw; *ntiers = m.num_tiers;
+    const oil::RegFormat t[4] = {m.tier1_fmt, m.tier2_fmt, m.tier3_fmt, m.tier4_fmt};
+    const float r[4] = {m.tier1_ratio, m.tier2_ratio, m.tier3_ratio, m.tier4_ratio};
+    for (int k = 0; k < 4; ++k) { tiers4[k] = (uint8_t)oil::regformat_to_format(t[k]); ratios4[k] = r[k]; }
+    return 1;
 }
 
 }  // extern "C"

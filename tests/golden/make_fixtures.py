@@ -176,7 +176,124 @@ def make_flat():
     print("flat.npz written")
 
 
+PLAN_TARGETS = [0.5, 1.0, 1.2, 1.5, 1.7, 1.925, 1.95, 2.0, 2.06, 2.075, 2.1, 2.2, 2.3, 2.5, 2.6, 2.75, 2.92, 3.0, 3.5,
+                4.0, 4.12, 4.2, 4.3, 4.5, 5.0, 5.84, 6.0, 7.0, 7.675, 8.0, 8.24, 8.4, 8.5, 10, 12, 16, 20, 24, 32, 40]
+PLAN_BLOCKS = [0, 1, 2, 3, 7, 10, 33, 100, 101, 257, 1000, 3906]
+
+
+def plan_scores(kind, nb, rng):
+    """Importance scores of a planner case: none, distinct, heavy ties, fewer scores than blocks."""
+    if kind == 0:
+        return np.zeros(0, np.float32)
+    if kind == 1:
+        return np.abs(rng.standard_normal(nb)).astype(np.float32)
+    if kind == 2:
+        return rng.integers(0, 4, nb).astype(np.float32)
+    return np.abs(rng.standard_normal(max(nb // 2, 1))).astype(np.float32)
+
+
+def mix_tensor(seed, n):
+    """Weights whose blocks differ in scale and outliers, so that every tier of a mix gets used."""
+    rng = np.random.default_rng(seed)
+    w = rng.standard_normal(n).astype(np.float32) * np.float32(0.02)
+    nb = (n + 255) // 256
+    for b in range(nb):
+        w[b * 256:(b + 1) * 256] *= np.float32(2.0 ** rng.integers(-3, 4))
+        if rng.random() < 0.3:
+            k = rng.integers(0, min(256, n - b * 256), 3)
+            w[b * 256 + k] *= np.float32(25.0)
+    return w
+
+
+MIX_CASES = [("SPARK_MIX_Q0", 1, 64 * 256, 256, 0, 0), ("QUAD_SPARK_Q1", 2, 64 * 256, 256, 0, 0),
+             ("SPARK_MIX_Q0", 3, 40 * 256 + 77, 256, 0, 0), ("QUAD_SPARK_Q1", 4, 96 * 100, 256, 96, 100),
+             ("OIL8+OIL2_10_90", 5, 48 * 256, 256, 48, 256), ("QUAD_OIL2_OIL4_OIL8_OIL16", 6, 32 * 256, 256, 0, 0),
+             ("SPARK_MIX_Q0", 7, 30 * 128, 128, 0, 0)]
+
+
+def make_planner():
+    """FormatPlanner::allocate / score_importance / FormatRegistry::allocate_mix_blocks and the
+    registry tables, as the compiled reference (AVX2+FMA build) answers."""
+    R = O.ref(True)
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    R.ref_mix_allocate.restype = C.c_int64
+    i64p, i32p = C.POINTER(C.c_int64), C.POINTER(C.c_int)
+    out = {}
+    # registry tables
+    names, kinds, bpws, tiers, ratios, ntiers = [], [], [], [], [], []
+    for kind in (0, 1, 2):
+        i = 0
+        while True:
+            nm = C.create_string_buffer(64)
+            bpw, nt = C.c_float(), C.c_int()
+            t, r = np.zeros(4, np.uint8), np.zeros(4, np.float32)
+            if not R.ref_registry_row(kind, i, nm, 64, C.byref(bpw), p(t, u8p), p(r, f32p), C.byref(nt)):
+                break
+            names.append(nm.value.decode()); kinds.append(kind); bpws.append(bpw.value)
+            tiers.append(t); ratios.append(r); ntiers.append(nt.value)
+            i += 1
+    out["reg_name"] = np.array(names)
+    out["reg_kind"] = np.array(kinds, np.int32)
+    out["reg_bpw"] = np.array(bpws, np.float32)
+    out["reg_tiers"] = np.stack(tiers)
+    out["reg_ratios"] = np.stack(ratios)
+    out["reg_ntiers"] = np.array(ntiers, np.int32)
+    # planner cases: scores are regenerated from (seed, kind, nb) by the test
+    rng = np.random.default_rng(5)
+    meta, fm, ach, est = [], [], [], []
+    for ti, target in enumerate(PLAN_TARGETS):
+        for nb in PLAN_BLOCKS:
+            for kind in range(4):
+                s = plan_scores(kind, nb, rng)
+                f = np.zeros(max(nb, 1), np.uint8)
+                a, e, u = C.c_float(), C.c_float(), C.c_int()
+                c7 = np.zeros(7, np.int32)
+                R.ref_plan_allocate(C.c_float(target), p(s, f32p) if s.size else None, C.c_int64(s.size), C.c_int(nb),
+                                    p(f, u8p), C.byref(a), C.byref(e), C.byref(u), p(c7, i32p))
+                meta.append([ti, nb, kind, u.value] + list(c7))
+                fm.append(f[:nb].copy()); ach.append(a.value); est.append(e.value)
+    out["plan_meta"] = np.array(meta, np.int32)
+    out["plan_fmts"] = np.concatenate(fm)
+    out["plan_achieved"] = np.array(ach, np.float32)
+    out["plan_estimated"] = np.array(est, np.float32)
+    # importance scores
+    rng = np.random.default_rng(6)
+    sm, sw, sa, ss = [], [], [], []
+    for n in (1, 255, 256, 257, 1000, 4096):
+        for bs in (256, 64, 100):
+            w = rng.standard_normal(n).astype(np.float32)
+            a = rng.standard_normal(n).astype(np.float32)
+            nb = (n + bs - 1) // bs
+            for mode in (0, 1, 2):      # magnitude without activations, with activations, fisher
+                sc = np.zeros(nb, np.float32)
+                R.ref_score_importance(p(w, f32p), p(a, f32p) if mode else None, C.c_int64(n), C.c_int(bs),
+                                       C.c_int(1 if mode == 2 else 0), p(sc, f32p))
+                sm.append([n, bs, mode]); ss.append(sc)
+            sw.append(w); sa.append(a)
+    out["score_meta"] = np.array(sm, np.int32)
+    out["score_w"] = np.concatenate(sw)
+    out["score_a"] = np.concatenate(sa)
+    out["score_out"] = np.concatenate(ss)
+    # adaptive mix allocation (inputs regenerated by mix_tensor(seed, n) in the test)
+    mm, mf, ms, ml = [], [], [], []
+    for name, seed, n, bs, rows, cols in MIX_CASES:
+        w = mix_tensor(seed, n)
+        cap = n
+        f, st, ln = np.zeros(cap, np.uint8), np.zeros(cap, np.int64), np.zeros(cap, np.int64)
+        nb = R.ref_mix_allocate(name.encode(), p(w, f32p), C.c_int64(n), C.c_int(bs), C.c_int64(rows), C.c_int64(cols),
+                                p(f, u8p), p(st, i64p), p(ln, i64p), C.c_int64(cap), None, None, None)
+        assert nb > 0
+        mm.append(nb); mf.append(f[:nb].copy()); ms.append(st[:nb].copy()); ml.append(ln[:nb].copy())
+        print(name, "tiers used:", np.unique(f[:nb], return_counts=True))
+    out["mix_nb"] = np.array(mm, np.int64)
+    out["mix_fmts"] = np.concatenate(mf)
+    out["mix_starts"] = np.concatenate(ms)
+    out["mix_lens"] = np.concatenate(ml)
+    np.savez_compressed(os.path.join(HERE, "planner.npz"), **out)
+    print("planner.npz written")
+
+
 if __name__ == "__main__":
-    make_codec()
-    make_gemv()
-    make_flat()
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner"]
+    for name in which:
+        {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner}[name]()
