@@ -124,6 +124,36 @@ int oilhip_weights_destroy(oilhip_weights* w);
 int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols,
                         uint32_t* nblocks, uint64_t* payload_bytes, int* uniform_fmt);
 
+/* ------------------------------------------------------------- .oil container
+ * OILReader (include/oil/oil_format.h:66-108, src/oil_format.cpp:289-527) and OILWriter
+ * (src/oil_format.cpp:189-283).  A file handle maps the file and indexes its block records once.
+ * oilhip_file_open / _open_memory : OILReader ctor (memory: the bytes are copied); a bad magic or a file cut
+ *                                   inside its tables is an error (the reference leaves valid() false)
+ * oilhip_file_info                : header() fields, num_blocks(), tensor count
+ * oilhip_file_config              : read_config()
+ * oilhip_file_tensor / _find_tensor : tensor_names() / tensor_blocks(); num_weights = sum of the records' nw
+ * oilhip_file_block               : read_block() / block_ptr() / format_entry(): pointers into the mapped file,
+ *                                   valid until oilhip_file_close; format ids above 14 read as OIL32 (:405-408)
+ * oilhip_file_upload_tensor       : a tensor's records straight into a device tensor (rows = cols = 0: 1 x numel)
+ * oilhip_file_write               : OILWriter's header -> format table -> tensor table -> blocks sequence for
+ *                                   tensors laid back to back (tensor i owns the next tensor_blocks[i] blocks) */
+typedef struct oilhip_file oilhip_file;
+int oilhip_file_open(const char* path, oilhip_file** out);
+int oilhip_file_open_memory(const uint8_t* bytes, uint64_t n, oilhip_file** out);
+int oilhip_file_close(oilhip_file* f);
+int oilhip_file_info(const oilhip_file* f, uint32_t* version, uint32_t* flags, uint32_t* config_size,
+                     uint32_t* num_blocks, uint32_t* num_tensors);
+int oilhip_file_config(const oilhip_file* f, uint8_t* out, uint32_t cap);
+int oilhip_file_tensor(const oilhip_file* f, uint32_t i, char* name, size_t name_cap, uint32_t* start,
+                       uint32_t* count, uint64_t* num_weights);
+int oilhip_file_find_tensor(const oilhip_file* f, const char* name, uint32_t* index);
+int oilhip_file_block(const oilhip_file* f, uint32_t id, uint8_t* fmt, uint32_t* nw, const uint8_t** cb,
+                      uint32_t* cb_bytes, const uint8_t** idx, uint32_t* idx_bytes);
+int oilhip_file_upload_tensor(const oilhip_file* f, uint32_t tensor, uint64_t rows, uint64_t cols, oilhip_weights** out);
+int oilhip_file_write(const char* path, uint32_t version, uint32_t flags, const uint8_t* config, uint32_t config_size,
+                      uint32_t ntensors, const char* const* names, const uint32_t* tensor_blocks,
+                      const uint8_t* payload, const oilhip_block_t* blocks, uint32_t nblocks);
+
 /* dequantize_block_all over every block, back to back (include/oil/block_codec.h:60-63,
  * OILReader::read_tensor src/oil_format.cpp:464-477).  d_out holds rows*cols
  * floats.  Bit-exact with the reference decode. */

@@ -44,6 +44,19 @@ _SIGNATURES = {
     "oilhip_weights_destroy": (C.c_int, [vp]),
     "oilhip_weights_info": (C.c_int, [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint32),
                                       C.POINTER(C.c_uint64), C.POINTER(C.c_int)]),
+    "oilhip_file_open": (C.c_int, [C.c_char_p, C.POINTER(vp)]),
+    "oilhip_file_open_memory": (C.c_int, [vp, C.c_uint64, C.POINTER(vp)]),
+    "oilhip_file_close": (C.c_int, [vp]),
+    "oilhip_file_info": (C.c_int, [vp] + [C.POINTER(C.c_uint32)] * 5),
+    "oilhip_file_config": (C.c_int, [vp, vp, C.c_uint32]),
+    "oilhip_file_tensor": (C.c_int, [vp, C.c_uint32, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32),
+                                     C.POINTER(C.c_uint64)]),
+    "oilhip_file_find_tensor": (C.c_int, [vp, C.c_char_p, C.POINTER(C.c_uint32)]),
+    "oilhip_file_block": (C.c_int, [vp, C.c_uint32, C.POINTER(C.c_uint8), C.POINTER(C.c_uint32), C.POINTER(u8p),
+                                    C.POINTER(C.c_uint32), C.POINTER(u8p), C.POINTER(C.c_uint32)]),
+    "oilhip_file_upload_tensor": (C.c_int, [vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
+    "oilhip_file_write": (C.c_int, [C.c_char_p, C.c_uint32, C.c_uint32, vp, C.c_uint32, C.c_uint32, C.POINTER(C.c_char_p), vp,
+                                    vp, vp, C.c_uint32]),
     "oilhip_dequant_f32": (C.c_int, [vp, vp, vp]),
     "oilhip_gemv_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_gemv_f32_general": (C.c_int, [vp, vp, vp, C.c_int, vp]),

@@ -8,6 +8,7 @@
 #include "oil/block_codec.h"
 #include "oil/format_planner.h"
 #include "oil/format_registry.h"
+#include "oil/oil_format.h"
 #include "oil/kernel.h"
 #include "oil/kernel_production.h"
 #include "oil/oil_engines.h"
@@ -16,6 +17,8 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <algorithm>
+#include <string>
 #include <vector>
 
 namespace oil {
@@ -169,6 +172,66 @@ int ref_registry_row(int kind, int i, char* name, int cap, float* bpw, uint8_t* 
     const float r[4] = {m.tier1_ratio, m.tier2_ratio, m.tier3_ratio, m.tier4_ratio};
     for (int k = 0; k < 4; ++k) { tiers4[k] = (uint8_t)oil::regformat_to_format(t[k]); ratios4[k] = r[k]; }
     return 1;
+}
+
+// OILWriter in the reference's own call order (tests/test_spark_mix.cpp:344-384): header, format
+// table, tensor table, blocks.  Block b of the file encodes data[starts[b] .. +lens[b]) as fmts[b].
+int ref_oil_write(const char* path, uint32_t version, uint32_t flags, const uint8_t* config, uint32_t config_size,
+                  uint32_t ntensors, const char* const* names, const uint32_t* tensor_blocks, const float* data,
+                  const uint8_t* fmts, const int64_t* starts, const int64_t* lens, uint32_t nblocks) {
+    oil::OILWriter writer(path);
+    oil::OILHeader hdr;
+    std::memcpy(hdr.magic, "OIL1", 4);
+    hdr.version = version; hdr.flags = flags; hdr.config_size = config_size;
+    writer.write_header(hdr, config);
+    std::vector<oil::FormatBlockEntry> ft;
+    std::vector<oil::TensorEntry> te;
+    std::vector<std::string> nm;
+    std::vector<oil::BlockData> blocks;
+    uint32_t id = 0;
+    for (uint32_t t = 0; t < ntensors; ++t) {
+        nm.push_back(names[t]);
+        oil::TensorEntry e;
+        e.name_len = (uint16_t)nm.back().size(); e.block_start = id; e.num_blocks = tensor_blocks[t];
+        te.push_back(e);
+        for (uint32_t b = 0; b < tensor_blocks[t]; ++b, ++id) {
+            oil::BlockData blk;
+            blk.format = (oil::Format)fmts[id];
+            blk.num_weights = (uint32_t)lens[id];
+            if (!oil::quantize_block_all(blk.format, data + starts[id], (int)lens[id], blk.indices, blk.codebook)) return -1;
+            oil::FormatBlockEntry fe;
+            fe.block_id = id; fe.format = fmts[id]; fe.cb_bytes = (uint32_t)blk.codebook.size();
+            ft.push_back(fe);
+            blocks.push_back(std::move(blk));
+        }
+    }
+    if (id != nblocks) return -2;
+    writer.write_format_table(ft);
+    writer.write_tensor_table(te, nm);
+    for (auto& b : blocks) writer.write_block(b);
+    writer.close();
+    return 0;
+}
+
+// OILReader::read_tensor; returns numel (or -1 when the file does not open / has no such tensor).
+int64_t ref_oil_read_tensor(const char* path, const char* name, float* out, int64_t cap) {
+    oil::OILReader r(path);
+    if (!r.valid()) return -1;
+    oil::Tensor t = r.read_tensor(name);
+    const int64_t n = t.numel();
+    if (n <= 0) return -1;
+    if (out) std::memcpy(out, t.data<float>(), (size_t)std::min(n, cap) * 4);
+    return n;
+}
+
+// OILReader metadata: block count, tensor count, and tensor_blocks() of one name.
+int ref_oil_meta(const char* path, const char* name, uint32_t* nblocks, uint32_t* ntensors, uint32_t* start, uint32_t* count) {
+    oil::OILReader r(path);
+    if (!r.valid()) return -1;
+    *nblocks = (uint32_t)r.num_blocks();
+    *ntensors = (uint32_t)r.tensor_names().size();
+    if (name && !r.tensor_blocks(name, *start, *count)) return -2;
+    return 0;
 }
 
 }  // extern "C"

@@ -293,7 +293,62 @@ def make_planner():
     print("planner.npz written")
 
 
+CONTAINER_CONFIG = b'{"dim": 256, "note": "fixture"}'
+CONTAINER_VERSION = (1 << 22) | (2 << 12) | 3
+CONTAINER_FLAGS = 5
+
+
+def container_tensors():
+    """[(name, data, fmts, starts, lens)]: every wire format, a ragged tail, one-block-per-row blocks."""
+    rng = np.random.default_rng(77)
+    out = []
+    w = (rng.standard_normal(32 * 256) * 0.3).astype(np.float32)
+    out.append(("layers.0.attention.q_proj.weight", w, np.arange(32, dtype=np.uint8) % 15,
+                np.arange(32, dtype=np.int64) * 256, np.full(32, 256, np.int64)))
+    w = (rng.standard_normal(1000) * 0.05 + 1.0).astype(np.float32)
+    out.append(("norm.weight", w, np.array([6, 5, 11, 4], np.uint8), np.arange(4, dtype=np.int64) * 256,
+                np.array([256, 256, 256, 232], np.int64)))
+    w = (rng.standard_normal(64 * 100) * 0.1).astype(np.float32)
+    out.append(("tok_embeddings.weight", w, (np.arange(64, dtype=np.uint8) * 7) % 15,
+                np.arange(64, dtype=np.int64) * 100, np.full(64, 100, np.int64)))
+    return out
+
+
+def make_container():
+    """tests/golden/mixed.oil written by the reference's OILWriter, and what its OILReader reads back."""
+    R = O.ref(True)
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    R.ref_oil_read_tensor.restype = C.c_int64
+    i64p = C.POINTER(C.c_int64)
+    ts = container_tensors()
+    names = (C.c_char_p * len(ts))(*[t[0].encode() for t in ts])
+    counts = np.array([len(t[2]) for t in ts], np.uint32)
+    data = np.concatenate([t[1] for t in ts])
+    fmts = np.concatenate([t[2] for t in ts])
+    base = np.cumsum([0] + [t[1].size for t in ts])[:-1]
+    starts = np.concatenate([t[3] + b for t, b in zip(ts, base)])
+    lens = np.concatenate([t[4] for t in ts])
+    path = os.path.join(HERE, "mixed.oil")
+    cfg = np.frombuffer(CONTAINER_CONFIG, np.uint8)
+    rc = R.ref_oil_write(path.encode(), C.c_uint32(CONTAINER_VERSION), C.c_uint32(CONTAINER_FLAGS), p(cfg, u8p),
+                         C.c_uint32(cfg.size), C.c_uint32(len(ts)), names, counts.ctypes.data_as(C.POINTER(C.c_uint32)),
+                         p(data, f32p), p(fmts, u8p), p(starts, i64p), p(lens, i64p), C.c_uint32(fmts.size))
+    assert rc == 0, rc
+    out = {}
+    for k, t in enumerate(ts):
+        dec = np.zeros(t[1].size, np.float32)
+        n = R.ref_oil_read_tensor(path.encode(), t[0].encode(), p(dec, f32p), C.c_int64(dec.size))
+        assert n == dec.size, (t[0], n)
+        out[f"decoded{k}"] = dec.view(np.uint32)
+    nb, nt, st, cnt = C.c_uint32(), C.c_uint32(), C.c_uint32(), C.c_uint32()
+    assert R.ref_oil_meta(path.encode(), ts[2][0].encode(), C.byref(nb), C.byref(nt), C.byref(st), C.byref(cnt)) == 0
+    out["meta"] = np.array([nb.value, nt.value, st.value, cnt.value], np.int64)
+    np.savez_compressed(os.path.join(HERE, "container.npz"), **out)
+    print("mixed.oil", os.path.getsize(path), "bytes; container.npz written", out["meta"])
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner"]
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container"]
     for name in which:
-        {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner}[name]()
+        {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner,
+         "container": make_container}[name]()
