@@ -196,6 +196,27 @@ int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb256, float scale,
 int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b_idx, const float* d_cb,
                              float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* ------------------------------------------------------------ mixture of experts
+ * oilhip_moe_route   : moe::softmax_with_topk (include/oil/moe_variants.h:693, src/moe_variants.cpp:97-134).
+ *                      Host arrays: logits/probs [T][E], indices (int64) and weights [T][k]; weights are the
+ *                      raw probabilities (no renormalisation), ties as std::partial_sort leaves them.
+ * oilhip_moe_forward : moe::moe_dispatch_batched (moe_variants.h:701-706, src/moe_variants.cpp:767-827) with
+ *                      ExpertFFN::forward (:77-91, SiLU): d_out[T][D] = sum over a token's experts of
+ *                      w * down_e(silu(gate_e x) * up_e x), experts visited in ascending order, tokens of an
+ *                      expert in ascending order.  gate[e], up[e]: F x D tensors, down[e]: D x F (Y = X W^T,
+ *                      no bias, any wire format with full blocks; uniform OIL4 runs the fast kernel).
+ *                      indices/weights are host arrays [T][K]; entries outside [0,E) are ignored, pairs with
+ *                      weight <= 0 are counted in *dropped.  d_workspace: device memory of at least
+ *                      oilhip_moe_workspace_bytes(T, K, D, F) bytes.  Returns after the token lists are on the
+ *                      device; with z_loss != NULL it also waits for the result (sum of squared contributions).
+ *                      Calls sharing a workspace must be ordered by the caller. */
+int oilhip_moe_route(const float* logits, int64_t T, int64_t E, int64_t k, float* probs, int64_t* indices, float* weights);
+size_t oilhip_moe_workspace_bytes(int64_t T, int64_t K, int64_t D, int64_t F);
+int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* const* up,
+                       const oilhip_weights* const* down, int E, const float* d_x, const int64_t* indices,
+                       const float* weights, int64_t T, int64_t K, float* d_out, void* d_workspace,
+                       size_t workspace_bytes, float* z_loss, int64_t* dropped, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -26,6 +26,7 @@
 #include <cstdlib>
 
 #include "common.h"
+#include "oil4_lds.h"
 
 #ifndef OILHIP_OIL4_PREFETCH
 #define OILHIP_OIL4_PREFETCH 6
@@ -34,78 +35,7 @@
 namespace oilhip {
 namespace {
 
-constexpr int kTabBytes = 256 * 64 * 4;   // [byte value][low|high nibble][32 lane copies] floats
-constexpr int kMaxLds = 160 * 1024;
-
-__device__ __forceinline__ float dpp_quad_xor1(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));   // quad_perm [1,0,3,2]
-}
-__device__ __forceinline__ float dpp_quad_xor2(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));   // quad_perm [2,3,0,1]
-}
-__device__ __forceinline__ float dpp_half_mirror(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));  // row_half_mirror
-}
-__device__ __forceinline__ float dpp_row_ror8(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, true));  // row_ror:8
-}
-__device__ __forceinline__ float dpp_row_mirror(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));  // row_mirror
-}
-// lane 15 of rows 0 and 2 into every lane of rows 1 and 3 (other rows receive 0)
-__device__ __forceinline__ float dpp_row_bcast15(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));
-}
-// lane 31 into every lane of rows 2 and 3 (other rows receive 0)
-__device__ __forceinline__ float dpp_row_bcast31(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));
-}
-// value of the first lane of each group of 8 lanes, in all 8 lanes
-__device__ __forceinline__ uint32_t dpp_bcast8(uint32_t v) {
-    const int q = __builtin_amdgcn_update_dpp(0, (int)v, 0x00, 0xF, 0xF, true);      // quad_perm [0,0,0,0]
-    return (uint32_t)__builtin_amdgcn_update_dpp(q, q, 0x114, 0xF, 0xA, false);     // row_shr:4 into quads 1 and 3
-}
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-
-constexpr uint32_t kOobOffset = 0xFFFFFF00u;   // beyond any buffer range: the load returns zeros, no fetch
-
-// The two level values of one packed byte: (low nibble, high nibble).
-struct LevelPair { float lo, hi; };
-
-// kOIL4Levels (src/block_codec.cpp:18-23) selected by compares on literals: no memory access.
-__device__ __forceinline__ float level_literal(uint32_t i) {
-    const float mag = (i == 7 || i == 8) ? 0.1260f : (i == 6 || i == 9) ? 0.3976f : (i == 5 || i == 10) ? 0.6508f
-                    : (i == 4 || i == 11) ? 0.9275f : (i == 3 || i == 12) ? 1.2392f : (i == 2 || i == 13) ? 1.5995f
-                    : (i == 1 || i == 14) ? 2.0522f : 2.7178f;
-    return i < 8 ? -mag : mag;
-}
-
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef __attribute__((address_space(3))) const f32x2 lds_cfloat2;
-typedef __attribute__((address_space(3))) const float lds_cfloat;
-
-// Pair table, 64 KB at LDS offset 0: entry of byte value v and lane copy c at
-// byte v*256 + c*8 = (level[v & 15], level[v >> 4]).  32 lane-private copies:
-// lanes of a half-wave never meet in a bank at different addresses.
-template <int J>
-__device__ __forceinline__ LevelPair lookup(uint32_t word, uint32_t lanebase) {
-    // byte J of the dword -> address bits 8..15, this lane's copy -> bits 0..7
-    const uint32_t addr = __builtin_amdgcn_perm(word, lanebase, 0x0C0C0000u | ((4u + J) << 8));
-    const f32x2 t = *(lds_cfloat2*)(uintptr_t)addr;
-    return LevelPair{t.x, t.y};
-}
-
-__device__ __forceinline__ void lookup_load(const u32x4& w, uint32_t lanebase, LevelPair (&t)[16]) {
-    const uint32_t wd[4] = {w.x, w.y, w.z, w.w};
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        t[d * 4 + 0] = lookup<0>(wd[d], lanebase);
-        t[d * 4 + 1] = lookup<1>(wd[d], lanebase);
-        t[d * 4 + 2] = lookup<2>(wd[d], lanebase);
-        t[d * 4 + 3] = lookup<3>(wd[d], lanebase);
-    }
-}
+using namespace oil4;
 
 constexpr int kPrefetch = OILHIP_OIL4_PREFETCH;   // wave-loads in flight per wavefront
 constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 32 so that neighbouring blocks start 32 banks apart

@@ -1,0 +1,201 @@
+// moe.hip -- mixture-of-experts step over quantized experts: routing on the host, batched expert
+// feed-forward on the device.  Counterparts: softmax_with_topk (src/moe_variants.cpp:97-134),
+// moe_dispatch_batched (:767-827) and ExpertFFN::forward with SiLU (:77-91), with each expert's
+// three projections held as .oil tensors (Y = X W^T, no bias) instead of dense FP32 Linear layers.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <utility>
+#include <vector>
+
+#include "common.h"
+
+namespace oilhip {
+namespace {
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0.0f;
+}
+
+// h = silu(g) * u, silu(v) = v / (1 + exp(-v))  (src/math.cpp:117-126)
+__global__ void __launch_bounds__(256) swiglu_kernel(float* __restrict__ g, const float* __restrict__ u, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
+        const float v = g[i];
+        g[i] = (v / (1.0f + expf(-v))) * u[i];
+    }
+}
+
+// x rows picked by tok[] into a dense [nt][D] batch (experts in formats without a gathering kernel)
+__global__ void __launch_bounds__(256) gather_rows_kernel(const float* __restrict__ x, const int* __restrict__ tok,
+                                                          float* __restrict__ out, uint32_t D) {
+    const float* src = x + (size_t)tok[blockIdx.x] * D;
+    float* dst = out + (size_t)blockIdx.x * D;
+    for (uint32_t d = threadIdx.x; d < D; d += 256) dst[d] = src[d];
+}
+
+// out[tok[i]][d] += wgt[i] * o[i][d] in list order (one thread per column walks the expert's rows, so a
+// token listed twice is added twice, in order); the squared contributions feed the z-loss sum.
+__global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ o, const int* __restrict__ tok,
+                                                      const float* __restrict__ wgt, int nt, uint32_t D,
+                                                      float* __restrict__ out, double* __restrict__ zacc) {
+    __shared__ double part[4];
+    const uint32_t d = blockIdx.x * 256 + threadIdx.x;
+    double z = 0.0;
+    if (d < D) {
+        for (int i = 0; i < nt; ++i) {
+            const float w = wgt[i];
+            if (!(w > 0.0f)) continue;
+            const float v = w * o[(size_t)i * D + d];
+            out[(size_t)tok[i] * D + d] += v;
+            z += (double)v * (double)v;
+        }
+    }
+    for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = z;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(zacc, (part[0] + part[1]) + (part[2] + part[3]));
+}
+
+size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+struct Workspace {
+    int* tok; float* wgt; float* g; float* u; float* o; float* xg; double* z;
+    size_t bytes;
+};
+
+Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
+    Workspace w{};
+    uint8_t* p = (uint8_t*)base;
+    size_t off = 0;
+    auto take = [&](size_t n) { uint8_t* r = p ? p + off : nullptr; off += align256(n); return r; };
+    w.z = (double*)take(8);
+    w.tok = (int*)take((size_t)pairs * 4);
+    w.wgt = (float*)take((size_t)pairs * 4);
+    w.g = (float*)take((size_t)pairs * F * 4);
+    w.u = (float*)take((size_t)pairs * F * 4);
+    w.o = (float*)take((size_t)pairs * D * 4);
+    w.xg = (float*)take((size_t)pairs * D * 4);
+    w.bytes = off;
+    return w;
+}
+
+// one projection of an expert batch: Y[nt][rows] from rows tok[] of X (or X itself when tok is null)
+int expert_gemv(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int nt, uint32_t xrows,
+                float* d_gather, hipStream_t s) {
+    if (w.uniform_fmt == OILHIP_OIL4 && w.uniform_stride == 128) {
+        const int rc = launch_gemv_oil4_multi(w, d_x, d_tok, d_y, nt, (uint32_t)w.cols, (uint32_t)w.rows, xrows, s);
+        if (rc <= 0) return rc;
+    }
+    const float* xin = d_x;
+    if (d_tok) {
+        hipLaunchKernelGGL(gather_rows_kernel, dim3((uint32_t)nt), dim3(256), 0, s, d_x, d_tok, d_gather, (uint32_t)w.cols);
+        OILHIP_HIP(hipGetLastError());
+        xin = d_gather;
+    }
+    return launch_gemv_generic(w, xin, d_y, nt, s);
+}
+
+}  // namespace
+}  // namespace oilhip
+
+using namespace oilhip;
+
+extern "C" {
+
+int oilhip_moe_route(const float* logits, int64_t T, int64_t E, int64_t k, float* probs, int64_t* indices, float* weights) {
+    if (!logits || !probs || !indices || !weights || T < 0 || E <= 0 || k <= 0 || k > E)
+        return fail(OILHIP_E_ARG, "moe_route: bad arguments");
+    std::vector<std::pair<float, int64_t>> scored;
+    for (int64_t t = 0; t < T; ++t) {
+        const float* l = logits + t * E;
+        float* p = probs + t * E;
+        float maxv = l[0];
+        for (int64_t e = 1; e < E; ++e) if (l[e] > maxv) maxv = l[e];
+        float sum = 0.0f;
+        for (int64_t e = 0; e < E; ++e) { const float v = std::exp(l[e] - maxv); p[e] = v; sum += v; }
+        const float inv = 1.0f / sum;
+        for (int64_t e = 0; e < E; ++e) p[e] *= inv;
+        scored.clear();
+        for (int64_t e = 0; e < E; ++e) scored.push_back({p[e], e});
+        std::partial_sort(scored.begin(), scored.begin() + k, scored.end(),
+                          [](const auto& a, const auto& b) { return a.first > b.first; });
+        for (int64_t j = 0; j < k; ++j) { indices[t * k + j] = scored[(size_t)j].second; weights[t * k + j] = scored[(size_t)j].first; }
+    }
+    return OILHIP_OK;
+}
+
+size_t oilhip_moe_workspace_bytes(int64_t T, int64_t K, int64_t D, int64_t F) {
+    if (T <= 0 || K <= 0 || D <= 0 || F <= 0) return 0;
+    return carve(nullptr, T * K, D, F).bytes;
+}
+
+int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* const* up,
+                       const oilhip_weights* const* down, int E, const float* d_x, const int64_t* indices,
+                       const float* weights, int64_t T, int64_t K, float* d_out, void* d_workspace,
+                       size_t workspace_bytes, float* z_loss, int64_t* dropped, void* stream) {
+    if (!gate || !up || !down || E <= 0 || !d_x || !indices || !weights || T <= 0 || K <= 0 || !d_out || !d_workspace)
+        return fail(OILHIP_E_ARG, "moe_forward: bad arguments");
+    const int64_t D = (int64_t)gate[0]->cols, F = (int64_t)gate[0]->rows;
+    for (int e = 0; e < E; ++e) {
+        if (!gate[e] || !up[e] || !down[e]) return fail(OILHIP_E_ARG, "moe_forward: null expert tensor");
+        if ((int64_t)gate[e]->cols != D || (int64_t)gate[e]->rows != F || (int64_t)up[e]->cols != D || (int64_t)up[e]->rows != F ||
+            (int64_t)down[e]->cols != F || (int64_t)down[e]->rows != D)
+            return fail(OILHIP_E_ARG, "moe_forward: expert " + std::to_string(e) + " has mismatched shapes");
+        for (const oilhip_weights* w : {gate[e], up[e], down[e]})
+            if (!w->all_full || (w->cols & 255)) return fail(OILHIP_E_ARG, "moe_forward: expert tensors need full 256-weight blocks");
+    }
+    if (T * K > 0x7FFFFFFF || T > 0x7FFFFFFF) return fail(OILHIP_E_ARG, "moe_forward: too many (token, expert) pairs");
+    const Workspace ws = carve(d_workspace, T * K, D, F);
+    if (workspace_bytes < ws.bytes) return fail(OILHIP_E_ARG, "moe_forward: workspace too small");
+    hipStream_t s = (hipStream_t)stream;
+
+    // tokens per expert in ascending token order, each with the weight of its first matching slot
+    std::vector<int> tok;
+    std::vector<float> wgt;
+    std::vector<int> begin((size_t)E + 1, 0);
+    int64_t drop = 0;
+    for (int e = 0; e < E; ++e) {
+        begin[(size_t)e] = (int)tok.size();
+        for (int64_t t = 0; t < T; ++t)
+            for (int64_t k = 0; k < K; ++k)
+                if (indices[t * K + k] == e) {
+                    float w = 0.0f;
+                    for (int64_t k2 = 0; k2 < K; ++k2) if (indices[t * K + k2] == e) { w = weights[t * K + k2]; break; }
+                    if (!(w > 0.0f)) drop++;
+                    tok.push_back((int)t);
+                    wgt.push_back(w);
+                }
+    }
+    begin[(size_t)E] = (int)tok.size();
+    if (!tok.empty()) {
+        OILHIP_HIP(hipMemcpyAsync(ws.tok, tok.data(), tok.size() * 4, hipMemcpyHostToDevice, s));
+        OILHIP_HIP(hipMemcpyAsync(ws.wgt, wgt.data(), wgt.size() * 4, hipMemcpyHostToDevice, s));
+        OILHIP_HIP(hipStreamSynchronize(s));          // the host vectors go out of scope
+    }
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(256), dim3(256), 0, s, d_out, (size_t)(T * D));
+    hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(256), 0, s, (float*)ws.z, (size_t)2);
+    OILHIP_HIP(hipGetLastError());
+    for (int e = 0; e < E; ++e) {
+        const int b = begin[(size_t)e], nt = begin[(size_t)e + 1] - b;
+        if (nt == 0) continue;
+        if (int rc = expert_gemv(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)T, ws.xg, s)) return rc;
+        if (int rc = expert_gemv(*up[e], d_x, ws.tok + b, ws.u, nt, (uint32_t)T, ws.xg, s)) return rc;
+        const size_t n = (size_t)nt * (size_t)F;
+        hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0, s, ws.g, ws.u, n);
+        OILHIP_HIP(hipGetLastError());
+        if (int rc = expert_gemv(*down[e], ws.g, nullptr, ws.o, nt, (uint32_t)nt, ws.xg, s)) return rc;
+        hipLaunchKernelGGL(combine_kernel, dim3((uint32_t)((D + 255) / 256)), dim3(256), 0, s, ws.o, ws.tok + b, ws.wgt + b, nt,
+                           (uint32_t)D, d_out, ws.z);
+        OILHIP_HIP(hipGetLastError());
+    }
+    if (dropped) *dropped = drop;
+    if (z_loss) {
+        double z = 0.0;
+        OILHIP_HIP(hipMemcpyAsync(&z, ws.z, 8, hipMemcpyDeviceToHost, s));
+        OILHIP_HIP(hipStreamSynchronize(s));
+        *z_loss = (float)z;
+    }
+    return OILHIP_OK;
+}
+
+}  // extern "C"

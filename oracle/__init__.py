@@ -294,3 +294,45 @@ def xorshift_fill(n: int, seed: int) -> np.ndarray:
         state ^= (state << 5) & 0xFFFFFFFF
         out[i] = (f(state & 0xFFFF) / f(65535.0) - f(0.5)) * f(2.0)
     return out
+
+
+# ---------------------------------------------------------------- mixture of experts
+def softmax_topk(logits: np.ndarray, k: int, fn=None):
+    """orc_softmax_topk -> (probs, indices, weights)."""
+    lg = np.ascontiguousarray(logits, np.float32)
+    T, E = lg.shape
+    probs = np.zeros((T, E), np.float32)
+    idx = np.zeros((T, k), np.int64)
+    w = np.zeros((T, k), np.float32)
+    (fn or lib().orc_softmax_topk)(C.c_void_p(lg.ctypes.data), C.c_int64(T), C.c_int64(E), C.c_int64(k),
+                                   C.c_void_p(probs.ctypes.data), C.c_void_p(idx.ctypes.data), C.c_void_p(w.ctypes.data))
+    return probs, idx, w
+
+
+def moe_dispatch(x, gate, up, down, indices, weights, wide: bool = False, fn=None):
+    """orc_moe_dispatch over decoded expert matrices (lists of [F][D], [F][D], [D][F] float32 arrays).
+    -> (out [T][D], z_loss, dropped).  fn: a compiled-reference entry point with the same leading arguments."""
+    x = np.ascontiguousarray(x, np.float32)
+    T, D = x.shape
+    E, F = len(gate), gate[0].shape[0]
+    idx = np.ascontiguousarray(indices, np.int64)
+    w = np.ascontiguousarray(weights, np.float32)
+    K = idx.shape[1]
+    keep = [[np.ascontiguousarray(m, np.float32) for m in lst] for lst in (gate, up, down)]
+    ptrs = [(C.c_void_p * E)(*[m.ctypes.data for m in lst]) for lst in keep]
+    out = np.zeros((T, D), np.float32)
+    z, dr = C.c_float(0), C.c_int64(0)
+    args = [C.c_void_p(x.ctypes.data), ptrs[0], ptrs[1], ptrs[2], C.c_void_p(idx.ctypes.data), C.c_void_p(w.ctypes.data),
+            C.c_int64(T), C.c_int64(K), C.c_int64(E), C.c_int64(D), C.c_int64(F), C.c_void_p(out.ctypes.data),
+            C.byref(z), C.byref(dr)]
+    if fn is None:
+        lib().orc_moe_dispatch(*args, C.c_int(1 if wide else 0))
+    else:
+        fn(*args)
+    return out, z.value, dr.value
+
+
+def ref_moe():
+    """The compiled reference's routing/dispatch library, or None where it has not been built."""
+    path = os.path.join(_HERE, "_ref", "liboilref_moe.so")
+    return C.CDLL(path) if os.path.exists(path) else None

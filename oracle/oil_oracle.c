@@ -965,3 +965,85 @@ void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
     }
     free(acc);
 }
+
+/* ------------------------------------------------------------------ mixture of experts */
+void orc_softmax_topk(const float* logits, int64_t T, int64_t E, int64_t k,
+                      float* probs, int64_t* indices, float* weights) {
+    mag_t* sc = (mag_t*)malloc((size_t)E * sizeof(mag_t));
+    for (int64_t t = 0; t < T; ++t) {
+        const float* l = logits + t * E;
+        float* p = probs + t * E;
+        float maxv = l[0];
+        for (int64_t e = 1; e < E; ++e) if (l[e] > maxv) maxv = l[e];
+        float sum = 0.0f;
+        for (int64_t e = 0; e < E; ++e) { const float v = expf(l[e] - maxv); p[e] = v; sum += v; }
+        const float inv = 1.0f / sum;
+        for (int64_t e = 0; e < E; ++e) p[e] *= inv;
+        for (int64_t e = 0; e < E; ++e) { sc[e].a = p[e]; sc[e].i = (int)e; }
+        top_k_by_magnitude(sc, (int)E, (int)k);
+        for (int64_t j = 0; j < k; ++j) { indices[t * k + j] = sc[j].i; weights[t * k + j] = sc[j].a; }
+    }
+    free(sc);
+}
+
+/* Y[nt][N] = X[nt][Kd] W[N][Kd]^T */
+static void moe_matmul(const float* X, const float* W, float* Y, int64_t nt, int64_t N, int64_t Kd, int as_double) {
+    for (int64_t m = 0; m < nt; ++m)
+        for (int64_t n = 0; n < N; ++n) {
+            const float* xr = X + m * Kd;
+            const float* wr = W + n * Kd;
+            if (as_double) {
+                double acc = 0.0;
+                for (int64_t k = 0; k < Kd; ++k) acc += (double)xr[k] * (double)wr[k];
+                Y[m * N + n] = (float)acc;
+            } else {
+                float acc = 0.0f;
+                for (int64_t k = 0; k < Kd; ++k) acc = fmaf(xr[k], wr[k], acc);
+                Y[m * N + n] = acc;
+            }
+        }
+}
+
+void orc_moe_dispatch(const float* x, const float* const* gate, const float* const* up,
+                      const float* const* down, const int64_t* indices, const float* weights,
+                      int64_t T, int64_t K, int64_t E, int64_t D, int64_t F,
+                      float* out, float* z_loss, int64_t* dropped, int as_double) {
+    double* wide = as_double ? (double*)calloc((size_t)(T * D), sizeof(double)) : NULL;
+    memset(out, 0, (size_t)(T * D) * sizeof(float));
+    float zl = 0.0f;
+    int64_t drop = 0;
+    int64_t* toks = (int64_t*)malloc((size_t)(T * K + 1) * sizeof(int64_t));
+    for (int64_t e = 0; e < E; ++e) {
+        int64_t nt = 0;
+        for (int64_t t = 0; t < T; ++t)
+            for (int64_t k = 0; k < K; ++k)
+                if (indices[t * K + k] == e) toks[nt++] = t;
+        if (nt == 0) continue;
+        float* bi = (float*)malloc((size_t)(nt * D) * sizeof(float));
+        float* g = (float*)malloc((size_t)(nt * F) * sizeof(float));
+        float* u = (float*)malloc((size_t)(nt * F) * sizeof(float));
+        float* bo = (float*)malloc((size_t)(nt * D) * sizeof(float));
+        for (int64_t i = 0; i < nt; ++i) memcpy(bi + i * D, x + toks[i] * D, (size_t)D * sizeof(float));
+        moe_matmul(bi, gate[e], g, nt, F, D, as_double);
+        moe_matmul(bi, up[e], u, nt, F, D, as_double);
+        for (int64_t i = 0; i < nt * F; ++i) { const float v = g[i]; g[i] = (v / (1.0f + expf(-v))) * u[i]; }
+        moe_matmul(g, down[e], bo, nt, D, F, as_double);
+        for (int64_t i = 0; i < nt; ++i) {
+            const int64_t t = toks[i];
+            float wgt = 0.0f;
+            for (int64_t k = 0; k < K; ++k) if (indices[t * K + k] == e) { wgt = weights[t * K + k]; break; }
+            if (wgt <= 0.0f) { drop++; continue; }
+            for (int64_t d = 0; d < D; ++d) {
+                const float v = wgt * bo[i * D + d];
+                if (as_double) wide[t * D + d] += (double)wgt * (double)bo[i * D + d];
+                else out[t * D + d] += v;
+                zl = fmaf(v, v, zl);
+            }
+        }
+        free(bi); free(g); free(u); free(bo);
+    }
+    if (as_double) { for (int64_t i = 0; i < T * D; ++i) out[i] = (float)wide[i]; free(wide); }
+    free(toks);
+    if (z_loss) *z_loss = zl;
+    if (dropped) *dropped = drop;
+}

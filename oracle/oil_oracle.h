@@ -136,6 +136,23 @@ void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
                            const float* cb, float* C,
                            int64_t M, int64_t N, int64_t K, int as_double);
 
+/* Mixture-of-experts routing and dispatch.
+ * orc_softmax_topk: softmax_with_topk (src/moe_variants.cpp:97-134): max-subtracted expf softmax in
+ *   FP32, probabilities scaled by 1/sum, top-k by libstdc++'s partial_sort with a > comparator
+ *   (ties land where its heap leaves them), weights = raw probabilities.
+ * orc_moe_dispatch: moe_dispatch_batched (src/moe_variants.cpp:767-827) over ExpertFFN::forward
+ *   (:77-91, SiLU) with bias-free experts given as decoded row-major matrices gate/up [F][D] and
+ *   down [D][F] per expert (Y = X W^T); the matmul chain follows kernel::scalar_gemm
+ *   (src/kernel_gemm.cpp:13-23: FP32, k ascending, each multiply-add fused as in the -mfma build),
+ *   silu = v / (1 + expf(-v)) (src/math.cpp:117-126).  as_double != 0: matmuls and the output sum in
+ *   double (the yardstick for the GPU path).  z_loss / dropped may be NULL. */
+void orc_softmax_topk(const float* logits, int64_t T, int64_t E, int64_t k,
+                      float* probs, int64_t* indices, float* weights);
+void orc_moe_dispatch(const float* x, const float* const* gate, const float* const* up,
+                      const float* const* down, const int64_t* indices, const float* weights,
+                      int64_t T, int64_t K, int64_t E, int64_t D, int64_t F,
+                      float* out, float* z_loss, int64_t* dropped, int as_double);
+
 #ifdef __cplusplus
 }
 #endif

@@ -347,8 +347,74 @@ def make_container():
     print("mixed.oil", os.path.getsize(path), "bytes; container.npz written", out["meta"])
 
 
+MOE_ROUTE_CASES = [(64, 8, 2), (5, 4, 1), (33, 16, 4), (7, 3, 3), (100, 8, 8), (16, 64, 6)]
+MOE_SHAPE = dict(T=10, E=3, K=2, D=256, F=512)
+
+
+def moe_route_logits(T, E, kind, rng):
+    lg = rng.standard_normal((T, E)).astype(np.float32)
+    if kind == 1:
+        lg = np.round(lg)                       # many exact ties
+    if kind == 2:
+        lg[:] = np.float32(0.5)                 # all experts equal
+    return lg
+
+
+def moe_experts(seed, E, D, F, fmts=(3, 3, 3)):
+    """Per expert: (payload, blocks) of gate [F][D], up [F][D], down [D][F], quantized with the oracle's
+    quantizer (byte-identical to the reference's), and their decoded matrices."""
+    rng = np.random.default_rng(seed)
+    packs, dense = [], []
+    for e in range(E):
+        pe, de = [], []
+        for (r, c), f in zip(((F, D), (F, D), (D, F)), fmts):
+            w = (rng.standard_normal(r * c) * (1.0 / np.sqrt(c))).astype(np.float32)
+            payload, blocks = O.quantize_tensor(w, f)
+            pe.append((payload, blocks))
+            de.append(O.dequant_blocks(payload, blocks).reshape(r, c))
+        packs.append(pe)
+        dense.append(de)
+    return packs, dense
+
+
+def make_moe():
+    """softmax_with_topk and moe_dispatch_batched as the compiled reference answers."""
+    R = O.ref_moe()
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    out = {}
+    rng = np.random.default_rng(1)
+    pr, ix, wt = [], [], []
+    for T, E, k in MOE_ROUTE_CASES:
+        for kind in range(3):
+            lg = moe_route_logits(T, E, kind, rng)
+            p_, i_, w_ = O.softmax_topk(lg, k, fn=R.ref_softmax_topk)
+            pr.append(p_.view(np.uint32).ravel()); ix.append(i_.ravel()); wt.append(w_.view(np.uint32).ravel())
+    out["route_probs"] = np.concatenate(pr)
+    out["route_idx"] = np.concatenate(ix)
+    out["route_w"] = np.concatenate(wt)
+    sh = MOE_SHAPE
+    _, dense = moe_experts(11, sh["E"], sh["D"], sh["F"])
+    rng = np.random.default_rng(12)
+    x = rng.standard_normal((sh["T"], sh["D"])).astype(np.float32)
+    lg = rng.standard_normal((sh["T"], sh["E"])).astype(np.float32)
+    _, idx, w = O.softmax_topk(lg, sh["K"], fn=R.ref_softmax_topk)
+    w[2, 0] = 0.0            # a dropped pair
+    idx[4, 1] = -1           # an entry outside the expert range
+    idx[6, 1] = idx[6, 0]    # the same expert twice
+    o, z, dr = O.moe_dispatch(x, [d[0] for d in dense], [d[1] for d in dense], [d[2] for d in dense], idx, w,
+                              fn=R.ref_moe_dispatch)
+    out["disp_x"] = x
+    out["disp_idx"] = idx
+    out["disp_w"] = w
+    out["disp_out"] = o.view(np.uint32)
+    out["disp_z"] = np.array([z], np.float32)
+    out["disp_dropped"] = np.array([dr], np.int64)
+    np.savez_compressed(os.path.join(HERE, "moe.npz"), **out)
+    print("moe.npz written; dropped", dr, "z", z)
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container"]
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe"]
     for name in which:
         {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner,
-         "container": make_container}[name]()
+         "container": make_container, "moe": make_moe}[name]()

@@ -81,6 +81,15 @@ def test_oil4_fast_kernel_shapes(rows, cols, M):
     assert rel_l2(ref32, want) <= TOL
 
 
+# the multi-token kernel: every pass width (1..4 token groups), a ragged last pass, several
+# row tiles per workgroup (rows > 48 * 256), several K-slabs, an odd number of blocks per row
+@pytest.mark.parametrize("rows,cols", [(130, 4096), (61, 11008), (13000, 512), (47, 14336), (3, 256)])
+@pytest.mark.parametrize("M", [3, 5, 8, 9, 13, 17, 40])
+def test_oil4_multi_token_counts(rows, cols, M):
+    err, *_ = run_case(ia.Format.OIL4, rows, cols, M, seed=7 * rows + cols + M)
+    assert err <= TOL
+
+
 def test_oil4_special_blocks():
     """Zero blocks (-0.0 levels), underflowing scales, huge outliers, zero activations."""
     rows, cols = 96, 4096
