@@ -146,6 +146,11 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
     if (regular && uniform && nblocks)
         w->uniform_stride = nblocks > 1 ? (db[1].off16 - db[0].off16) * 16u
                                         : (uint32_t)((db[0].cb_bytes + db[0].idx_bytes + 15u) & ~15u);
+    if (w->uniform_stride) {
+        w->uniform_cb = db[0].cb_bytes;
+        w->uniform_idx = db[0].idx_bytes;
+        w->uniform_base = db[0].off16 * 16u;
+    }
     *out = w;
     return OILHIP_OK;
 }
@@ -237,6 +242,8 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
                                                        (uint32_t)M, (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
+    const int rc = launch_gemv_runs(*w, d_x, d_y, M, (hipStream_t)stream);
+    if (rc <= 0) return rc;
     return launch_gemv_generic(*w, d_x, d_y, M, (hipStream_t)stream);
 }
 

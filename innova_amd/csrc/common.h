@@ -39,6 +39,8 @@ struct oilhip_weights {
     uint32_t nblocks = 0;
     int uniform_fmt = -1;                   // single format id, or -1
     uint32_t uniform_stride = 0;            // bytes between consecutive blocks when regular, else 0
+    uint32_t uniform_cb = 0, uniform_idx = 0;   // channel sizes of every block when regular
+    uint32_t uniform_base = 0;              // byte offset of block 0 when regular
     bool all_full = false;                  // every block holds exactly 256 weights
 };
 
@@ -51,5 +53,7 @@ int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int 
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s);
+// every format and mixed rows, a lane per run of 32 weights
+int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
 }  // namespace oilhip
