@@ -196,6 +196,23 @@ int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb256, float scale,
 int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b_idx, const float* d_cb,
                              float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* The engines whose B operand is not a codebook index, same [K][N] flat layout and loop order:
+ *   kind 1  Oil1Engine::quant_gemm  (include/oil/oil_engines.h:123, src/oil_engines_oil1.cpp:61-82):
+ *           d_b = one float per 32 flat positions
+ *   kind 3  SparkEngine::quant_gemm (oil_engines.h:103, src/oil_engines_spark.cpp:154-186): d_b = 2-bit codes
+ *           (2 -> +, 0 -> -, else 0), d_scales[flat / block] with block = the engine's block size
+ *   kind 16 OIL16Engine::quant_gemm (oil_engines.h:167, src/oil_engines_fp.cpp:433-451): d_b = FP16 bits
+ *   kind 32 OIL32Engine::quant_gemm (src/oil_engines_fp.cpp:531-547): d_b = FP32                        */
+/* OIL{8,4,2}Engine::dequant_tensor (oil_engines.h:48,77,150; src/oil_engines_oil8.cpp:171-183, oil4.cpp:205-220,
+ * oil2.cpp:184-193) when d_scales is NULL: n packed codes -> codebook values.  With d_scales:
+ * OIL8Engine::dequantize_per_block (src/oil_engines_oil8.cpp:121-134, one scale per block) and
+ * OIL4Engine::dequantize_per_block (src/oil_engines_oil4.cpp:136-150, {center, half_range} per block) over one
+ * index byte per weight. */
+int oilhip_engine_dequant(int bits, const uint8_t* d_idx, const float* d_cb, int64_t n, const float* d_scales,
+                          int64_t block, float* d_out, void* stream);
+int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const float* d_scales, int64_t block,
+                             float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
+
 /* ------------------------------------------------------------ mixture of experts
  * oilhip_moe_route   : moe::softmax_with_topk (include/oil/moe_variants.h:693, src/moe_variants.cpp:97-134).
  *                      Host arrays: logits/probs [T][E], indices (int64) and weights [T][k]; weights are the

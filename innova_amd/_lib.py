@@ -57,6 +57,8 @@ _SIGNATURES = {
     "oilhip_file_upload_tensor": (C.c_int, [vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
     "oilhip_file_write": (C.c_int, [C.c_char_p, C.c_uint32, C.c_uint32, vp, C.c_uint32, C.c_uint32, C.POINTER(C.c_char_p), vp,
                                     vp, vp, C.c_uint32]),
+    "oilhip_engine_dequant": (C.c_int, [C.c_int, vp, vp, C.c_int64, vp, C.c_int64, vp, vp]),
+    "oilhip_engine_dense_gemm": (C.c_int, [C.c_int, vp, vp, vp, C.c_int64, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
     "oilhip_moe_route": (C.c_int, [vp, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]),
     "oilhip_moe_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
     "oilhip_moe_forward": (C.c_int, [vp, vp, vp, C.c_int, vp, vp, vp, C.c_int64, C.c_int64, vp, vp, C.c_size_t,

@@ -5,6 +5,8 @@
 //   oil::engines::OIL{8,4,2}Engine::quant_gemm  src/oil_engines_oil{8,4,2}.cpp
 // One workgroup of 256 threads per output row; the codebook sits in LDS; thread t
 // walks k = t, t+256, ... so index bytes are read coalesced.
+#include <algorithm>
+
 #include "common.h"
 
 namespace oilhip {
@@ -138,6 +140,62 @@ engine_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const
     C[m * N + n] = acc;
 }
 
+// The engines whose B operand is not a codebook index: kind 1 = Oil1Engine (one float per 32 flat positions,
+// src/oil_engines_oil1.cpp:61-82), 3 = SparkEngine (2-bit codes: 2 -> +s, 0 -> -s, else 0, with s = a * scale of
+// the flat position's block, src/oil_engines_spark.cpp:154-186), 16 = OIL16Engine (FP16 widened as
+// math::vec_fp16_to_fp32 does, src/math.cpp:509-526; src/oil_engines_fp.cpp:433-451), 32 = OIL32Engine (:531-547).
+// Terms with a == 0 are skipped and k runs in ascending order, as in the reference loops.
+template <int KIND>
+__global__ void __launch_bounds__(256)
+engine_dense_kernel(const float* __restrict__ A, const void* __restrict__ B, const float* __restrict__ scales,
+                    long long block, float* __restrict__ C, long long M, long long N, long long K) {
+    const long long n = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long m = blockIdx.y;
+    if (n >= N) return;
+    float acc = 0.0f;
+    for (long long k = 0; k < K; ++k) {
+        const float a = A[m * K + k];
+        if (a == 0.0f) continue;
+        const long long flat = k * N + n;
+        if (KIND == 1) {
+            acc = __fmaf_rn(a, reinterpret_cast<const float*>(B)[flat / 32], acc);
+        } else if (KIND == 32) {
+            acc = __fmaf_rn(a, reinterpret_cast<const float*>(B)[flat], acc);
+        } else if (KIND == 16) {
+            const uint32_t h = reinterpret_cast<const uint16_t*>(B)[flat];
+            const float b = (h & 0x7FFFu) == 0u ? 0.0f : half_bits_to_float(h);    // -0 widens to +0 there
+            acc = __fmaf_rn(a, b, acc);
+        } else {
+            const float s = a * scales[flat / block];
+            const uint32_t code = (reinterpret_cast<const uint8_t*>(B)[flat / 4] >> ((flat % 4) * 2)) & 3u;
+            if (code == 2u) acc += s;
+            else if (code == 0u) acc -= s;
+        }
+    }
+    C[m * N + n] = acc;
+}
+
+// OIL{8,4,2}Engine::dequant_tensor (src/oil_engines_oil8.cpp:171-183, oil4.cpp:205-220, oil2.cpp:184-193): packed
+// codes -> codebook values; with scales, OIL8Engine / OIL4Engine::dequantize_per_block (oil8.cpp:121-134:
+// cb[i] * scale; oil4.cpp:136-150: cb[i] * half_range + center, one multiply-add in the reference build) over
+// one index byte per weight.
+__global__ void __launch_bounds__(256)
+engine_dequant_kernel(int bits, const uint8_t* __restrict__ idx, const float* __restrict__ cb, long long n,
+                      const float* __restrict__ scales, long long block, float* __restrict__ out) {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+        if (!scales) {
+            const int per = 8 / bits;
+            const uint32_t code = (idx[i / per] >> ((i % per) * bits)) & ((1u << bits) - 1u);
+            out[i] = cb[code];
+        } else if (bits == 8) {
+            out[i] = cb[idx[i]] * scales[i / block];
+        } else {
+            const long long b = i / block;
+            out[i] = __fmaf_rn(cb[idx[i] & 15u], scales[2 * b + 1], scales[2 * b]);
+        }
+    }
+}
+
 // Negative sizes are errors; an empty output (M or N zero) needs no pointers at all.
 int check(const void* a, const void* b, const void* c, const void* d, long long M, long long N, long long K) {
     if (M < 0 || N < 0 || K < 0) return fail(OILHIP_E_ARG, "negative dimension");
@@ -214,6 +272,37 @@ int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b, con
     if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     else if (bits == 4) hipLaunchKernelGGL(engine_kernel<4>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     else hipLaunchKernelGGL(engine_kernel<2>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_engine_dequant(int bits, const uint8_t* d_idx, const float* d_cb, int64_t n, const float* d_scales,
+                          int64_t block, float* d_out, void* stream) {
+    if (n < 0) return fail(OILHIP_E_ARG, "negative length");
+    if (n == 0) return OILHIP_OK;
+    if (!d_idx || !d_cb || !d_out) return fail(OILHIP_E_ARG, "null argument");
+    if (bits != 2 && bits != 4 && bits != 8) return fail(OILHIP_E_ARG, "bits must be 2, 4 or 8");
+    if (d_scales && (bits == 2 || block <= 0)) return fail(OILHIP_E_ARG, "per-block dequantize exists for 4 and 8 bits with a positive block size");
+    const uint32_t grid = (uint32_t)std::min<int64_t>((n + 255) / 256, 65535);
+    hipLaunchKernelGGL(engine_dequant_kernel, dim3(grid), dim3(256), 0, (hipStream_t)stream, bits, d_idx, d_cb, (long long)n,
+                       d_scales, (long long)block, d_out);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const float* d_scales, int64_t block,
+                             float* d_c, int64_t M, int64_t N, int64_t K, void* stream) {
+    if (int rc = check(d_a, d_b, d_c, d_c, M, N, K)) return rc;
+    if (kind != 1 && kind != 3 && kind != 16 && kind != 32) return fail(OILHIP_E_ARG, "kind must be 1, 3, 16 or 32");
+    if (M == 0 || N == 0) return OILHIP_OK;
+    if (kind == 3 && (!d_scales || block <= 0)) return fail(OILHIP_E_ARG, "the SPARK engine needs scales and a block size");
+    if (M > 65535) return fail(OILHIP_E_ARG, "M exceeds the grid limit");
+    const dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)M);
+    hipStream_t s = (hipStream_t)stream;
+    if (kind == 1) hipLaunchKernelGGL(engine_dense_kernel<1>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else if (kind == 3) hipLaunchKernelGGL(engine_dense_kernel<3>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else if (kind == 16) hipLaunchKernelGGL(engine_dense_kernel<16>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else hipLaunchKernelGGL(engine_dense_kernel<32>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }

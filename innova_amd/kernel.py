@@ -101,3 +101,43 @@ def engine_quant_gemm(bits: int, a, b_idx, codebook, M: int, N: int, K: int):
     _lib.check(_lib.lib().oilhip_engine_quant_gemm(bits, ad.data_ptr(), bd.data_ptr(), cd.data_ptr(), out.data_ptr(),
                                                    M, N, K, _lib.current_stream()))
     return _ret(out, d1 and d2)
+
+
+def engine_dense_gemm(kind: int, a, b, M: int, N: int, K: int, scales=None, block_size: int = 128):
+    """quant_gemm of the engines whose B operand is not a codebook index (include/oil/oil_engines.h:103,123,167):
+    kind 1 Oil1Engine (b: float32, one value per 32 flat positions), 3 SparkEngine (b: uint8 2-bit codes,
+    scales: float32 per block_size flat positions), 16 OIL16Engine (b: uint16 FP16 bits), 32 OIL32Engine (b: float32)."""
+    import torch
+    bdt = {1: np.float32, 3: np.uint8, 16: np.uint16, 32: np.float32}.get(kind)
+    if bdt is None:
+        raise _lib.OilHipError("engine_dense_gemm: kind must be 1, 3, 16 or 32")
+    ad, d1 = _dev(a, np.float32)
+    if bdt is np.uint16 and not hasattr(b, "is_cuda"):
+        b = np.ascontiguousarray(b, np.uint16).view(np.int16)
+        bd, d2 = torch.from_numpy(b).cuda(), True
+    else:
+        bd, d2 = _dev(b, bdt)
+    sd = None
+    if kind == 3:
+        if scales is None:
+            raise _lib.OilHipError("engine_dense_gemm: the SPARK engine needs scales")
+        sd, _ = _dev(scales, np.float32)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_engine_dense_gemm(kind, ad.data_ptr(), bd.data_ptr(), sd.data_ptr() if sd is not None else None,
+                                                   int(block_size), out.data_ptr(), M, N, K, _lib.current_stream()))
+    return _ret(out, d1 and d2)
+
+
+def engine_dequant(bits: int, indices, codebook, n: int, scales=None, block_size: int = 0):
+    """OIL{8,4,2}Engine::dequant_tensor (packed codes; scales None) or OIL8/OIL4Engine::dequantize_per_block
+    (one index byte per weight; OIL8: one scale per block, OIL4: {center, half_range} per block)."""
+    import torch
+    i, d1 = _dev(indices, np.uint8)
+    c, _ = _dev(codebook, np.float32)
+    sd = None
+    if scales is not None:
+        sd, _ = _dev(scales, np.float32)
+    out = torch.empty(n, dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_engine_dequant(bits, i.data_ptr(), c.data_ptr(), n, sd.data_ptr() if sd is not None else None,
+                                                int(block_size), out.data_ptr(), _lib.current_stream()))
+    return _ret(out, d1)

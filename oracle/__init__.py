@@ -336,3 +336,18 @@ def ref_moe():
     """The compiled reference's routing/dispatch library, or None where it has not been built."""
     path = os.path.join(_HERE, "_ref", "liboilref_moe.so")
     return C.CDLL(path) if os.path.exists(path) else None
+
+
+def engine_dense_gemm(kind: int, A, B, M: int, N: int, K: int, scales=None, block: int = 128, fn=None):
+    """orc_engine_dense_gemm, or with fn = the compiled reference's ref_engine_dense_gemm."""
+    A = np.ascontiguousarray(A, np.float32)
+    B = np.ascontiguousarray(B)
+    sc = np.ascontiguousarray(scales, np.float32) if scales is not None else np.zeros(1, np.float32)
+    out = np.zeros((M, N), np.float32)
+    if fn is None:
+        lib().orc_engine_dense_gemm(C.c_int(kind), C.c_void_p(A.ctypes.data), C.c_void_p(B.ctypes.data), C.c_void_p(sc.ctypes.data),
+                                    C.c_int64(block), C.c_void_p(out.ctypes.data), C.c_int64(M), C.c_int64(N), C.c_int64(K))
+    else:
+        fn(C.c_int(kind), C.c_void_p(A.ctypes.data), C.c_void_p(B.ctypes.data), C.c_size_t(B.nbytes), C.c_void_p(sc.ctypes.data),
+           C.c_int64(sc.size), C.c_int64(block), C.c_void_p(out.ctypes.data), C.c_int64(M), C.c_int64(N), C.c_int64(K))
+    return out

@@ -1047,3 +1047,42 @@ void orc_moe_dispatch(const float* x, const float* const* gate, const float* con
     if (z_loss) *z_loss = zl;
     if (dropped) *dropped = drop;
 }
+
+/* ------------------------------------------------------------------ dense / sign-coded engines */
+static float widen_fp16_engine(uint16_t h) {          /* src/math.cpp:509-526 */
+    const uint32_t sign = (uint32_t)(h >> 15) << 31;
+    const int32_t e = (h >> 10) & 0x1F;
+    const uint32_t mant = h & 0x03FF;
+    uint32_t bits;
+    float out;
+    if (e == 0) {
+        if (mant == 0) return 0.0f;
+        return (sign ? -1.0f : 1.0f) * ((float)mant / 1024.0f) * 1.5258789e-5f;
+    }
+    bits = e == 31 ? (sign | 0x7F800000u | (mant << 13)) : (sign | ((uint32_t)(e + 112) << 23) | (mant << 13));
+    memcpy(&out, &bits, 4);
+    return out;
+}
+
+void orc_engine_dense_gemm(int kind, const float* A, const void* B, const float* scales, int64_t block,
+                           float* C, int64_t M, int64_t N, int64_t K) {
+    for (int64_t i = 0; i < M * N; ++i) C[i] = 0.0f;
+    for (int64_t m = 0; m < M; ++m)
+        for (int64_t k = 0; k < K; ++k) {
+            const float a = A[m * K + k];
+            if (a == 0.0f) continue;
+            for (int64_t n = 0; n < N; ++n) {
+                const int64_t flat = k * N + n;
+                float* c = &C[m * N + n];
+                if (kind == 1) *c = fmaf(a, ((const float*)B)[flat / 32], *c);
+                else if (kind == 32) *c = fmaf(a, ((const float*)B)[flat], *c);
+                else if (kind == 16) *c = fmaf(a, widen_fp16_engine(((const uint16_t*)B)[flat]), *c);
+                else {
+                    const float s = a * scales[flat / block];
+                    const unsigned code = (((const uint8_t*)B)[flat / 4] >> ((flat % 4) * 2)) & 3u;
+                    if (code == 2u) *c += s;
+                    else if (code == 0u) *c -= s;
+                }
+            }
+        }
+}

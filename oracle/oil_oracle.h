@@ -136,6 +136,13 @@ void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
                            const float* cb, float* C,
                            int64_t M, int64_t N, int64_t K, int as_double);
 
+/* Engines with a dense or sign-coded B operand, [K][N] flat layout, k ascending, a == 0 skipped, each
+ * multiply-add fused as in the -mfma build: kind 1 Oil1Engine (src/oil_engines_oil1.cpp:61-82), 3 SparkEngine
+ * (src/oil_engines_spark.cpp:154-186), 16 OIL16Engine (src/oil_engines_fp.cpp:433-451, widening as
+ * src/math.cpp:509-526), 32 OIL32Engine (src/oil_engines_fp.cpp:531-547). */
+void orc_engine_dense_gemm(int kind, const float* A, const void* B, const float* scales, int64_t block,
+                           float* C, int64_t M, int64_t N, int64_t K);
+
 /* Mixture-of-experts routing and dispatch.
  * orc_softmax_topk: softmax_with_topk (src/moe_variants.cpp:97-134): max-subtracted expf softmax in
  *   FP32, probabilities scaled by 1/sum, top-k by libstdc++'s partial_sort with a > comparator

@@ -234,4 +234,46 @@ int ref_oil_meta(const char* path, const char* name, uint32_t* nblocks, uint32_t
     return 0;
 }
 
+// Oil1Engine / SparkEngine / OIL16Engine / OIL32Engine::quant_gemm (include/oil/oil_engines.h:103,123,167).
+// b holds the engine's packed operand verbatim (floats, 2-bit codes, FP16 bits, floats).
+void ref_engine_dense_gemm(int kind, const float* A, const void* b, size_t b_bytes, const float* scales, int64_t nscales,
+                           int64_t block, float* C, int64_t M, int64_t N, int64_t K) {
+    oil::Tensor a({M, K});
+    std::memcpy(a.data<float>(), A, (size_t)(M * K) * 4);
+    oil::Tensor c;
+    if (kind == 16) {
+        oil::Tensor bt({(int64_t)(b_bytes / 2)}, oil::DType::F16);
+        std::memcpy(bt.data<uint16_t>(), b, b_bytes);
+        oil::engines::OIL16Engine e;
+        c = e.quant_gemm(a, bt, M, N, K);
+    } else {
+        oil::Tensor bt({(int64_t)((b_bytes + 3) / 4)});
+        std::memcpy(bt.data<float>(), b, b_bytes);
+        if (kind == 1) { oil::engines::Oil1Engine e; c = e.quant_gemm(a, bt, 1.0f, M, N, K); }
+        else if (kind == 32) { oil::engines::OIL32Engine e; c = e.quant_gemm(a, bt, M, N, K); }
+        else {
+            oil::Tensor st({nscales});
+            std::memcpy(st.data<float>(), scales, (size_t)nscales * 4);
+            oil::engines::SparkEngine e(block);
+            c = e.quant_gemm(a, bt, st, M, N, K);
+        }
+    }
+    std::memcpy(C, c.data<float>(), (size_t)(M * N) * 4);
+}
+
+// dequant_tensor (scales null) / dequantize_per_block of the engines with their default codebooks.
+void ref_engine_dequant(int bits, const uint8_t* idx, int64_t n, const float* scales, int64_t block, float* out) {
+    if (!scales) {
+        oil::Tensor t;
+        if (bits == 8) { oil::engines::OIL8Engine e; t = e.dequant_tensor(idx, n); }
+        else if (bits == 4) { oil::engines::OIL4Engine e; t = e.dequant_tensor(idx, n); }
+        else { oil::engines::OIL2Engine e; t = e.dequant_tensor(idx, n); }
+        std::memcpy(out, t.data<float>(), (size_t)n * 4);
+    } else if (bits == 8) {
+        oil::engines::OIL8Engine e; e.dequantize_per_block(idx, scales, n, block, out);
+    } else {
+        oil::engines::OIL4Engine e; e.dequantize_per_block(idx, scales, n, block, out);
+    }
+}
+
 }  // extern "C"

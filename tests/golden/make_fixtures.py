@@ -413,8 +413,77 @@ def make_moe():
     print("moe.npz written; dropped", dr, "z", z)
 
 
+ENGINE_DENSE = dict(M=3, N=96, K=80, block=128)
+
+
+def engine_dense_inputs(kind):
+    """(A, B, scales) for Oil1 / Spark / OIL16 / OIL32 engine quant_gemm cases; some activations are zero."""
+    sh = ENGINE_DENSE
+    rng = np.random.default_rng(40 + kind)
+    A = rng.standard_normal((sh["M"], sh["K"])).astype(np.float32)
+    A[:, ::7] = 0.0
+    flat = sh["K"] * sh["N"]
+    scales = None
+    if kind == 1:
+        B = rng.standard_normal((flat + 31) // 32).astype(np.float32)
+    elif kind == 32:
+        B = rng.standard_normal(flat).astype(np.float32)
+    elif kind == 16:
+        B = rng.standard_normal(flat).astype(np.float16).view(np.uint16).copy()
+        B[:8] = [0x8000, 0x0000, 0x0001, 0x83FF, 0x7C00, 0xFC00, 0x0400, 0x3C00]     # signed zero, subnormals, infinities
+        A[:, 0] = 0.0                                                                # keep the infinities out of the sums
+        B[4 * sh["N"]: 4 * sh["N"] + 0] = 0
+        B[4:6] = [0x3800, 0xB800]
+    else:
+        B = rng.integers(0, 256, (flat + 3) // 4).astype(np.uint8)
+        scales = np.abs(rng.standard_normal((flat + sh["block"] - 1) // sh["block"])).astype(np.float32)
+    return A, B, scales
+
+
+def engine_dequant_inputs(bits):
+    n = {8: 1001, 4: 999, 2: 1003}[bits]
+    rng = np.random.default_rng(60 + bits)
+    return rng.integers(0, 256, (n * bits + 7) // 8).astype(np.uint8), n
+
+
+def engine_block_inputs(bits):
+    n, block = 777, 64
+    rng = np.random.default_rng(70 + bits)
+    idx = rng.integers(0, 1 << bits, n).astype(np.uint8)
+    nb = (n + block - 1) // block
+    scales = rng.standard_normal(nb * (2 if bits == 4 else 1)).astype(np.float32)
+    return idx, scales, n, block
+
+
+def make_engines():
+    R = O.ref(True)
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    sh = ENGINE_DENSE
+    out = {}
+    for kind in (1, 3, 16, 32):
+        A, B, scales = engine_dense_inputs(kind)
+        Cc = O.engine_dense_gemm(kind, A, B, sh["M"], sh["N"], sh["K"], scales, sh["block"], fn=R.ref_engine_dense_gemm)
+        out[f"c{kind}"] = Cc.view(np.uint32)
+    # dequant_tensor (packed codes) and dequantize_per_block (one index byte per weight), default codebooks
+    for bits in (8, 4, 2):
+        cb = np.zeros(256, np.float32)
+        ncb = R.ref_engine_codebook(bits, p(cb, f32p))
+        out[f"cb{bits}"] = cb[:ncb].view(np.uint32)
+        idx, n = engine_dequant_inputs(bits)
+        o = np.zeros(n, np.float32)
+        R.ref_engine_dequant(C.c_int(bits), p(idx, u8p), C.c_int64(n), None, C.c_int64(0), p(o, f32p))
+        out[f"dq{bits}"] = o.view(np.uint32)
+    for bits in (8, 4):
+        idx, scales, n, block = engine_block_inputs(bits)
+        o = np.zeros(n, np.float32)
+        R.ref_engine_dequant(C.c_int(bits), p(idx, u8p), C.c_int64(n), p(scales, f32p), C.c_int64(block), p(o, f32p))
+        out[f"pb{bits}"] = o.view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "engines.npz"), **out)
+    print("engines.npz written")
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe"]
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe", "engines"]
     for name in which:
         {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner,
-         "container": make_container, "moe": make_moe}[name]()
+         "container": make_container, "moe": make_moe, "engines": make_engines}[name]()

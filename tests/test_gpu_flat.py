@@ -102,3 +102,39 @@ def test_empty_and_bad_arguments():
     assert ia.kernel.oil8_gemm(np.zeros(0, np.uint8), np.zeros(256, np.float32), np.zeros(0, np.float32), 0, 0, 4).shape == (0, 0)
     with pytest.raises(ia.OilHipError):
         ia.kernel.engine_quant_gemm(3, np.zeros(4, np.float32), np.zeros(4, np.uint8), np.zeros(8, np.float32), 1, 1, 4)
+
+
+@pytest.mark.parametrize("kind", [1, 3, 16, 32])
+def test_engine_dense_gemm_bit_exact(kind):
+    """Oil1 / Spark / OIL16 / OIL32 engine quant_gemm on the device: same k order and fused multiply-add as the
+    reference build, so the compiled reference's output is reproduced bit for bit."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(os.path.dirname(__file__), "golden", "make_fixtures.py"))
+    MF = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(MF)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "engines.npz"))
+    sh = MF.ENGINE_DENSE
+    A, B, scales = MF.engine_dense_inputs(kind)
+    got = ia.kernel.engine_dense_gemm(kind, A, B, sh["M"], sh["N"], sh["K"], scales=scales, block_size=sh["block"])
+    assert np.array_equal(np.asarray(got).view(np.uint32), gold[f"c{kind}"])
+    with pytest.raises(ia.OilHipError):
+        ia.kernel.engine_dense_gemm(5, A, B, 1, 1, 1)
+
+
+def test_engine_dequant_bit_exact():
+    """dequant_tensor (packed codes) and dequantize_per_block against the compiled reference's outputs."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(os.path.dirname(__file__), "golden", "make_fixtures.py"))
+    MF = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(MF)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "engines.npz"))
+    for bits in (8, 4, 2):
+        idx, n = MF.engine_dequant_inputs(bits)
+        got = ia.kernel.engine_dequant(bits, idx, gold[f"cb{bits}"].view(np.float32), n)
+        assert np.array_equal(np.asarray(got).view(np.uint32), gold[f"dq{bits}"]), bits
+    for bits in (8, 4):
+        idx, scales, n, block = MF.engine_block_inputs(bits)
+        got = ia.kernel.engine_dequant(bits, idx, gold[f"cb{bits}"].view(np.float32), n, scales=scales, block_size=block)
+        assert np.array_equal(np.asarray(got).view(np.uint32), gold[f"pb{bits}"]), bits
+    with pytest.raises(ia.OilHipError):
+        ia.kernel.engine_dequant(2, np.zeros(4, np.uint8), np.zeros(4, np.float32), 4, scales=np.zeros(1, np.float32), block_size=4)

@@ -153,3 +153,30 @@ def test_flat_against_compiled_reference():
         R.ref_oil4_gemm(pk.ctypes.data_as(u8p), cb16.ctypes.data_as(u16p), act4.ctypes.data_as(f32p),
                         out.ctypes.data_as(f32p), M, N, K)
         assert np.array_equal(out, O.oil4_gemm(pk, cb16, act4, M, N, K, 1).ravel())
+
+
+@pytest.mark.parametrize("kind", [1, 3, 16, 32])
+def test_engine_dense_gemm_matches_reference(kind):
+    """Oil1 / Spark / OIL16 / OIL32 engine quant_gemm: oracle bit-equal to the compiled reference's output."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(os.path.dirname(__file__), "golden", "make_fixtures.py"))
+    MF = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(MF)
+    gold = np.load(os.path.join(os.path.dirname(__file__), "golden", "engines.npz"))
+    sh = MF.ENGINE_DENSE
+    A, B, scales = MF.engine_dense_inputs(kind)
+    got = O.engine_dense_gemm(kind, A, B, sh["M"], sh["N"], sh["K"], scales, sh["block"])
+    assert np.array_equal(got.view(np.uint32), gold[f"c{kind}"])
+    # brute force in double on the decoded operand
+    flat = np.arange(sh["K"] * sh["N"])
+    if kind == 1:
+        dense = B[flat // 32]
+    elif kind == 32:
+        dense = B
+    elif kind == 16:
+        dense = B.view(np.float16).astype(np.float32)
+    else:
+        code = (B[flat // 4] >> ((flat % 4) * 2)) & 3
+        dense = np.where(code == 2, 1.0, np.where(code == 0, -1.0, 0.0)) * scales[flat // sh["block"]]
+    want = A.astype(np.float64) @ np.asarray(dense, np.float64).reshape(sh["K"], sh["N"])
+    assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5
