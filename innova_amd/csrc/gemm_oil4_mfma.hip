@@ -183,6 +183,172 @@ gemm_oil4_bf16_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict_
         }
 }
 
+// Pipelined kernel for larger M: 256 tokens x 128 weight rows per workgroup, 8 wavefronts (4 x 2, each
+// 64 x 64 outputs), 64 columns per step, two LDS tile buffers: while the matrix cores work on step kt, the
+// same wavefronts decode the weights of step kt+1 into the other buffer and the global loads of the
+// following steps are in flight, with one barrier per step.  Per step a thread stages 64 bytes of X' and
+// decodes 8 bytes (16 nibbles) of weights.
+#ifndef OILHIP_GEMM_DEPTH
+#define OILHIP_GEMM_DEPTH 2
+#endif
+constexpr int PK = 64;                      // columns per step
+constexpr int PLD = PK;                     // LDS row pitch in bf16: 128 bytes = 8 chunks of 16 bytes; the chunk index of a
+                                            // row is XOR-swizzled with (row / 2) % 8 so that the tile stores (2 rows x 8
+                                            // chunks per 16 lanes) and the fragment reads (16 rows x 1 chunk) touch every bank once
+constexpr int PBM = 256, PBN = 128;
+
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
+                           uint32_t M, uint32_t N, uint32_t K) {
+    extern __shared__ __align__(16) uint8_t lds[];
+    float* tab = reinterpret_cast<float*>(lds);
+    __bf16* As = reinterpret_cast<__bf16*>(lds + kTabBytes);                      // [2][PBM][PLD]
+    __bf16* Bs = As + 2 * PBM * PLD;                                              // [2][PBN][PLD]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t m0 = blockIdx.y * PBM, n0 = blockIdx.x * PBN;
+    const uint32_t bpr = K >> 8, KT = K / PK;
+
+    {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 512*k
+        const float lv_lane = level_literal(lane & 15u);
+        const float lo = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
+            reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo, hi, lo, hi);
+        }
+    }
+
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(W + (size_t)n0 * bpr * 128u), 0,
+        (int)((uint64_t)(N - n0 < (uint32_t)PBN ? N - n0 : (uint32_t)PBN) * bpr * 128u), 0x00020000);
+    const uint16_t* xa = Xp + (size_t)m0 * K;
+    const uint32_t brow = tid >> 2, bq = tid & 3u;                               // weight row of the tile, 8-byte piece of the 32 bytes of a step
+    const uint32_t lanebase = (lane & 31u) * 8u;
+
+    constexpr int D = OILHIP_GEMM_DEPTH;        // steps of global loads in flight: even, divides K / 64
+    u32x4 ar[D][4];
+    uint32_t br[D][2], sr[D];
+    auto load_regs = [&](int set, uint32_t kt) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
+            ar[set][c] = *reinterpret_cast<const u32x4*>(xa + (size_t)row * K + kt * PK + kc * 8u);
+        }
+        const uint32_t blk_off = (brow * bpr + (kt >> 2)) * 128u;
+        const uint32_t off = blk_off + (kt & 3u) * 32u + bq * 8u;
+        br[set][0] = __builtin_amdgcn_raw_buffer_load_b32(wrs, off, 0, 0);
+        br[set][1] = __builtin_amdgcn_raw_buffer_load_b32(wrs, off + 4u, 0, 0);
+        sr[set] = __builtin_amdgcn_raw_buffer_load_b16(wrs, blk_off, 0, 0);
+    };
+    // decode of the next step, split so that its table reads are issued before the fragment reads of the
+    // current step and its arithmetic runs in the shadow of the MFMAs
+    auto lookup_tiles = [&](int set, f32x2 (&t)[8]) {
+#pragma unroll
+        for (int d = 0; d < 2; ++d)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t addr = __builtin_amdgcn_perm(br[set][d], lanebase, 0x0C0C0000u | ((4u + j) << 8));
+                t[d * 4 + j] = *(lds_cfloat2*)(uintptr_t)addr;
+            }
+    };
+    auto finish_tiles = [&](int set, int buf, const f32x2 (&t)[8]) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
+            *reinterpret_cast<u32x4*>(As + (buf * PBM + row) * PLD + ((kc ^ ((row >> 1) & 7u)) * 8u)) = ar[set][c];
+        }
+        const float scale = __half2float(__ushort_as_half((unsigned short)sr[set]));
+        uint32_t packed[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const bf16x2 pr = bf16x2{(__bf16)(t[j].x * scale), (__bf16)(t[j].y * scale)};
+            packed[j] = *reinterpret_cast<const uint32_t*>(&pr);
+        }
+        const uint32_t sb = (brow >> 1) & 7u;
+        __bf16* dst = Bs + (buf * PBN + brow) * PLD;
+        *reinterpret_cast<u32x4*>(dst + (((2u * bq) ^ sb) * 8u)) = u32x4{packed[0], packed[1], packed[2], packed[3]};
+        *reinterpret_cast<u32x4*>(dst + (((2u * bq + 1u) ^ sb) * 8u)) = u32x4{packed[4], packed[5], packed[6], packed[7]};
+    };
+    auto store_tiles = [&](int set, int buf) {
+        f32x2 t[8];
+        lookup_tiles(set, t);
+        finish_tiles(set, buf, t);
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+
+    const uint32_t sw = ((lane & 31u) >> 1) & 7u;
+    auto step_mfmas = [&](int buf) {
+        const __bf16* ap = As + (buf * PBM + wm * 64u + (lane & 31u)) * PLD;
+        const __bf16* bp = Bs + (buf * PBN + wn * 64u + (lane & 31u)) * PLD;
+        bf16x8 a[4][2], b[4][2];
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const uint32_t ch = (((uint32_t)kk * 2u + (lane >> 5)) ^ sw) * 8u;
+#pragma unroll
+            for (int i = 0; i < 2; ++i) a[kk][i] = *reinterpret_cast<const bf16x8*>(ap + i * 32 * PLD + ch);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) b[kk][j] = *reinterpret_cast<const bf16x8*>(bp + j * 32 * PLD + ch);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+    };
+
+    // K is a multiple of 256, so KT is a multiple of 4 and of D.  Every load and every decode below is issued
+    // unconditionally (steps past the end are clamped to the last one and decoded into a buffer nobody reads):
+    // the number of loads in flight is then a compile-time fact and each wait covers exactly the step it needs.
+    static_assert(D == 2 || D == 4, "D must be even and divide 4");
+    const uint32_t last = KT - 1u;
+    auto clampk = [&](uint32_t k) { return k < last ? k : last; };
+#pragma unroll
+    for (int u = 0; u < D; ++u) load_regs(u, clampk((uint32_t)u));
+    __syncthreads();                                   // table complete
+    store_tiles(0, 0);
+    load_regs(0, clampk((uint32_t)D));
+    __syncthreads();
+    // register set s holds the steps congruent to s modulo D.  Iteration kt issues the table reads of step kt+1,
+    // then the fragment reads of step kt (buffer kt & 1), multiplies, finishes the decode of step kt+1 into the
+    // other buffer in the shadow of the MFMAs and refills that register set with step kt+1+D.
+    for (uint32_t kt0 = 0; kt0 < KT; kt0 += D) {
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const uint32_t kt = kt0 + u;
+            f32x2 t[8];
+            lookup_tiles((u + 1) % D, t);
+            step_mfmas(u & 1);
+            finish_tiles((u + 1) % D, (u + 1) & 1, t);
+            load_regs((u + 1) % D, clampk(kt + 1u + D));
+            __syncthreads();
+        }
+    }
+
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const uint32_t col = n0 + (wn * 2 + j) * 32u + (lane & 31u);
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t row = m0 + (wm * 2 + i) * 32u + 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u);
+                if (row < M && col < N) Y[(size_t)row * N + col] = acc[i][j][v];
+            }
+        }
+}
+
 // grow-only device scratch for X' (one per process and device; calls that overlap on one device race on it)
 std::mutex g_scratch_mu;
 uint16_t* g_scratch[64] = {};
@@ -238,6 +404,21 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
     if (gx > 64) gx = 64;
     hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
     OILHIP_HIP(hipGetLastError());
+    static const int pipe = [] { const char* e = getenv("OILHIP_GEMM_PIPE"); return e ? atoi(e) : 1; }();
+    if (big && pipe) {
+        static bool attr_done = false;
+        if (!attr_done) {
+            OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+            attr_done = true;
+        }
+        const uint32_t N = (uint32_t)w.rows;
+        const size_t lds_bytes = (size_t)kTabBytes + 2ull * (PBM + PBN) * PLD * 2;
+        hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel, dim3((N + PBN - 1) / PBN, Mpad / PBM), dim3(512), lds_bytes, s,
+                           w.d_payload, xp, d_y, (uint32_t)M, N, K);
+        OILHIP_HIP(hipGetLastError());
+        return OILHIP_OK;
+    }
     return big ? launch<4, 4>(w, xp, d_y, (uint32_t)M, Mpad, s) : launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
 }
 
