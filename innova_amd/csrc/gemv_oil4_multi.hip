@@ -13,9 +13,9 @@
 // A wavefront owns two blocks of the row per K-pass (8 wavefronts = 16 blocks = 4096 columns) and
 // keeps the activations of those blocks in registers (2 x 64 per lane), so the main loop is:
 // two 16-byte loads per lane and unit (16 rows x 1 block), 32 byte-pair table lookups, 64
-// multiplies by the block scale, 64 MFMAs.  The activations reach nibble order through a
-// wave-private LDS staging area that is reused for the 64 KB level table afterwards.  Partial
-// sums of the wavefronts are added through LDS once per tile of 64 rows.
+// multiplies by the block scale, 64 MFMAs.  The activations pass through a wave-private LDS
+// staging area in natural order; each lane gathers the values of its nibble positions from it.
+// Partial sums of the wavefronts are added through LDS once per tile of 64 rows.
 #include <hip/hip_fp16.h>
 
 #include "common.h"
@@ -29,16 +29,17 @@ using namespace oil4;
 typedef float v4f __attribute__((ext_vector_type(4)));
 
 constexpr int kGroups = 4;                // groups of 16 rows per tile
-constexpr int kTokStride = 292;           // floats per token in the staging area: 36 mod 64 spreads 16 tokens over all banks
-constexpr int kStageBytes = 16 * kTokStride * 4;   // per wavefront: 16 tokens x one block
+constexpr int kTokStride = 132;           // floats per token in the staging area: half a block plus the overlap
+constexpr int kStageBytes = 16 * kTokStride * 4;   // per wavefront: 16 tokens x 132 weights, natural order
+constexpr int kStageBase = kTabBytes;     // staging areas follow the level table
 
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const int* __restrict__ tok,
                        float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t ldy,
                        uint32_t xrows, uint32_t g_base, uint32_t g_rem) {
     extern __shared__ __align__(16) uint8_t lds[];
-    float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table (main loop)
-    float* red = reinterpret_cast<float*>(lds + kTabBytes);                // [8 waves][kGroups][64 lanes][4]
+    float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
+    float* red = reinterpret_cast<float*>(lds + kStageBase);               // [8 waves][kGroups][64 lanes][4], over the staging areas
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, kq = lane >> 4;
@@ -56,23 +57,10 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void*)x, 0, (int)(xbytes < 0x80000000ull ? xbytes : 0x80000000ull), 0x00020000);
 
-    // nibble-order offsets of the four floats of float4 number `lane` of a block:
-    // weight i sits at nibble p = i - i/64 + 4; position p is float (p/4 % 8)*32 + (p/32)*4 + p%4
-    uint32_t xoff[4];
-    bool xlast_ok;
-    {
-        const uint32_t w = lane * 4u;
-        xlast_ok = (w & 63u) != 60u;                                       // i % 64 == 63 is a slot
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const uint32_t pnib = w + k - (w >> 6) + 4u;
-            xoff[k] = ((pnib >> 2) & 7u) * 32u + (pnib >> 5) * 4u + (pnib & 3u);
-        }
-    }
-    float* stage = reinterpret_cast<float*>(lds + wave * kStageBytes);
+    float* stage = reinterpret_cast<float*>(lds + kStageBase + wave * kStageBytes);
 
     float breg[2][64];                     // activations of this wavefront's two blocks, token li, chunks kq and kq+4
-    v4f acc[kGroups];
+    v4f acc[kGroups][2];                   // two accumulation chains per group: consecutive MFMAs do not wait for each other
     const uint32_t lanebase = (lane & 31u) * 8u;
 
     u32x4 wv[2][2][2];                     // [buffer][block of the pair][half]
@@ -88,68 +76,84 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
         }
     };
 
+    // Nibble p = 32*(kq + 4h) + s of a block holds weight i = q + q/63 with q = p - 4 (p < 4: the scale).
+    // Inside a chunk q/63 steps at most once, at s = thr[h]; below it the weight index is base[h] + s.
+    int32_t gbase[2], gthr[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int32_t q0 = 32 * (int32_t)(kq + 4u * h) - 4;
+        const int32_t c0 = q0 >= 0 ? q0 / 63 : 0;
+        const int32_t t = 63 * (c0 + 1) - q0;                              // first s with q/63 == c0 + 1
+        gbase[h] = q0 + c0;
+        gthr[h] = t < 32 ? t : 32;
+    }
+
+    issue_group(0, g0, 0);                 // weights of the first group fly during the set-up
+    {   // pair table from literals (see gemv_oil4.hip)
+        const float lv_lane = level_literal(lane & 15u);
+        const float lo_fix = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
+            reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
+        }
+    }
+    bool table_synced = false;
+
     for (uint32_t tile = 0; tile < ntiles; ++tile) {
         const uint32_t tg0 = g0 + tile * kGroups;
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) acc[g] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int g = 0; g < kGroups; ++g) { acc[g][0] = v4f{0.f, 0.f, 0.f, 0.f}; acc[g][1] = v4f{0.f, 0.f, 0.f, 0.f}; }
         for (uint32_t pass = 0; pass < npass; ++pass) {
-            issue_group(0, tg0, pass);                                     // weights of the first group fly during the set-up
+            if (tile > 0 || pass > 0) issue_group(0, tg0, pass);
             if (npass > 1 || tile == 0) {
-                if (tile > 0 || pass > 0) __syncthreads();                 // the table is about to be overwritten
-                // ---- activations of this wavefront's two blocks -> registers, via wave-private LDS --------
-                // every activation load of the pass is requested at once: one memory round trip
-                u32x4 xv[2][16];
+                // ---- activations of this wavefront's two blocks -> registers.  The wavefront copies them in natural
+                // order (one 16-byte store per lane and token) into its own staging area, half a block at a time,
+                // and every lane then picks the 32 values of its token and chunk, skipping slot weights.
+                if (tile > 0) __syncthreads();                             // partial sums of the previous tile have been read
 #pragma unroll
                 for (int b2 = 0; b2 < 2; ++b2) {
                     const uint32_t blk = pass * 16u + wave * 2u + b2;
 #pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        const int m = m0 + t;
-                        const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
-                        xv[b2][t] = __builtin_amdgcn_raw_buffer_load_b128(
-                            xrsrc, (blk < bpr && src < xrows) ? src * ldx * 4u + (blk * 256u + lane * 4u) * 4u : kOobOffset, 0, 0);
-                    }
-                }
+                    for (int h = 0; h < 2; ++h) {                          // weights 0..131 and 124..255 of the block
+                        u32x4 xv[16];
 #pragma unroll
-                for (int b2 = 0; b2 < 2; ++b2) {
-#pragma unroll
-                    for (int t = 0; t < 16; ++t) {
-                        float* dst = stage + t * kTokStride;
-                        dst[xoff[0]] = __uint_as_float(xv[b2][t].x);
-                        dst[xoff[1]] = __uint_as_float(xv[b2][t].y);
-                        dst[xoff[2]] = __uint_as_float(xv[b2][t].z);
-                        if (xlast_ok) dst[xoff[3]] = __uint_as_float(xv[b2][t].w);
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-#pragma unroll
-                        for (int c8 = 0; c8 < 8; ++c8) {
-                            const float4 v = *reinterpret_cast<const float4*>(stage + li * kTokStride + c8 * 32 + (kq + 4 * h) * 4);
-                            breg[b2][32 * h + 4 * c8 + 0] = v.x; breg[b2][32 * h + 4 * c8 + 1] = v.y;
-                            breg[b2][32 * h + 4 * c8 + 2] = v.z; breg[b2][32 * h + 4 * c8 + 3] = v.w;
+                        for (int t = 0; t < 16; ++t) {
+                            const int m = m0 + t;
+                            const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
+                            xv[t] = __builtin_amdgcn_raw_buffer_load_b128(
+                                xrsrc, (lane < 33u && blk < bpr && src < xrows) ? src * ldx * 4u + (blk * 256u + h * 124u + lane * 4u) * 4u : kOobOffset, 0, 0);
                         }
-                    if (kq == 0) {                                         // nibbles 0..3 of a block hold its scale
-                        breg[b2][0] = 0.f; breg[b2][1] = 0.f; breg[b2][2] = 0.f; breg[b2][3] = 0.f;
-                    }
-                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                    __builtin_amdgcn_wave_barrier();
-                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                }
-                __syncthreads();                                           // every wavefront has left its staging area
-                {   // pair table from literals (see gemv_oil4.hip)
-                    const float lv_lane = level_literal(lane & 15u);
-                    const float lo_fix = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+                        if (lane < 33u) {
 #pragma unroll
-                    for (int k = 0; k < 8; ++k) {
-                        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
-                        reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
+                            for (int t = 0; t < 16; ++t)
+                                *reinterpret_cast<u32x4*>(stage + t * kTokStride + lane * 4u) = xv[t];
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                        {
+                            // LDS byte address of the value below the step of q/63; from the step on it is one float
+                            // further.  The address is made opaque so that the 64 element addresses are formed here,
+                            // next to their reads, instead of being precomputed for the whole kernel.
+                            uint32_t lo = (uint32_t)(kStageBase + wave * kStageBytes) + (li * kTokStride + (uint32_t)(gbase[h] - h * 124)) * 4u;
+                            asm volatile("" : "+v"(lo));
+                            const uint32_t thr = (uint32_t)gthr[h];
+#pragma unroll
+                            for (int sI = 0; sI < 32; ++sI) {
+                                const uint32_t a = ((uint32_t)sI >= thr ? lo + 4u : lo) + 4u * sI;
+                                const float v = *(lds_cfloat*)(uintptr_t)a;
+                                if (h == 0 && sI < 4) breg[b2][sI] = kq == 0u ? 0.f : v;        // nibbles 0..3 of a block: its scale
+                                else breg[b2][32 * h + sI] = v;
+                            }
+                        }
+                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                        __builtin_amdgcn_wave_barrier();
+                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                     }
                 }
-                __syncthreads();
             }
+            if (!table_synced) { __syncthreads(); table_synced = true; }   // the level table is complete
             // ---- main loop: groups of the tile, two blocks each -------------------------------------------
             LevelPair lv[16];
 #pragma unroll
@@ -169,19 +173,21 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
                         __builtin_amdgcn_sched_barrier(0);                 // all 16 table reads in flight before the first multiply
 #pragma unroll
                         for (int k = 0; k < 16; ++k) {
-                            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].lo * scale, breg[b2][32 * h + 2 * k], acc[g], 0, 0, 0);
-                            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].hi * scale, breg[b2][32 * h + 2 * k + 1], acc[g], 0, 0, 0);
+                            acc[g][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].lo * scale, breg[b2][32 * h + 2 * k], acc[g][0], 0, 0, 0);
+                            acc[g][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].hi * scale, breg[b2][32 * h + 2 * k + 1], acc[g][1], 0, 0, 0);
                         }
                         __builtin_amdgcn_sched_barrier(0);
                     }
                 }
             }
         }
-        // ---- tile finished: add the wavefronts' partial sums --------------------------------------------------
+        // ---- tile finished: add the wavefronts' partial sums (the staging areas are idle now) ------------------
+        __syncthreads();
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g)
-            *reinterpret_cast<float4*>(red + (((size_t)wave * kGroups + g) * 64 + lane) * 4) =
-                make_float4(acc[g][0], acc[g][1], acc[g][2], acc[g][3]);
+        for (int g = 0; g < kGroups; ++g) {
+            const v4f d = acc[g][0] + acc[g][1];
+            *reinterpret_cast<float4*>(red + (((size_t)wave * kGroups + g) * 64 + lane) * 4) = make_float4(d[0], d[1], d[2], d[3]);
+        }
         __syncthreads();
         for (uint32_t o = tid; o < kGroups * 16u * 16u; o += 512u) {
             const uint32_t rl = o & 63u, j = o >> 6;                       // row of the tile, token of the pass
@@ -212,8 +218,8 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
-    const size_t lds_bytes = 8 * (size_t)kStageBytes + 64;                // covers table (64 KB) + partial sums (32 KB)
-    static_assert(8 * kStageBytes >= kTabBytes + 8 * kGroups * 64 * 16, "staging area must cover table and partial sums");
+    const size_t lds_bytes = (size_t)kStageBase + 8 * (size_t)kStageBytes + 64;   // table, then staging areas / partial sums
+    static_assert(8 * kStageBytes >= 8 * kGroups * 64 * 16, "the staging areas must cover the partial sums");
     const uint32_t groups = ((uint32_t)w.rows + 15u) / 16u;
     uint32_t grid = (uint32_t)device_cu_count();
     if (grid > groups) grid = groups;
