@@ -316,7 +316,7 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     if (grid == 0) grid = 1;
     const uint32_t Jn = grid * G;
     const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
-    const int budget = 12 / best_cs;                               // <= 12 wave-loads in flight per wave
+    const int budget = MB >= 4 ? 3 : 12 / best_cs;                 // wave-loads in flight per wave (register budget)
     int rpw = 1;
     for (int cand : {1, 2, 3, 4, 6, 12}) if (cand <= budget) { rpw = cand; if ((uint32_t)cand >= max_rows) break; }
     p->cs = best_cs; p->rpw = rpw; p->maxt = 512;
@@ -345,9 +345,12 @@ int dispatch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipSt
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || M > 16) return 1;
     Oil4Plan p;
-    const int MB = M == 1 ? 1 : 2;
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) return 1;
-    return MB == 1 ? dispatch<1>(w, d_x, d_y, M, s, p) : dispatch<2>(w, d_x, d_y, M, s, p);
+    const int MB = M == 1 ? 1 : (M == 2 ? 2 : 4);
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) {
+        if (MB != 4 || !make_plan((uint32_t)w.rows, (uint32_t)w.cols, 2, 8, &p)) return 1;
+        return dispatch<2>(w, d_x, d_y, M, s, p);
+    }
+    return MB == 1 ? dispatch<1>(w, d_x, d_y, M, s, p) : MB == 2 ? dispatch<2>(w, d_x, d_y, M, s, p) : dispatch<4>(w, d_x, d_y, M, s, p);
 }
 
 }  // namespace oilhip
