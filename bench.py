@@ -131,6 +131,74 @@ def time_gemvs(torch, items, xs, ys, reps):
     return e0.elapsed_time(e1) * 1e-3 / reps
 
 
+def bench_fused_layer(torch, ia, unfused_s):
+    """The same Llama-7B-shaped layer with q/k/v and gate/up stacked into one tensor each, both RMSNorms and the
+    SwiGLU product formed inside the GEMVs that consume them: 4 launches per layer instead of 7 GEMVs + glue."""
+    import numpy as np
+    from innova_amd import layers
+    L = _lib_handles(ia)
+    copies = 12                                                            # 12 x 101 MB of OIL4 payload per layer > 256 MB cache
+    sets = []
+    for c in range(copies):
+        d = {}
+        for name, (r, k) in (("qkv", (12288, 4096)), ("o", (4096, 4096)), ("gate_up", (22016, 4096)), ("down", (4096, 11008))):
+            if c == 0:
+                w = make_weights(r, k, seed=300 + len(name))
+                d[name] = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+            else:
+                d[name] = sets[0][name + "_host"]
+        sets.append({**{n: ia.DeviceWeights.from_blocks(*d[n], *shape) for n, shape in
+                        (("qkv", (12288, 4096)), ("o", (4096, 4096)), ("gate_up", (22016, 4096)), ("down", (4096, 11008)))},
+                     **{n + "_host": d[n] for n in d}})
+    x = torch.randn(1, 4096, device="cuda")
+    wn = torch.randn(4096, device="cuda") * 0.1
+    xn = torch.empty_like(x)
+    qkv = torch.empty((1, 12288), device="cuda")
+    att = torch.randn(1, 4096, device="cuda")
+    o = torch.empty((1, 4096), device="cuda")
+    y = torch.empty((1, 4096), device="cuda")
+    scratch = torch.empty(3 * 11008 + 4096, device="cuda")
+    st = lambda: ia._lib.current_stream()  # noqa: E731
+
+    def layer(sx):
+        ia._lib.check(L.oilhip_gemv_rmsnorm_f32(sx["qkv"].handle, x.data_ptr(), wn.data_ptr(), qkv.data_ptr(), 1, None, st()))
+        sx["o"].gemv(att, out=o)                                         # attention itself is not modelled
+        ia._lib.check(L.oilhip_mlp_step_f32(sx["gate_up"].handle, sx["down"].handle, o.data_ptr(), wn.data_ptr(),
+                                            y.data_ptr(), 1, scratch.data_ptr(), st()))
+
+    for sx in sets:
+        layer(sx)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            for sx in sets:
+                layer(sx)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(20):
+            graph.replay()
+        e1.record(stream)
+        torch.cuda.synchronize()
+    t = e0.elapsed_time(e1) * 1e-3 / (20 * copies)
+    for sx in sets:
+        for n in ("qkv", "o", "gate_up", "down"):
+            sx[n].close()
+    payload = (12288 + 4096 + 22016) * 4096 // 2 + 4096 * 11008 // 2
+    return {"fused_layer_us": round(t * 1e6, 1), "fused_layer_GBps": round(payload / t / 1e9, 1),
+            "decode_tok_per_s_7B_fused_layers": round(1.0 / (32 * t), 1),
+            "decode_tok_per_s_7B_unfused_gemvs": round(1.0 / unfused_s, 1)}
+
+
+def _lib_handles(ia):
+    return ia._lib.lib()
+
+
 def bench_oil8(torch, ia):
     """OIL8 M=1, K=N=4096: block-codec GEMV and the flat kernel::oil8_gemm form (16.8 MB of codes each)."""
     import numpy as np
@@ -369,6 +437,7 @@ def main():
         per_layer = 4 * t_qkvo + 2 * sec + s_d
         extra["qkvo_4096x4096_M1_GBps"] = round(pq.size / t_qkvo / 1e9, 1)
         extra["decode_tok_per_s_7B_weight_gemvs_only"] = round(1.0 / (32 * per_layer), 1)
+        extra.update(bench_fused_layer(torch, ia, 32 * per_layer))
         extra.update(bench_oil8(torch, ia))
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))

@@ -213,6 +213,33 @@ int oilhip_engine_dequant(int bits, const uint8_t* d_idx, const float* d_cb, int
 int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const float* d_scales, int64_t block,
                              float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
 
+/* ------------------------------------------------------------ decode-step pieces
+ * oilhip_weights_stack_rows : several uploaded tensors of one format, width and regular block layout as one
+ *                             tensor of their rows in order (device copy; the parts stay valid).  Lets the gate
+ *                             and up projections (or q, k, v) run as one launch.  No reference counterpart: the
+ *                             reference walks each tensor separately.
+ * oilhip_rmsnorm_f32        : Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:39-44) over `rows` rows of
+ *                             n floats: out = x * r * (1 + w), r = 1 / sqrt(mean(x^2) + 1e-6)
+ * oilhip_gemv_rmsnorm_f32   : y[M][rows] = W . rmsnorm(x; normw), the rmsnorm + gemm pair in front of every projection
+ *                             (:484-486 attention input, :611-614 MLP input).  With M = 1 and an OIL4 tensor the
+ *                             norm is formed while the GEMV stages x (one launch, d_xn unused and may be NULL);
+ *                             otherwise d_xn[M][cols] receives the normalised rows and the GEMV reads them.
+ * oilhip_mlp_step_f32       : Qwen35Engine::mlp_step (:611-621): y[M][D] = down(siluf(gate x) * up x), gate_up = the
+ *                             gate and up projections stacked (2F x D, gate rows first), down = D x F.  A non-NULL
+ *                             d_normw applies rmsnorm(x; d_normw) first, as the caller of mlp_step does.
+ *                             d_scratch holds M * (3*F + D) floats.  With M = 1 and OIL4 tensors the norm rides on
+ *                             the first GEMV and the SwiGLU product on the second: two launches for the whole step.
+ * oilhip_embed_rows_f32     : the embedding lookup of Qwen35Engine::append_token (:756-760, decode_block :17-28):
+ *                             rows d_ids[i] of a quantized [vocab][cols] tensor decoded to d_out[i][cols]; ids outside
+ *                             the table give zero rows */
+int oilhip_weights_stack_rows(const oilhip_weights* const* parts, int n, oilhip_weights** out);
+int oilhip_rmsnorm_f32(const float* d_x, const float* d_w, int n, int rows, float* d_out, void* stream);
+int oilhip_gemv_rmsnorm_f32(const oilhip_weights* w, const float* d_x, const float* d_normw, float* d_y, int M, float* d_xn,
+                            void* stream);
+int oilhip_mlp_step_f32(const oilhip_weights* gate_up, const oilhip_weights* down, const float* d_x, const float* d_normw,
+                        float* d_y, int M, float* d_scratch, void* stream);
+int oilhip_embed_rows_f32(const oilhip_weights* w, const int32_t* d_ids, int n, float* d_out, void* stream);
+
 /* ------------------------------------------------------------ mixture of experts
  * oilhip_moe_route   : moe::softmax_with_topk (include/oil/moe_variants.h:693, src/moe_variants.cpp:97-134).
  *                      Host arrays: logits/probs [T][E], indices (int64) and weights [T][k]; weights are the

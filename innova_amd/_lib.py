@@ -59,6 +59,11 @@ _SIGNATURES = {
                                     vp, vp, C.c_uint32]),
     "oilhip_engine_dequant": (C.c_int, [C.c_int, vp, vp, C.c_int64, vp, C.c_int64, vp, vp]),
     "oilhip_engine_dense_gemm": (C.c_int, [C.c_int, vp, vp, vp, C.c_int64, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
+    "oilhip_weights_stack_rows": (C.c_int, [vp, C.c_int, C.POINTER(vp)]),
+    "oilhip_rmsnorm_f32": (C.c_int, [vp, vp, C.c_int, C.c_int, vp, vp]),
+    "oilhip_gemv_rmsnorm_f32": (C.c_int, [vp, vp, vp, vp, C.c_int, vp, vp]),
+    "oilhip_mlp_step_f32": (C.c_int, [vp, vp, vp, vp, vp, C.c_int, vp, vp]),
+    "oilhip_embed_rows_f32": (C.c_int, [vp, vp, C.c_int, vp, vp]),
     "oilhip_moe_route": (C.c_int, [vp, C.c_int64, C.c_int64, C.c_int64, vp, vp, vp]),
     "oilhip_moe_workspace_bytes": (C.c_size_t, [C.c_int64, C.c_int64, C.c_int64, C.c_int64]),
     "oilhip_moe_forward": (C.c_int, [vp, vp, vp, C.c_int, vp, vp, vp, C.c_int64, C.c_int64, vp, vp, C.c_size_t,

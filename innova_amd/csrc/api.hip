@@ -218,6 +218,53 @@ int oilhip_weights_destroy(oilhip_weights* w) {
     return OILHIP_OK;
 }
 
+// Several tensors of the same width and regular layout as one tensor of their rows, one after the other
+// (device-to-device copy of the payloads; the parts stay valid).
+int oilhip_weights_stack_rows(const oilhip_weights* const* parts, int n, oilhip_weights** out) {
+    if (!parts || n <= 0 || !out) return fail(OILHIP_E_ARG, "stack_rows: bad arguments");
+    *out = nullptr;
+    const oilhip_weights* p0 = parts[0];
+    uint64_t rows = 0, nblocks = 0, bytes = 0, algo = 0;
+    for (int i = 0; i < n; ++i) {
+        const oilhip_weights* p = parts[i];
+        if (!p || !p->uniform_stride || p->uniform_fmt != p0->uniform_fmt || p->uniform_stride != p0->uniform_stride ||
+            p->cols != p0->cols || !p->all_full || p->uniform_cb != p0->uniform_cb || p->uniform_idx != p0->uniform_idx)
+            return fail(OILHIP_E_ARG, "stack_rows: parts must share one format, width and regular block layout");
+        rows += p->rows; nblocks += p->nblocks; bytes += (uint64_t)p->nblocks * p->uniform_stride; algo += p->payload_bytes;
+    }
+    if (nblocks > 0xFFFFFFFFull || bytes / 16 > 0xFFFFFFFFull) return fail(OILHIP_E_ARG, "stack_rows: too large");
+    auto* w = new (std::nothrow) oilhip_weights();
+    if (!w) return fail(OILHIP_E_NOMEM, "host allocation failed");
+    auto bail = [&](hipError_t e, const char* what) {
+        oilhip_weights_destroy(w);
+        return fail(e == hipErrorOutOfMemory ? OILHIP_E_NOMEM : OILHIP_E_DEVICE, std::string(what) + ": " + hipGetErrorString(e));
+    };
+    hipError_t e;
+    if ((e = hipGetDevice(&w->device)) != hipSuccess) return bail(e, "hipGetDevice");
+    w->alloc_bytes = bytes + 64;
+    if ((e = hipMalloc(&w->d_payload, w->alloc_bytes)) != hipSuccess) return bail(e, "hipMalloc(payload)");
+    if ((e = hipMemset(w->d_payload + bytes, 0, 64)) != hipSuccess) return bail(e, "hipMemset");
+    uint64_t off = 0;
+    for (int i = 0; i < n; ++i) {
+        const uint64_t nb = (uint64_t)parts[i]->nblocks * parts[i]->uniform_stride;
+        if ((e = hipMemcpy(w->d_payload + off, parts[i]->d_payload + parts[i]->uniform_base, nb, hipMemcpyDeviceToDevice)) != hipSuccess)
+            return bail(e, "hipMemcpy(payload)");
+        off += nb;
+    }
+    std::vector<DevBlock> db((size_t)nblocks);
+    for (uint64_t b = 0; b < nblocks; ++b)
+        db[(size_t)b] = DevBlock{(uint32_t)(b * p0->uniform_stride / 16), p0->uniform_idx, 256u, (uint16_t)p0->uniform_cb, (uint8_t)p0->uniform_fmt, 0};
+    if ((e = hipMalloc(&w->d_blocks, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(blocks)");
+    if ((e = hipMemcpy(w->d_blocks, db.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
+        return bail(e, "hipMemcpy(blocks)");
+    w->payload_bytes = algo;
+    w->rows = rows; w->cols = p0->cols; w->nblocks = (uint32_t)nblocks;
+    w->uniform_fmt = p0->uniform_fmt; w->all_full = true;
+    w->uniform_stride = p0->uniform_stride; w->uniform_cb = p0->uniform_cb; w->uniform_idx = p0->uniform_idx; w->uniform_base = 0;
+    *out = w;
+    return OILHIP_OK;
+}
+
 int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols, uint32_t* nblocks,
                         uint64_t* payload_bytes, int* uniform_fmt) {
     if (!w) return fail(OILHIP_E_ARG, "null weights");

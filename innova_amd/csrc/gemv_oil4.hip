@@ -42,9 +42,14 @@ constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 3
 
 // CS: column sets (wave-loads) per row and wave; RPW: rows per chunk, all loads of
 // a chunk in flight at once; MB: activation rows handled together; MAXT: workgroup size bound.
-template <int CS, int RPW, int MB, int MAXT>
+// XF = 1: the activation row is not x itself but silu(h[k]) * h[cols + k] of a row h of 2*cols floats (the gate and
+// up projections of an MLP step, Qwen35Engine::mlp_step, src/adapters/tools/qwen35_engine.cpp:611-621), formed
+// while x is staged, so the SwiGLU product never makes a round trip through memory.
+// XF = 2: the activation row is rmsnorm(x) = x * r * (1 + xw), r = 1 / sqrt(mean(x^2) + 1e-6) (rmsnorm, same file :39-44):
+// x * (1 + xw) is staged, every workgroup forms r from the whole row it loads anyway, and r scales the dot products.
+template <int CS, int RPW, int MB, int MAXT, int XF = 0>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(2, 2)))
-gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, float* __restrict__ y,
+gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const float* __restrict__ xw, float* __restrict__ y,
                  uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M,
                  uint32_t rg_base, uint32_t rg_rem) {
     constexpr int NL = CS * RPW;      // wave-loads per chunk
@@ -76,17 +81,53 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
     // Nothing that waits on vector memory may follow the weight loads before their use:
     // loads return in order, so it would wait for every weight byte.
     constexpr int XPT = 4;            // float4 pieces of x fetched up front per thread
+    constexpr uint32_t XW = XF == 1 ? 2u : 1u;                                // input floats per activation
+    const __amdgpu_buffer_rsrc_t nrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(XF == 2 ? xw : x), 0, (int)(cols * 4u), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(x + (size_t)m0 * cols), 0, (int)((uint32_t)(M - m0 < MB ? M - m0 : MB) * cols * 4u), 0x00020000);
-    u32x4 xpre[MB][XPT];
+        (void*)(x + (size_t)m0 * cols * XW), 0, (int)((uint32_t)(M - m0 < MB ? M - m0 : MB) * cols * XW * 4u), 0x00020000);
+    u32x4 xpre[MB][XPT], xup[XF ? MB : 1][XF ? XPT : 1];
 #pragma unroll
     for (int u = 0; u < XPT; ++u) {
         const uint32_t d4 = tid + u * 512u;                             // float4 index into the padded row
 #pragma unroll
-        for (int m = 0; m < MB; ++m)
-            xpre[m][u] = __builtin_amdgcn_raw_buffer_load_b128(
-                xrsrc, (d4 * 4u < cols && m0 + m < M) ? d4 * 16u + m * cols * 4u : kOobOffset, 0, 0);
+        for (int m = 0; m < MB; ++m) {
+            const uint32_t off = (d4 * 4u < cols && m0 + m < M) ? d4 * 16u + m * cols * XW * 4u : kOobOffset;
+            xpre[m][u] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 0, 0);
+            if (XF == 1) xup[m][u] = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + cols * 4u, 0, 0);
+            if (XF == 2) xup[m][u] = __builtin_amdgcn_raw_buffer_load_b128(nrsrc, d4 * 4u < cols ? d4 * 16u : kOobOffset, 0, 0);
+        }
     }
+    auto swiglu4 = [&](const u32x4& g, const u32x4& up) {                     // (g * sigmoid(g)) * up, sigmoid = 1 / (1 + exp(-g))
+        u32x4 r;
+        const uint32_t gg[4] = {g.x, g.y, g.z, g.w}, uu[4] = {up.x, up.y, up.z, up.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float v = __uint_as_float(gg[k]);
+            o[k] = __float_as_uint((v * __builtin_amdgcn_rcpf(1.0f + __expf(-v))) * __uint_as_float(uu[k]));
+        }
+        r.x = o[0]; r.y = o[1]; r.z = o[2]; r.w = o[3];
+        return r;
+    };
+    float ssq = 0.0f;                                                         // XF = 2: this thread's share of sum(x^2)
+    auto norm4 = [&](const u32x4& g, const u32x4& nw) {                       // x * (1 + xw), and x^2 into ssq
+        u32x4 r;
+        const uint32_t gg[4] = {g.x, g.y, g.z, g.w}, ww[4] = {nw.x, nw.y, nw.z, nw.w};
+        uint32_t o[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const float v = __uint_as_float(gg[k]);
+            ssq = __fmaf_rn(v, v, ssq);
+            o[k] = __float_as_uint(v * (1.0f + __uint_as_float(ww[k])));
+        }
+        r.x = o[0]; r.y = o[1]; r.z = o[2]; r.w = o[3];
+        return r;
+    };
+    auto transform4 = [&](const u32x4& g, const u32x4& b) {
+        if constexpr (XF == 1) return swiglu4(g, b);
+        else if constexpr (XF == 2) return norm4(g, b);
+        else return g;
+    };
     const uint32_t lane_off = (slab * CS * 8u + (lane >> 3)) * 128u + lp * 16u;   // first column set of this lane
     // The 64 KB pair table is written while the weight loads queue up: float4 number e of the
     // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + 512*k,
@@ -155,16 +196,36 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
         const uint32_t d4 = tid + u * 512u;
         if (d4 * 4u < cols) {
 #pragma unroll
-            for (int m = 0; m < MB; ++m) scatter4(d4, xpre[m][u], m);
+            for (int m = 0; m < MB; ++m) scatter4(d4, transform4(xpre[m][u], xup[XF ? m : 0][XF ? u : 0]), m);
         }
     }
     for (uint32_t d4 = tid + XPT * 512u; d4 * 4u < cols; d4 += 512u) {    // rows wider than XPT*4*workgroup
 #pragma unroll
-        for (int m = 0; m < MB; ++m)
-            scatter4(d4, __builtin_amdgcn_raw_buffer_load_b128(
-                xrsrc, (m0 + m < M) ? d4 * 16u + m * cols * 4u : kOobOffset, 0, 0), m);
+        for (int m = 0; m < MB; ++m) {
+            const uint32_t off = (m0 + m < M) ? d4 * 16u + m * cols * XW * 4u : kOobOffset;
+            const u32x4 g = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off, 0, 0);
+            if (XF == 1) scatter4(d4, swiglu4(g, __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + cols * 4u, 0, 0)), m);
+            else if (XF == 2) scatter4(d4, norm4(g, __builtin_amdgcn_raw_buffer_load_b128(nrsrc, d4 * 16u, 0, 0)), m);
+            else scatter4(d4, g, m);
+        }
+    }
+    float* ssq_part = red + (size_t)G * RPW * MB * S;                         // 8 floats past the slab partials
+    if (XF == 2) {
+        float v = ssq;
+        v += dpp_quad_xor1(v);
+        v += dpp_quad_xor2(v);
+        v += dpp_half_mirror(v);
+        v += dpp_row_mirror(v);
+        v += dpp_row_bcast15(v);
+        v += dpp_row_bcast31(v);
+        if (lane == 63) ssq_part[wave] = v;
     }
     __syncthreads();
+    float yscale = 1.0f;
+    if (XF == 2) {
+        const float tot = ((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) + ((ssq_part[4] + ssq_part[5]) + (ssq_part[6] + ssq_part[7]));
+        yscale = 1.0f / sqrtf(tot / (float)cols + 1e-6f);
+    }
 
     // ---- this lane's activations: 8 float4 per column set ------------------------------------
     float xr[MB][CS][32];
@@ -239,7 +300,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
                 for (int it = 0; it < RPW; ++it)
 #pragma unroll
                     for (int m = 0; m < MB; ++m)
-                        if (cbase + it < r1 && m0 + m < M) y[(size_t)(m0 + m) * rows + cbase + it] = part[m][it];
+                        if (cbase + it < r1 && m0 + m < M) y[(size_t)(m0 + m) * rows + cbase + it] = XF == 2 ? part[m][it] * yscale : part[m][it];
             }
             continue;
         }
@@ -261,7 +322,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
                 const float* pr = red + (size_t)o * S;
                 float s = 0.0f;
                 for (uint32_t k = 0; k < S; ++k) s += pr[k];
-                y[(size_t)(m0 + m) * rows + r] = s;
+                y[(size_t)(m0 + m) * rows + r] = XF == 2 ? s * yscale : s;
             }
         }
         __syncthreads();
@@ -275,10 +336,10 @@ struct Oil4Plan {
     size_t lds_bytes;
 };
 
-template <int CS, int RPW, int MB, int MAXT>
-int launch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
+template <int CS, int RPW, int MB, int MAXT, int XF = 0>
+int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
     static bool attr_done = false;
-    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT>;
+    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT, XF>;
     if (!attr_done) {
         OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
@@ -286,7 +347,7 @@ int launch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStre
     }
     const uint32_t J = p.grid * p.G;
     for (int m0 = 0; m0 < M; m0 += MB) {
-        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_y,
+        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_xw, d_y,
                            (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M,
                            (uint32_t)w.rows / J, (uint32_t)w.rows % J);
         OILHIP_HIP(hipGetLastError());
@@ -327,10 +388,10 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     return p->lds_bytes <= (size_t)kMaxLds && S * G <= 8;
 }
 
-template <int MB>
-int dispatch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
+template <int MB, int XF = 0>
+int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
 #define OIL4_CASE(CS_, RPW_) \
-    if (p.cs == CS_ && p.rpw == RPW_) return launch<CS_, RPW_, MB, 512>(w, d_x, d_y, M, s, p);
+    if (p.cs == CS_ && p.rpw == RPW_) return launch<CS_, RPW_, MB, 512, XF>(w, d_x, d_xw, d_y, M, s, p);
     OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
     if constexpr (MB == 1) {
         OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)
@@ -348,9 +409,26 @@ int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int 
     const int MB = M == 1 ? 1 : (M == 2 ? 2 : 4);
     if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) {
         if (MB != 4 || !make_plan((uint32_t)w.rows, (uint32_t)w.cols, 2, 8, &p)) return 1;
-        return dispatch<2>(w, d_x, d_y, M, s, p);
+        return dispatch<2>(w, d_x, nullptr, d_y, M, s, p);
     }
-    return MB == 1 ? dispatch<1>(w, d_x, d_y, M, s, p) : MB == 2 ? dispatch<2>(w, d_x, d_y, M, s, p) : dispatch<4>(w, d_x, d_y, M, s, p);
+    return MB == 1 ? dispatch<1>(w, d_x, nullptr, d_y, M, s, p)
+         : MB == 2 ? dispatch<2>(w, d_x, nullptr, d_y, M, s, p) : dispatch<4>(w, d_x, nullptr, d_y, M, s, p);
+}
+
+// y = W . (silu(h[0..K)) * h[K..2K)) for one activation row h of 2K floats.  Returns 1 when the shape is not covered.
+int launch_gemv_oil4_swiglu(const oilhip_weights& w, const float* d_h, float* d_y, hipStream_t s) {
+    if (w.rows > 0x7FFFFFFFull || w.cols > 0x3FFFFFFFull) return 1;
+    Oil4Plan p;
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, 8, &p)) return 1;
+    return dispatch<1, 1>(w, d_h, nullptr, d_y, 1, s, p);
+}
+
+// y = W . rmsnorm(x; xw) for one activation row.  Returns 1 when the shape is not covered.
+int launch_gemv_oil4_rmsnorm(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, hipStream_t s) {
+    if (w.rows > 0x7FFFFFFFull || w.cols > 0x3FFFFFFFull) return 1;
+    Oil4Plan p;
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, 8, &p)) return 1;
+    return dispatch<1, 2>(w, d_x, d_xw, d_y, 1, s, p);
 }
 
 }  // namespace oilhip

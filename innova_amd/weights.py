@@ -45,6 +45,15 @@ class DeviceWeights:
         payload, blocks = quantize_tensor(w, fmts)
         return cls.from_blocks(payload, blocks, rows, cols)
 
+    @classmethod
+    def stack_rows(cls, parts) -> "DeviceWeights":
+        """Tensors of one format, width and regular block layout as one tensor of their rows (device copy);
+        gate + up or q + k + v then run as a single launch."""
+        arr = (C.c_void_p * len(parts))(*[p.handle for p in parts])
+        h = C.c_void_p(0)
+        _lib.check(_lib.lib().oilhip_weights_stack_rows(arr, len(parts), C.byref(h)))
+        return cls(h.value, sum(p.rows for p in parts), parts[0].cols)
+
     # ---- lifetime -------------------------------------------------------------
     def close(self) -> None:
         if self._h:

@@ -351,3 +351,24 @@ def engine_dense_gemm(kind: int, A, B, M: int, N: int, K: int, scales=None, bloc
         fn(C.c_int(kind), C.c_void_p(A.ctypes.data), C.c_void_p(B.ctypes.data), C.c_size_t(B.nbytes), C.c_void_p(sc.ctypes.data),
            C.c_int64(sc.size), C.c_int64(block), C.c_void_p(out.ctypes.data), C.c_int64(M), C.c_int64(N), C.c_int64(K))
     return out
+
+
+# ---------------------------------------------------------------- decode-step pieces
+def rmsnorm(x, w) -> np.ndarray:
+    x = np.ascontiguousarray(x, np.float32)
+    w = np.ascontiguousarray(w, np.float32)
+    out = np.zeros_like(x)
+    for r in range(x.reshape(-1, w.size).shape[0]):
+        xr = np.ascontiguousarray(x.reshape(-1, w.size)[r])
+        o = np.zeros(w.size, np.float32)
+        lib().orc_rmsnorm(C.c_void_p(xr.ctypes.data), C.c_void_p(w.ctypes.data), C.c_int(w.size), C.c_void_p(o.ctypes.data))
+        out.reshape(-1, w.size)[r] = o
+    return out
+
+
+def swiglu(g, u) -> np.ndarray:
+    g = np.ascontiguousarray(g, np.float32)
+    u = np.ascontiguousarray(u, np.float32)
+    h = np.zeros_like(g)
+    lib().orc_swiglu(C.c_void_p(g.ctypes.data), C.c_void_p(u.ctypes.data), C.c_int64(g.size), C.c_void_p(h.ctypes.data))
+    return h

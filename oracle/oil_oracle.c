@@ -1086,3 +1086,18 @@ void orc_engine_dense_gemm(int kind, const float* A, const void* B, const float*
             }
         }
 }
+
+/* ------------------------------------------------------------------ decode-step pieces */
+void orc_rmsnorm(const float* x, const float* w, int n, float* out) {
+    float s = 0.0f;
+    for (int i = 0; i < n; ++i) s = fmaf(x[i], x[i], s);
+    const float r = 1.0f / sqrtf(s / (float)n + 1e-6f);
+    for (int i = 0; i < n; ++i) out[i] = x[i] * r * (1.0f + w[i]);
+}
+
+void orc_swiglu(const float* g, const float* u, int64_t n, float* h) {
+    for (int64_t i = 0; i < n; ++i) {
+        const float v = g[i];
+        h[i] = (v * (1.0f / (1.0f + expf(-v)))) * u[i];
+    }
+}

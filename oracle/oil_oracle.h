@@ -143,6 +143,15 @@ void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
 void orc_engine_dense_gemm(int kind, const float* A, const void* B, const float* scales, int64_t block,
                            float* C, int64_t M, int64_t N, int64_t K);
 
+/* Decode-step pieces of Qwen35Engine (src/adapters/tools/qwen35_engine.cpp), FP32 in the reference's order with the
+ * multiply-adds fused as the -mfma build does:
+ * orc_rmsnorm  (:39-44): out = x * r * (1 + w), r = 1 / sqrtf(sum(x^2) / n + 1e-6f)
+ * orc_swiglu   (:31,37,617): h[k] = (g[k] * (1 / (1 + expf(-g[k])))) * u[k]
+ * (mlp_step :611-621 is orc_block_gemm of gate and up, orc_swiglu, orc_block_gemm of down; the embedding lookup
+ * :756-760 is orc_dequant_blocks over the row's blocks.) */
+void orc_rmsnorm(const float* x, const float* w, int n, float* out);
+void orc_swiglu(const float* g, const float* u, int64_t n, float* h);
+
 /* Mixture-of-experts routing and dispatch.
  * orc_softmax_topk: softmax_with_topk (src/moe_variants.cpp:97-134): max-subtracted expf softmax in
  *   FP32, probabilities scaled by 1/sum, top-k by libstdc++'s partial_sort with a > comparator
