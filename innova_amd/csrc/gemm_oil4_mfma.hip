@@ -38,11 +38,17 @@ constexpr int kTabBytes = 256 * 64 * 4;     // pair table: byte v, lane copy c a
 constexpr int BK = 64;                      // columns per step (a quarter of a block)
 constexpr int LDK = BK + 8;                 // LDS row pitch in bf16: 144 bytes keeps 16-byte reads of 16 rows on distinct banks
 
-__device__ __forceinline__ float level_literal(uint32_t i) {      // kOIL4Levels, src/block_codec.cpp:18-23
-    const float mag = (i == 7 || i == 8) ? 0.1260f : (i == 6 || i == 9) ? 0.3976f : (i == 5 || i == 10) ? 0.6508f
-                    : (i == 4 || i == 11) ? 0.9275f : (i == 3 || i == 12) ? 1.2392f : (i == 2 || i == 13) ? 1.5995f
-                    : (i == 1 || i == 14) ? 2.0522f : 2.7178f;
-    return i < 8 ? -mag : mag;
+__device__ __forceinline__ float level_literal(uint32_t i) {      // kOIL4Levels, src/block_codec.cpp:18-23; selects only
+    const uint32_t m = i < 8u ? 7u - i : i - 8u;
+    uint32_t bits = __float_as_uint(0.1260f);
+    bits = m == 1u ? __float_as_uint(0.3976f) : bits;
+    bits = m == 2u ? __float_as_uint(0.6508f) : bits;
+    bits = m == 3u ? __float_as_uint(0.9275f) : bits;
+    bits = m == 4u ? __float_as_uint(1.2392f) : bits;
+    bits = m == 5u ? __float_as_uint(1.5995f) : bits;
+    bits = m == 6u ? __float_as_uint(2.0522f) : bits;
+    bits = m == 7u ? __float_as_uint(2.7178f) : bits;
+    return __uint_as_float(bits | (i < 8u ? 0x80000000u : 0u));
 }
 
 // X (bf16 bit patterns, [M][K]) -> X' ([Mpad][K], rows >= M zero), columns in nibble order.

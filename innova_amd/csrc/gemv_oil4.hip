@@ -28,8 +28,10 @@
 #include "common.h"
 #include "oil4_lds.h"
 
-#ifndef OILHIP_OIL4_PREFETCH
-#define OILHIP_OIL4_PREFETCH 6
+#ifndef OILHIP_PFA
+#define OILHIP_PFA 3
+#define OILHIP_PFB 6
+#define OILHIP_PFC 6
 #endif
 
 namespace oilhip {
@@ -37,7 +39,6 @@ namespace {
 
 using namespace oil4;
 
-constexpr int kPrefetch = OILHIP_OIL4_PREFETCH;   // wave-loads in flight per wavefront
 constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 32 so that neighbouring blocks start 32 banks apart
 
 // CS: column sets (wave-loads) per row and wave; RPW: rows per chunk, all loads of
@@ -47,11 +48,11 @@ constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 3
 // while x is staged, so the SwiGLU product never makes a round trip through memory.
 // XF = 2: the activation row is rmsnorm(x) = x * r * (1 + xw), r = 1 / sqrt(mean(x^2) + 1e-6) (rmsnorm, same file :39-44):
 // x * (1 + xw) is staged, every workgroup forms r from the whole row it loads anyway, and r scales the dot products.
-template <int CS, int RPW, int MB, int MAXT, int XF = 0>
+template <int CS, int RPW, int MB, int MAXT, int XF = 0, bool ROLL = false>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const float* __restrict__ xw, float* __restrict__ y,
                  uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M,
-                 uint32_t rg_base, uint32_t rg_rem) {
+                 uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups) {
     constexpr int NL = CS * RPW;      // wave-loads per chunk
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
@@ -60,8 +61,9 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     float* xs = reinterpret_cast<float*>(lds + kTabBytes);                    // [MB][nblk][8 c][8 lp][4 e] (+32 pad), nibble order
     float* red = xs + (size_t)MB * xstride;                                   // [G][RPW][MB][S]
 
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t slab = wave % S, grp = wave / S;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));      // uniform: scalar registers
+    const uint32_t grp = (wave_groups >> (4u * wave)) & 15u, slab = wave - grp * S;         // wave / S, wave % S
     const uint32_t bpr = cols >> 8;
     const uint32_t lp = lane & 7u;
 
@@ -71,11 +73,10 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     const bool working = wave < S * G;                                        // spare wavefronts only help with the prologue
     const uint32_t r0 = working ? group_begin(jg) : 0u, r1 = working ? group_begin(jg + 1) : 0u;
     const uint32_t row_bytes = bpr * 128u;
-    // buffer resource over this workgroup's rows (offsets stay below 2^31)
-    const uint32_t wg_r0 = group_begin(blockIdx.x * G);
-    const uint64_t remain = (uint64_t)(rows - wg_r0) * row_bytes;
+    // Buffer resource over this wavefront's rows only: a load of a row past r1 is out of range (zeros, no fetch)
+    // without any compare.  The host checks that a row group plus two chunks of rows stays below 2^31 bytes.
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(W + (size_t)wg_r0 * row_bytes), 0, (int)(remain < 0x80000000ull ? remain : 0x80000000ull), 0x00020000);
+        (void*)(W + (size_t)r0 * row_bytes), 0, (int)((r1 - r0) * row_bytes), 0x00020000);
 
     // ---- x first (needed soonest), then every weight load of the first chunk ----------
     // Nothing that waits on vector memory may follow the weight loads before their use:
@@ -128,34 +129,47 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         else if constexpr (XF == 2) return norm4(g, b);
         else return g;
     };
-    const uint32_t lane_off = (slab * CS * 8u + (lane >> 3)) * 128u + lp * 16u;   // first column set of this lane
+    // Byte offset of this lane inside a row for each column set; lanes past the end of the row get an offset that
+    // stays out of range whatever row offset is added.
+    uint32_t vcol[CS];
+#pragma unroll
+    for (int cs = 0; cs < CS; ++cs) {
+        const uint32_t blk = (slab * CS + cs) * 8u + (lane >> 3);
+        vcol[cs] = blk < bpr ? blk * 128u + lp * 16u : 0x80000000u;
+    }
+    // Wave-load n of a chunk: row n / CS of the chunk, column set n % CS.  About six loads per wavefront are
+    // queued before the prologue is over (the memory pipeline of a CU holds a limited number of outstanding
+    // lines; queueing more only stalls the wavefront in front of its prologue), the first three while the table
+    // is written so that the younger wavefronts get their first rows early too; the rest follow once the
+    // prologue is done, while the first ones are being consumed.
+    constexpr int PFA = NL < OILHIP_PFA ? NL : OILHIP_PFA;          // queued while the table is written
+    constexpr int PFB = NL < OILHIP_PFB ? NL : OILHIP_PFB;          // ... by the time x is staged
+    constexpr int PFC = NL < OILHIP_PFC ? NL : OILHIP_PFC;          // ... by the barrier
+    u32x4 wv[NL];
+    auto issue_load = [&](int n, uint32_t rel) {           // rel: first row of the chunk, counted from r0
+        const int it = n / CS, cs = n % CS;
+        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, 0);
+    };
     // The 64 KB pair table is written while the weight loads queue up: float4 number e of the
     // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + 512*k,
     // k = 0..7, so its low nibble (tid >> 4) & 15 is fixed and its high nibble is (tid >> 8) + 2k,
     // uniform across the wavefront.  Levels come from literals: no memory access, no barrier.
+    // A wave-load takes the address unit of the CU a good dozen cycles and eight wavefronts queue there, so the
+    // table writes are slotted in between the loads instead of after them.
+    issue_load(0, 0u);
+    __builtin_amdgcn_sched_barrier(0);
     const float lv_lane = level_literal(lane & 15u);                          // lane i holds level[i & 15]
-    const float lo_fix = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
-    auto table_chunk = [&](int k) {
-        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
+    const float lo_fix = level_literal((tid >> 4) & 15u);
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        if (k + 1 < PFA) issue_load(k + 1, 0u);
+        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((wave >> 2) + 2u * k)));
         reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
-    };
-    // Wave-load n of a chunk: row cbase + n / CS, column set n % CS.  Only PF loads are queued up
-    // front (the memory pipeline of a CU holds a limited number of outstanding lines; queueing
-    // more only stalls the wavefront in front of its prologue); the rest follow once the
-    // prologue is done, while the first PF are being consumed.
-    constexpr int PF = NL < kPrefetch ? NL : kPrefetch;
-    u32x4 wv[NL];
-    auto issue_load = [&](int n, uint32_t cbase) {
-        const int it = n / CS, cs = n % CS;
-        const uint32_t r = cbase + it;
-        const bool ok = (slab * CS + cs) * 8u + (lane >> 3) < bpr && r < r1;
-        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(
-            rsrc, ok ? (r - wg_r0) * row_bytes + lane_off + cs * 1024u : kOobOffset, 0, 0);
-    };
+        __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
-    for (int n = 0; n < PF; ++n) issue_load(n, r0);
-#pragma unroll
-    for (int k = 0; k < 8; ++k) table_chunk(k);
+    for (int n = (PFA < 9 ? PFA : 9); n < PFB; ++n) issue_load(n, 0u);
+    __builtin_amdgcn_sched_barrier(0);
 
     // ---- x into LDS in nibble order -------------------------------------------------------------
     // Weight i of a block sits at nibble p = i - i/64 + 4 (slots i % 64 == 63 own no nibble); lane
@@ -209,6 +223,8 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
             else scatter4(d4, g, m);
         }
     }
+#pragma unroll
+    for (int n = PFB; n < PFC; ++n) issue_load(n, 0u);
     float* ssq_part = red + (size_t)G * RPW * MB * S;                         // 8 floats past the slab partials
     if (XF == 2) {
         float v = ssq;
@@ -243,20 +259,29 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
 
     const uint32_t lanebase = (lane & 31u) * 8u;          // byte offset of this lane's table copy
 
+#pragma unroll
+    for (int n = PFC; n < NL; ++n) issue_load(n, 0u);     // rest of the first chunk
     for (uint32_t ch = 0; ch < nchunks; ++ch) {
         const uint32_t cbase = r0 + ch * RPW;
-        if (ch > 0) {
+        if (!ROLL && ch > 0) {
 #pragma unroll
-            for (int n = 0; n < PF; ++n) issue_load(n, cbase);
+            for (int n = 0; n < NL; ++n) issue_load(n, ch * RPW);
         }
-#pragma unroll
-        for (int n = PF; n < NL; ++n) issue_load(n, cbase);
         float part[MB][RPW];                              // per-lane partial of each row, block scales applied
         LevelPair cur[16];
         lookup_load(wv[0], lanebase, cur);
 #pragma unroll
         for (int n = 0; n < NL; ++n) {
             const int it = n / CS, cs = n % CS;
+            // The two wavefronts of a SIMD are served oldest first; left alone the older one runs ahead and the
+            // younger finishes its rows on its own.  Priority falls with progress, so whichever is behind goes first.
+            if (!ROLL && (n == 0 || (n * 4) / NL != ((n - 1) * 4) / NL)) {
+                const int pr = 3 - (n * 4) / NL;
+                if (pr == 3) __builtin_amdgcn_s_setprio(3);
+                else if (pr == 2) __builtin_amdgcn_s_setprio(2);
+                else if (pr == 1) __builtin_amdgcn_s_setprio(1);
+                else __builtin_amdgcn_s_setprio(0);
+            }
             LevelPair nxt[16];
             if (n + 1 < NL) lookup_load(wv[n + 1], lanebase, nxt);    // next load's table reads fly during these FMAs
             __builtin_amdgcn_sched_barrier(0);                        // keep them above the FMAs
@@ -278,6 +303,10 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
 #pragma unroll
                 for (int k = 0; k < 16; ++k) cur[k] = nxt[k];
             }
+            // ROLL (shapes with more than one chunk): wv[n] is free, the same wave-load of the next chunk takes its
+            // place, so NL loads stay in flight across chunks.  Issued unconditionally (past the last row the offset is
+            // out of range: zeros, no fetch), which keeps the count of outstanding loads at every wait a constant.
+            if (ROLL) issue_load(n, (ch + 1u) * RPW);
             __builtin_amdgcn_sched_barrier(0);                        // one scheduling region per wave-load
         }
         // ---- all rows of the chunk reduced over the 64 lanes together (independent chains) ----
@@ -336,20 +365,22 @@ struct Oil4Plan {
     size_t lds_bytes;
 };
 
-template <int CS, int RPW, int MB, int MAXT, int XF = 0>
+template <int CS, int RPW, int MB, int MAXT, int XF, bool ROLL>
 int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
     static bool attr_done = false;
-    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT, XF>;
+    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT, XF, ROLL>;
     if (!attr_done) {
         OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
     const uint32_t J = p.grid * p.G;
+    uint32_t wave_groups = 0;                                   // wave / S for each of the 8 wavefronts, 4 bits each
+    for (uint32_t wv = 0; wv < 8; ++wv) wave_groups |= (wv / p.S) << (4u * wv);
     for (int m0 = 0; m0 < M; m0 += MB) {
         hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_xw, d_y,
                            (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M,
-                           (uint32_t)w.rows / J, (uint32_t)w.rows % J);
+                           (uint32_t)w.rows / J, (uint32_t)w.rows % J, wave_groups);
         OILHIP_HIP(hipGetLastError());
     }
     return OILHIP_OK;
@@ -379,19 +410,33 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
     const int budget = MB >= 4 ? 3 : 12 / best_cs;                 // wave-loads in flight per wave (register budget)
     int rpw = 1;
-    for (int cand : {1, 2, 3, 4, 6, 12}) if (cand <= budget) { rpw = cand; if ((uint32_t)cand >= max_rows) break; }
+    if (max_rows <= (uint32_t)budget) {                            // one chunk: the smallest that holds every row
+        for (int cand : {1, 2, 3, 4, 6, 12}) if ((uint32_t)cand >= max_rows) { rpw = cand; break; }
+    } else {                                                       // several chunks, loads rolling from one into the next:
+        int lo = (6 + best_cs - 1) / best_cs;                      // about six wave-loads in flight are enough, more only
+        if (lo > budget) lo = budget;                              // crowd the memory pipeline; least padded row slots
+        uint32_t best_slots = ~0u;
+        for (int cand : {1, 2, 3, 4, 6, 12}) {
+            if (cand < lo || cand > budget) continue;
+            const uint32_t slots = (max_rows + cand - 1) / cand * cand;
+            if (slots < best_slots) { best_slots = slots; rpw = cand; }
+        }
+    }
     p->cs = best_cs; p->rpw = rpw; p->maxt = 512;
     p->S = S; p->G = G; p->grid = grid;
     p->nchunks = (max_rows + rpw - 1) / rpw;
     if (p->nchunks == 0) p->nchunks = 1;
     p->lds_bytes = (size_t)kTabBytes + 4ull * MB * (S * best_cs * 8 * kXsBlock) + 4ull * G * rpw * MB * S + 64;
+    if ((uint64_t)(max_rows + 2u * (uint32_t)rpw) * ((uint64_t)(cols >> 8) * 128u) >= 0x80000000ull) return false;   // per-wave buffer range
     return p->lds_bytes <= (size_t)kMaxLds && S * G <= 8;
 }
 
 template <int MB, int XF = 0>
 int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
 #define OIL4_CASE(CS_, RPW_) \
-    if (p.cs == CS_ && p.rpw == RPW_) return launch<CS_, RPW_, MB, 512, XF>(w, d_x, d_xw, d_y, M, s, p);
+    if (p.cs == CS_ && p.rpw == RPW_) \
+        return p.nchunks > 1 ? launch<CS_, RPW_, MB, 512, XF, true>(w, d_x, d_xw, d_y, M, s, p) \
+                             : launch<CS_, RPW_, MB, 512, XF, false>(w, d_x, d_xw, d_y, M, s, p);
     OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
     if constexpr (MB == 1) {
         OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)

@@ -49,10 +49,17 @@ struct LevelPair { float lo, hi; };
 
 // kOIL4Levels (src/block_codec.cpp:18-23) selected by compares on literals: no memory access.
 __device__ __forceinline__ float level_literal(uint32_t i) {
-    const float mag = (i == 7 || i == 8) ? 0.1260f : (i == 6 || i == 9) ? 0.3976f : (i == 5 || i == 10) ? 0.6508f
-                    : (i == 4 || i == 11) ? 0.9275f : (i == 3 || i == 12) ? 1.2392f : (i == 2 || i == 13) ? 1.5995f
-                    : (i == 1 || i == 14) ? 2.0522f : 2.7178f;
-    return i < 8 ? -mag : mag;
+    // selects only: a branch tree here costs the prologue a string of instruction-cache misses
+    const uint32_t m = i < 8u ? 7u - i : i - 8u;                   // magnitude index, 0 = innermost level
+    uint32_t bits = __float_as_uint(0.1260f);
+    bits = m == 1u ? __float_as_uint(0.3976f) : bits;
+    bits = m == 2u ? __float_as_uint(0.6508f) : bits;
+    bits = m == 3u ? __float_as_uint(0.9275f) : bits;
+    bits = m == 4u ? __float_as_uint(1.2392f) : bits;
+    bits = m == 5u ? __float_as_uint(1.5995f) : bits;
+    bits = m == 6u ? __float_as_uint(2.0522f) : bits;
+    bits = m == 7u ? __float_as_uint(2.7178f) : bits;
+    return __uint_as_float(bits | (i < 8u ? 0x80000000u : 0u));
 }
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
