@@ -195,6 +195,31 @@ def bench_fused_layer(torch, ia, unfused_s):
             "decode_tok_per_s_7B_unfused_gemvs": round(1.0 / unfused_s, 1)}
 
 
+def bench_tall(torch, ia):
+    """The same kernel on taller tensors of the same width (the stacked gate+up rows of a layer, an output head):
+    the per-launch set-up is amortised over more rows.  The payload is random index bytes with a fixed FP16 block
+    scale (bandwidth does not depend on the values)."""
+    import numpy as np
+    out = {}
+    rng = np.random.default_rng(5)
+    for label, rows, copies in (("stacked_gate_up_22016x4096", 22016, 14), ("head_131072x4096", 131072, 3)):
+        nb = rows * COLS // 256
+        payload = rng.integers(0, 256, nb * 128, dtype=np.uint8)
+        payload[0::128], payload[1::128] = 0x1F, 0x25                      # FP16 0x251F = 0.0200
+        blocks = np.zeros(nb, dtype=ia._lib.BLOCK_DTYPE)
+        blocks["idx_off"] = np.arange(nb, dtype=np.uint64) * 128
+        blocks["cb_off"] = blocks["idx_off"]
+        blocks["idx_bytes"], blocks["nw"], blocks["fmt"] = 128, 256, int(ia.Format.OIL4)
+        ring = Ring(ia, payload, blocks, rows, COLS, copies)
+        x = torch.randn(1, COLS, device="cuda")
+        y = torch.empty((1, rows), dtype=torch.float32, device="cuda")
+        s_t, _ = time_ring(torch, ring, x, y, 40 * copies, copies)
+        out[f"{label}_M1_us"] = round(s_t * 1e6, 2)
+        out[f"{label}_M1_GBps"] = round(ring.payload_bytes / s_t / 1e9, 1)
+        ring.close()
+    return out
+
+
 def _lib_handles(ia):
     return ia._lib.lib()
 
@@ -438,6 +463,7 @@ def main():
         extra["qkvo_4096x4096_M1_GBps"] = round(pq.size / t_qkvo / 1e9, 1)
         extra["decode_tok_per_s_7B_weight_gemvs_only"] = round(1.0 / (32 * per_layer), 1)
         extra.update(bench_fused_layer(torch, ia, 32 * per_layer))
+        extra.update(bench_tall(torch, ia))
         extra.update(bench_oil8(torch, ia))
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))
