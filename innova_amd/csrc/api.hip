@@ -290,6 +290,10 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
                                         (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
+    if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256 && M <= 4) {
+        const int rc = launch_gemv_oil8(*w, d_x, d_y, M, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
     const int rc = launch_gemv_runs(*w, d_x, d_y, M, (hipStream_t)stream);
     if (rc <= 0) return rc;
     return launch_gemv_generic(*w, d_x, d_y, M, (hipStream_t)stream);

@@ -50,6 +50,7 @@ int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
 int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+int launch_gemv_oil8(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s);

@@ -90,6 +90,39 @@ def test_oil4_multi_token_counts(rows, cols, M):
     assert err <= TOL
 
 
+# the OIL8 kernel: one and several slabs per row, rows not a multiple of the wave count, several chunks per
+# wavefront (tall tensors), every activation-row grouping, a partial last column set
+@pytest.mark.parametrize("rows,cols", [(64, 4096), (1000, 4096), (37, 11008), (300, 1024), (5000, 256), (3, 256),
+                                       (40000, 512), (4096, 4096), (130, 14336), (77, 2304)])
+@pytest.mark.parametrize("M", [1, 2, 3, 4])
+def test_oil8_fast_kernel_shapes(rows, cols, M):
+    if rows * cols > 16e6 and M > 1:
+        pytest.skip("the large shapes run once")
+    err, payload, blocks, X, want = run_case(ia.Format.OIL8, rows, cols, M, seed=3 * rows + cols + M)
+    assert err <= TOL
+
+
+def test_oil8_special_blocks():
+    """Zero blocks, underflowing scales, huge outliers, zero activations, activations with a large common offset
+    (the kernel forms sum(q x) - 127.5 sum(x), which must not lose the small difference)."""
+    rows, cols = 96, 4096
+    w = gaussian_weights(rows * cols, 177)
+    w[0:256] = 0.0
+    w[256 * 20: 256 * 21] *= np.float32(1e-7)
+    w[256 * 40: 256 * 41] *= np.float32(1e4)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL8)
+    rng = np.random.default_rng(178)
+    for offset in (0.0, 30.0):
+        X = (rng.standard_normal((2, cols)) + offset).astype(np.float32)
+        X[0, ::5] = 0.0
+        with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+            got = dw.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
+            gen = dw.gemv(torch.from_numpy(X).cuda(), general=True).cpu().numpy()
+        want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+        assert rel_l2(gen, want) <= TOL
+        assert rel_l2(got, want) <= TOL
+
+
 def test_oil4_special_blocks():
     """Zero blocks (-0.0 levels), underflowing scales, huge outliers, zero activations."""
     rows, cols = 96, 4096
