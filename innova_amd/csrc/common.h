@@ -51,6 +51,9 @@ int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, i
 // fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemv_oil8(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+// kernel::oil8_gemm form: rows of K index bytes, any 256-entry codebook; out[m*N + n] = scale * dot
+int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_act, float* d_out, int M, int N, int K, float scale,
+                      hipStream_t s);
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s);

@@ -215,6 +215,10 @@ int oilhip_flat_oil8_gemm(const uint8_t* d_idx, const float* d_cb, const float* 
                           int M, int N, int K, void* stream) {
     if (int rc = check(d_idx, d_cb, d_act, d_out, M, N, K)) return rc;
     if (M == 0 || N == 0) return OILHIP_OK;
+    if (M <= 4) {                                     // decode shapes: the register-resident kernel
+        const int rc = launch_gemv_flat8(d_idx, d_cb, d_act, d_out, M, N, K, 1.0f, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
     hipLaunchKernelGGL(flat8_kernel, dim3(N), dim3(256), 0, (hipStream_t)stream, d_idx, d_cb, d_act, d_out, M, N, K, 1.0f);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
@@ -256,6 +260,10 @@ int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb, float scale, co
                           int M, int K, int batch, void* stream) {
     if (int rc = check(d_w, d_cb, d_x, d_y, M, batch, K)) return rc;
     if (M == 0 || batch == 0) return OILHIP_OK;
+    if (batch <= 4) {
+        const int rc = launch_gemv_flat8(d_w, d_cb, d_x, d_y, batch, M, K, scale, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
     hipLaunchKernelGGL(flat8_kernel, dim3(M), dim3(256), 0, (hipStream_t)stream, d_w, d_cb, d_x, d_y, batch, M, K, scale);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;

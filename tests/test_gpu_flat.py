@@ -44,7 +44,10 @@ def test_golden_engine_quant_gemm():
         assert np.array_equal(got.ravel().view(np.uint32), FL[f"eng/c{bits}_bits"])
 
 
-@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 300, 1000), (3, 17, 37), (2, 5, 1)])
+# K a multiple of 16 and M <= 4 take the register-resident kernel (one and several slabs per row, several chunks per
+# wavefront, a partial last column set); the rest the plain one
+@pytest.mark.parametrize("M,N,K", [(1, 4096, 4096), (4, 300, 1000), (3, 17, 37), (2, 5, 1), (1, 1000, 11008), (2, 77, 2304),
+                                   (4, 300, 1024), (3, 50, 4096), (1, 40000, 512), (1, 9, 16), (1, 5000, 48), (5, 64, 1024)])
 def test_oil8_gemm_against_oracle(M, N, K):
     rng = np.random.default_rng(M * 1000 + N + K)
     idx = rng.integers(0, 256, N * K, dtype=np.uint8).astype(np.uint8)
