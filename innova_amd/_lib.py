@@ -89,6 +89,10 @@ def lib():
             raise OilHipError(
                 f"{LIB_PATH} is missing: build it first (make -C innova_amd/csrc, or "
                 "python -c 'import __graft_entry__ as g; g.build()'); there is no CPU fallback")
+        try:                          # torch ships its own HIP runtime: it has to be the one both of us use, so it
+            import torch  # noqa: F401  # is loaded first (the other order leaves torch without a visible GPU)
+        except ImportError:
+            pass
         L = C.CDLL(LIB_PATH)
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(L, name)

@@ -2,6 +2,8 @@
 // GEMV/GEMM that decodes every weight through decode_weight().  They cover every
 // wire format, mixed-format rows and ragged tail blocks; the specialised kernels
 // (gemv_oil4.hip, ...) take over for the shapes that matter for throughput.
+#include <algorithm>
+
 #include "common.h"
 
 namespace oilhip {
@@ -21,6 +23,66 @@ dequant_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__
         float* o = out + (out_off ? out_off[b] : (uint64_t)b * uniform_nw);
         for (uint32_t i = threadIdx.x; i < d.nw; i += 256)
             o[i] = decode_weight(d.fmt, cb, d.cb_bytes, idx, d.idx_bytes, d.nw, i, T);
+    }
+}
+
+// Full OIL2 / OIL4 / OIL8 blocks laid out back to back (one format, regular stride): a wavefront per block, lane l decodes
+// weights 4l .. 4l+3 from two dwords and stores one float4, so a block is one coalesced 1 KB store.  Values are
+// formed exactly as decode_weight forms them: level (literal table / host-built table) times the FP16 scale widened
+// by the integer rule; slot weights are 0.
+template <int BITS>
+__global__ void __launch_bounds__(256)
+dequant_lattice_kernel(const uint8_t* __restrict__ base, uint32_t stride, const DecodeTables* __restrict__ T,
+                       float* __restrict__ out, uint32_t nblocks) {
+    __shared__ float lv[256];
+    if (BITS == 8) lv[threadIdx.x] = T->lv8[threadIdx.x];
+    else if (BITS == 4 && threadIdx.x < 16) lv[threadIdx.x] = kLv4[threadIdx.x];
+    else if (BITS == 2 && threadIdx.x < 4) lv[threadIdx.x] = kLv2[threadIdx.x];
+    __syncthreads();
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    for (uint32_t b = blockIdx.x * 4u + wave; b < nblocks; b += gridDim.x * 4u) {
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(base + (size_t)b * stride);
+        const float scale = half_bits_to_float(q[0] & 0xFFFFu);
+        // first code bit of weight 4l: 16 + BITS * (4l - slots before it); one slot per 16*BITS weights
+        const uint32_t i0 = 4u * lane;
+        const uint32_t bit = 16u + BITS * (i0 - i0 / (16u * BITS));
+        const uint32_t lo = q[bit >> 5], hi = q[(bit >> 5) + 1u];            // hi may be the first dword after the block: unused bits
+        const uint32_t v = __builtin_amdgcn_alignbit(hi, lo, bit & 31u);
+        const bool last_is_slot = ((i0 + 4u) % (16u * BITS)) == 0u;
+        float4 o;
+        if (BITS == 2) {
+            o.x = lv[v & 3u] * scale; o.y = lv[(v >> 2) & 3u] * scale; o.z = lv[(v >> 4) & 3u] * scale;
+            o.w = last_is_slot ? 0.0f : lv[(v >> 6) & 3u] * scale;
+        } else if (BITS == 4) {
+            o.x = lv[v & 15u] * scale; o.y = lv[(v >> 4) & 15u] * scale; o.z = lv[(v >> 8) & 15u] * scale;
+            o.w = last_is_slot ? 0.0f : lv[(v >> 12) & 15u] * scale;
+        } else {
+            o.x = lv[v & 255u] * scale; o.y = lv[(v >> 8) & 255u] * scale; o.z = lv[(v >> 16) & 255u] * scale;
+            o.w = last_is_slot ? 0.0f : lv[v >> 24] * scale;
+        }
+        reinterpret_cast<float4*>(out + (size_t)b * 256u)[lane] = o;
+    }
+}
+
+// Full OIL1 (FMT 0: eight FP16 run means, 16 bytes) and SPARK_Q0 (FMT 1: per run of 32 an FP16 scale and 32 sign
+// bits, 48 bytes) blocks laid out back to back; lane l stores weights 4l .. 4l+3 of its wavefront's block.
+template <int FMT>
+__global__ void __launch_bounds__(256)
+dequant_runs_kernel(const uint8_t* __restrict__ base, uint32_t stride, float* __restrict__ out, uint32_t nblocks) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint32_t run = lane >> 3, j0 = 4u * (lane & 7u);
+    for (uint32_t b = blockIdx.x * 4u + wave; b < nblocks; b += gridDim.x * 4u) {
+        const uint16_t* h = reinterpret_cast<const uint16_t*>(base + (size_t)b * stride);
+        float4 o;
+        if (FMT == 0) {
+            const float m = half_bits_to_float(h[run]);
+            o = make_float4(m, m, m, m);
+        } else {
+            const float sc = half_bits_to_float(h[3u * run]);
+            const uint32_t bits = ((uint32_t)h[3u * run + 1u] | ((uint32_t)h[3u * run + 2u] << 16)) >> j0;
+            o = make_float4((bits & 1u) ? sc : -sc, (bits & 2u) ? sc : -sc, (bits & 4u) ? sc : -sc, (bits & 8u) ? sc : -sc);
+        }
+        reinterpret_cast<float4*>(out + (size_t)b * 256u)[lane] = o;
     }
 }
 
@@ -98,6 +160,29 @@ int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s) {
     const DecodeTables* T = nullptr;
     if (int rc = get_tables(&T)) return rc;
     if (w.nblocks == 0) return OILHIP_OK;
+    if (w.all_full && w.uniform_stride > 0 && !w.d_out_off && (w.uniform_base & 3u) == 0 && (w.uniform_stride & 3u) == 0) {
+        const uint32_t g = std::min<uint32_t>((w.nblocks + 3u) / 4u, (uint32_t)device_cu_count() * 16u);
+        const uint8_t* base = w.d_payload + w.uniform_base;
+        const int f = w.uniform_fmt;
+        const uint32_t st = w.uniform_stride;
+        bool done = true;
+        if (f == OILHIP_OIL4 && st == 128 && w.uniform_cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<4>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL8 && st == 256 && w.uniform_cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<8>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL2 && st == 64 && w.uniform_cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<2>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL1 && st == 16 && w.uniform_cb == 16)
+            hipLaunchKernelGGL(dequant_runs_kernel<0>, dim3(g), dim3(256), 0, s, base, st, d_out, w.nblocks);
+        else if (f == OILHIP_SPARK_Q0 && st == 48 && w.uniform_cb == 0)
+            hipLaunchKernelGGL(dequant_runs_kernel<1>, dim3(g), dim3(256), 0, s, base, st, d_out, w.nblocks);
+        else
+            done = false;
+        if (done) {
+            OILHIP_HIP(hipGetLastError());
+            return OILHIP_OK;
+        }
+    }
     const uint32_t grid = w.nblocks < (1u << 20) ? w.nblocks : (1u << 20);
     hipLaunchKernelGGL(dequant_kernel, dim3(grid), dim3(256), 0, s, w.d_payload, w.d_blocks,
                        w.d_out_off, T, d_out, w.nblocks, 256u);

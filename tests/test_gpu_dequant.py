@@ -88,6 +88,33 @@ def test_truncated_and_garbage_payloads_match_reference_rules():
                 assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (fmt, n, cut)
 
 
+@pytest.mark.parametrize("fmt,nbytes", [(ia.Format.OIL4, 128), (ia.Format.OIL8, 256), (ia.Format.OIL2, 64),
+                                        (ia.Format.OIL1, 16), (ia.Format.SPARK_Q0, 48)])
+def test_uniform_full_blocks_random_payload_bit_exact(fmt, nbytes):
+    """Tensors of full OIL1 / SPARK_Q0 / OIL2 / OIL4 / OIL8 blocks take the wavefront-per-block kernels: random payload bytes (every code, scales
+    including subnormals, infinities and NaNs) against the oracle, and quantized data against it as well."""
+    rng = np.random.default_rng(int(fmt) + 40)
+    nb = 3001
+    payload = rng.integers(0, 256, nb * nbytes, dtype=np.uint8).astype(np.uint8)
+    blocks = np.zeros(nb, dtype=ia._lib.BLOCK_DTYPE)
+    blocks["cb_off"] = np.arange(nb, dtype=np.uint64) * nbytes
+    if fmt == ia.Format.OIL1:                      # the run means live in the codebook channel
+        blocks["cb_bytes"], blocks["idx_off"], blocks["idx_bytes"] = nbytes, blocks["cb_off"] + nbytes, 0
+    else:
+        blocks["idx_off"], blocks["idx_bytes"] = blocks["cb_off"], nbytes
+    blocks["nw"], blocks["fmt"] = 256, int(fmt)
+    with ia.DeviceWeights.from_blocks(payload, blocks, nb, 256) as dw:
+        assert dw.info()["uniform_fmt"] == int(fmt)
+        got = dw.dequant().cpu().numpy()
+    want = O.dequant_blocks(payload, to_orc_blocks(blocks))
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    w = gaussian_weights(256 * 777, seed=3 + int(fmt), outlier_every=19)
+    payload, blocks = ia.block_codec.quantize_tensor(w, fmt)
+    with ia.DeviceWeights.from_blocks(payload, blocks, 777, 256) as dw:
+        got = dw.dequant().cpu().numpy()
+    assert np.array_equal(got.view(np.uint32), O.dequant_blocks(payload, to_orc_blocks(blocks)).view(np.uint32))
+
+
 def test_full_size_tensor_oil4_bit_exact():
     """The 4096 x 11008 OIL4 matrix of the decode benchmark, checked whole."""
     rows, cols = 11008, 4096
