@@ -119,25 +119,61 @@ prod_packed_kernel(const uint8_t* __restrict__ wq, const uint16_t* __restrict__ 
 // Engine layout: codes packed along the flat [K][N] index; thread per output column
 // n, sequential in k like the reference loop (terms with A == 0 are skipped).
 template <int BITS>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 engine_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const float* __restrict__ cb,
               float* __restrict__ C, long long M, long long N, long long K) {
-    __shared__ float c[1 << BITS];
-    for (int i = threadIdx.x; i < (1 << BITS); i += 256) c[i] = cb[i];
+    // One wavefront per 64 outputs of a row of C: the chain of every output stays one thread's k-ordered FMA
+    // sequence (bit-identical to the reference loop), so the only parallelism is across outputs; what can be taken
+    // off the chain is taken off: the codes of 32 steps are fetched together, A[m][k] is wave-uniform and read
+    // through the scalar cache, and the codebook sits in LDS in 8 copies.
+    __shared__ float c[(1 << BITS) * 8];
+    for (int i = threadIdx.x; i < (1 << BITS) * 8; i += 64) c[i] = cb[i >> 3];
     __syncthreads();
-    const long long n = (long long)blockIdx.x * 256 + threadIdx.x;
+    const long long n = (long long)blockIdx.x * 64 + threadIdx.x;
     const long long m = blockIdx.y;
-    if (n >= N) return;
+    const bool live = n < N;
+    const long long nn = live ? n : N - 1;                // idle lanes follow the last column and store nothing
     constexpr int PER = 8 / BITS;
+    constexpr int UN = 32;
+    const float* a_row = A + m * K;
+    const uint32_t copy = threadIdx.x & 7u;
     float acc = 0.0f;
-    for (long long k = 0; k < K; ++k) {
-        const float a = A[m * K + k];
-        if (a == 0.0f) continue;
-        const long long flat = k * N + n;
-        const uint32_t code = (bq[flat / PER] >> ((flat % PER) * BITS)) & ((1u << BITS) - 1u);
-        acc = __fmaf_rn(a, c[code], acc);
+    long long k = 0;
+    uint8_t raw[UN], nxt[UN];
+    auto fetch = [&](uint8_t (&dst)[UN], long long k0) {
+#pragma unroll
+        for (int j = 0; j < UN; ++j) dst[j] = bq[((unsigned long long)(k0 + j) * (unsigned long long)N + (unsigned long long)nn) / PER];
+    };
+    if (K >= UN) fetch(raw, 0);
+    for (; k + UN <= K; k += UN) {
+        const bool more = k + 2 * UN <= K;
+        if (more) fetch(nxt, k + UN);                     // the next 32 steps fly while these are folded in
+        float lv[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {                    // look-ups off the chain: none of them depends on acc
+            const uint32_t sub = (uint32_t)((unsigned long long)(k + j) * (unsigned long long)N + (unsigned long long)nn) & (uint32_t)(PER - 1);
+            const uint32_t code = ((uint32_t)raw[j] >> (sub * BITS)) & ((1u << BITS) - 1u);
+            lv[j] = c[code * 8u + copy];
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const float a = a_row[k + j];
+            const float t = __fmaf_rn(a, lv[j], acc);
+            acc = a != 0.0f ? t : acc;                    // the reference skips the term, 0 * inf must not reach acc
+        }
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) raw[j] = nxt[j];
+        }
     }
-    C[m * N + n] = acc;
+    for (; k < K; ++k) {
+        const float a = a_row[k];
+        if (a == 0.0f) continue;
+        const long long flat = k * N + nn;
+        const uint32_t code = (bq[flat / PER] >> ((flat % PER) * BITS)) & ((1u << BITS) - 1u);
+        acc = __fmaf_rn(a, c[code * 8u + copy], acc);
+    }
+    if (live) C[m * N + n] = acc;
 }
 
 // The engines whose B operand is not a codebook index: kind 1 = Oil1Engine (one float per 32 flat positions,
@@ -146,33 +182,89 @@ engine_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const
 // math::vec_fp16_to_fp32 does, src/math.cpp:509-526; src/oil_engines_fp.cpp:433-451), 32 = OIL32Engine (:531-547).
 // Terms with a == 0 are skipped and k runs in ascending order, as in the reference loops.
 template <int KIND>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(64)
 engine_dense_kernel(const float* __restrict__ A, const void* __restrict__ B, const float* __restrict__ scales,
                     long long block, float* __restrict__ C, long long M, long long N, long long K) {
-    const long long n = (long long)blockIdx.x * 256 + threadIdx.x;
+    // Same frame as engine_kernel: a wavefront per 64 outputs, the operand of 32 steps fetched together and one
+    // batch ahead, the k-ordered chain of every output untouched.
+    const long long n = (long long)blockIdx.x * 64 + threadIdx.x;
     const long long m = blockIdx.y;
-    if (n >= N) return;
-    float acc = 0.0f;
-    for (long long k = 0; k < K; ++k) {
-        const float a = A[m * K + k];
-        if (a == 0.0f) continue;
-        const long long flat = k * N + n;
-        if (KIND == 1) {
-            acc = __fmaf_rn(a, reinterpret_cast<const float*>(B)[flat / 32], acc);
-        } else if (KIND == 32) {
-            acc = __fmaf_rn(a, reinterpret_cast<const float*>(B)[flat], acc);
+    const bool live = n < N;
+    const unsigned long long nn = (unsigned long long)(live ? n : N - 1);
+    constexpr int UN = KIND == 3 ? 16 : 32;              // kind 3 fetches two operands per step
+    const float* a_row = A + m * K;
+    struct Term { float b; float s; };                   // kind 3: b = +1 / -1 / 0 by code, s = scale of the flat position's block
+    // kind 3: block index and offset of the next flat position to be fetched (fetches go through k in order)
+    const unsigned long long ublock = block > 0 ? (unsigned long long)block : 1ull;
+    unsigned long long fq = nn / ublock, fr = nn % ublock;
+    const unsigned long long dq = (unsigned long long)N / ublock, dr = (unsigned long long)N % ublock;
+    auto fetch_one = [&](long long kk) {
+        const unsigned long long flat = (unsigned long long)kk * (unsigned long long)N + nn;
+        Term t{0.0f, 1.0f};
+        if (KIND == 1) t.b = reinterpret_cast<const float*>(B)[flat / 32];
+        else if (KIND == 32) t.b = reinterpret_cast<const float*>(B)[flat];
+        else if (KIND == 16) t.b = __uint_as_float((uint32_t)reinterpret_cast<const uint16_t*>(B)[flat]);   // raw half, widened later
+        else {
+            t.s = scales[fq];
+            t.b = __uint_as_float((uint32_t)((reinterpret_cast<const uint8_t*>(B)[flat / 4] >> ((flat % 4) * 2)) & 3u));
+            fq += dq; fr += dr;
+            if (fr >= ublock) { fr -= ublock; ++fq; }
+        }
+        return t;
+    };
+    auto widen = [](float raw) {                          // math::vec_fp16_to_fp32: -0 widens to +0; selects only
+        const uint32_t h = __float_as_uint(raw);
+        const uint32_t sg = (h & 0x8000u) << 16, e = (h >> 10) & 31u, mt = h & 0x3FFu;
+        const uint32_t normal = sg | ((e + 112u) << 23) | (mt << 13);
+        const uint32_t infnan = sg | 0x7F800000u | (mt << 13);
+        const uint32_t sub = sg | __float_as_uint(__uint2float_rn(mt) * 0x1p-24f);      // exact
+        const uint32_t r = e == 31u ? infnan : (e != 0u ? normal : sub);
+        return (h & 0x7FFFu) == 0u ? 0.0f : __uint_as_float(r);
+    };
+    auto fold = [&](float acc, float a, const Term& t) {
+        if (KIND == 1 || KIND == 32) {
+            const float r = __fmaf_rn(a, t.b, acc);
+            return a != 0.0f ? r : acc;
         } else if (KIND == 16) {
-            const uint32_t h = reinterpret_cast<const uint16_t*>(B)[flat];
-            const float b = (h & 0x7FFFu) == 0u ? 0.0f : half_bits_to_float(h);    // -0 widens to +0 there
-            acc = __fmaf_rn(a, b, acc);
+            const float r = __fmaf_rn(a, t.b, acc);                                  // widened before the chain starts
+            return a != 0.0f ? r : acc;
         } else {
-            const float s = a * scales[flat / block];
-            const uint32_t code = (reinterpret_cast<const uint8_t*>(B)[flat / 4] >> ((flat % 4) * 2)) & 3u;
-            if (code == 2u) acc += s;
-            else if (code == 0u) acc -= s;
+            const float s = __fmul_rn(a, t.s);                                       // a product, then a sum: no fused form here
+            const uint32_t code = __float_as_uint(t.b);
+            const float r = code == 2u ? __fadd_rn(acc, s) : (code == 0u ? __fsub_rn(acc, s) : acc);
+            return a != 0.0f ? r : acc;
+        }
+    };
+    float acc = 0.0f;
+    long long k = 0;
+    Term cur[UN], nxt[UN];
+    if (K >= UN) {
+#pragma unroll
+        for (int j = 0; j < UN; ++j) cur[j] = fetch_one(j);
+    }
+    for (; k + UN <= K; k += UN) {
+        const bool more = k + 2 * UN <= K;
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) nxt[j] = fetch_one(k + UN + j);
+        }
+        if (KIND == 16) {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) cur[j].b = widen(cur[j].b);
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) acc = fold(acc, a_row[k + j], cur[j]);
+        if (more) {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) cur[j] = nxt[j];
         }
     }
-    C[m * N + n] = acc;
+    for (; k < K; ++k) {
+        Term t = fetch_one(k);
+        if (KIND == 16) t.b = widen(t.b);
+        acc = fold(acc, a_row[k], t);
+    }
+    if (live) C[m * N + n] = acc;
 }
 
 // OIL{8,4,2}Engine::dequant_tensor (src/oil_engines_oil8.cpp:171-183, oil4.cpp:205-220, oil2.cpp:184-193): packed
@@ -275,11 +367,11 @@ int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b, con
     if (bits != 2 && bits != 4 && bits != 8) return fail(OILHIP_E_ARG, "bits must be 2, 4 or 8");
     if (M == 0 || N == 0) return OILHIP_OK;
     if (M > 65535) return fail(OILHIP_E_ARG, "M exceeds the grid limit");
-    const dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)M);
+    const dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)M);
     hipStream_t s = (hipStream_t)stream;
-    if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
-    else if (bits == 4) hipLaunchKernelGGL(engine_kernel<4>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
-    else hipLaunchKernelGGL(engine_kernel<2>, grid, dim3(256), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    else if (bits == 4) hipLaunchKernelGGL(engine_kernel<4>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    else hipLaunchKernelGGL(engine_kernel<2>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }
@@ -305,12 +397,12 @@ int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const 
     if (M == 0 || N == 0) return OILHIP_OK;
     if (kind == 3 && (!d_scales || block <= 0)) return fail(OILHIP_E_ARG, "the SPARK engine needs scales and a block size");
     if (M > 65535) return fail(OILHIP_E_ARG, "M exceeds the grid limit");
-    const dim3 grid((uint32_t)((N + 255) / 256), (uint32_t)M);
+    const dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)M);
     hipStream_t s = (hipStream_t)stream;
-    if (kind == 1) hipLaunchKernelGGL(engine_dense_kernel<1>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
-    else if (kind == 3) hipLaunchKernelGGL(engine_dense_kernel<3>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
-    else if (kind == 16) hipLaunchKernelGGL(engine_dense_kernel<16>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
-    else hipLaunchKernelGGL(engine_dense_kernel<32>, grid, dim3(256), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    if (kind == 1) hipLaunchKernelGGL(engine_dense_kernel<1>, grid, dim3(64), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else if (kind == 3) hipLaunchKernelGGL(engine_dense_kernel<3>, grid, dim3(64), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else if (kind == 16) hipLaunchKernelGGL(engine_dense_kernel<16>, grid, dim3(64), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
+    else hipLaunchKernelGGL(engine_dense_kernel<32>, grid, dim3(64), 0, s, d_a, d_b, d_scales, (long long)block, d_c, M, N, K);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }
