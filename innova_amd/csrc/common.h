@@ -50,6 +50,9 @@ int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
 int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+// production gemv_oil4 form for one activation row: rows of K/2 code bytes, FP16 codebook of 16, one scale
+int launch_gemv_flat4(const uint8_t* d_w, const uint16_t* d_cb16, float scale, const float* d_x, float* d_y, int rows, int K,
+                      hipStream_t s);
 int launch_gemv_oil8(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // kernel::oil8_gemm form: rows of K index bytes, any 256-entry codebook; out[m*N + n] = scale * dot
 int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_act, float* d_out, int M, int N, int K, float scale,

@@ -341,6 +341,12 @@ int oilhip_prod_gemv_oil4(const uint8_t* d_w, const uint16_t* d_cb16, float scal
                           float* d_y, int M, int K, int batch, void* stream) {
     if (int rc = check(d_w, d_cb16, d_x, d_y, M, batch, K)) return rc;
     if (M == 0 || batch == 0) return OILHIP_OK;
+    if (batch <= 2) {                                 // decode: the register-resident kernel, one activation row per launch
+        int rc = 0;
+        for (int b = 0; b < batch && rc == 0; ++b)
+            rc = launch_gemv_flat4(d_w, d_cb16, scale, d_x + (size_t)b * K, d_y + (size_t)b * M, M, K, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
     hipLaunchKernelGGL(prod_packed_kernel<4>, dim3(M), dim3(256), 0, (hipStream_t)stream, d_w, d_cb16, scale,
                        d_x, d_y, M, K, batch);
     OILHIP_HIP(hipGetLastError());

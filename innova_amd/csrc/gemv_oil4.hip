@@ -48,11 +48,14 @@ constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 3
 // while x is staged, so the SwiGLU product never makes a round trip through memory.
 // XF = 2: the activation row is rmsnorm(x) = x * r * (1 + xw), r = 1 / sqrt(mean(x^2) + 1e-6) (rmsnorm, same file :39-44):
 // x * (1 + xw) is staged, every workgroup forms r from the whole row it loads anyway, and r scales the dot products.
+// XF = 3: not a block tensor but rows of cols/2 bytes of packed codes (low nibble first) with a 16-entry FP16 codebook
+// passed through xw and one scale for the whole matrix (gemv_oil4 of src/kernel_production.cpp): x stays in natural
+// order, the pair table is built from the codebook, there is no block scale and y is multiplied by out_scale.
 template <int CS, int RPW, int MB, int MAXT, int XF = 0, bool ROLL = false>
 __global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const float* __restrict__ xw, float* __restrict__ y,
                  uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M,
-                 uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups) {
+                 uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups, float out_scale) {
     constexpr int NL = CS * RPW;      // wave-loads per chunk
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
@@ -158,8 +161,18 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     // table writes are slotted in between the loads instead of after them.
     issue_load(0, 0u);
     __builtin_amdgcn_sched_barrier(0);
-    const float lv_lane = level_literal(lane & 15u);                          // lane i holds level[i & 15]
-    const float lo_fix = level_literal((tid >> 4) & 15u);
+    float lv_lane, lo_fix;                                                    // lane i holds level[i & 15]
+    if (XF == 3) {
+        const uint16_t* cb16 = reinterpret_cast<const uint16_t*>(xw);
+        auto widen = [](uint32_t h) {                                         // fp16_to_float of the flat kernels: NaNs become the default NaN
+            return ((h >> 10) & 31u) == 31u && (h & 0x3FFu) != 0u ? __uint_as_float(0x7FC00000u) : half_bits_to_float(h);
+        };
+        lv_lane = widen(cb16[lane & 15u]);
+        lo_fix = widen(cb16[(tid >> 4) & 15u]);
+    } else {
+        lv_lane = level_literal(lane & 15u);
+        lo_fix = level_literal((tid >> 4) & 15u);
+    }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
         if (k + 1 < PFA) issue_load(k + 1, 0u);
@@ -182,10 +195,10 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     bool xlast_ok;
     {
         const uint32_t w = (tid * 4u) & 255u;
-        xlast_ok = (w & 63u) != 60u;                                          // i % 64 == 63 is a slot
+        xlast_ok = XF == 3 || (w & 63u) != 60u;                               // i % 64 == 63 is a slot
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const uint32_t pnib = w + k - (w >> 6) + 4u;
+            const uint32_t pnib = XF == 3 ? w + k : w + k - (w >> 6) + 4u;
             xoff[k] = ((pnib >> 2) & 7u) * 32u + (pnib >> 5) * 4u + (pnib & 3u);
         }
     }
@@ -196,7 +209,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         dst[xoff[2]] = __uint_as_float(v.z);
         if (xlast_ok) dst[xoff[3]] = __uint_as_float(v.w);
     };
-    for (uint32_t bz = tid; bz < nblk * MB; bz += 512u) {                     // scale nibbles of every block
+    for (uint32_t bz = tid; XF != 3 && bz < nblk * MB; bz += 512u) {          // scale nibbles of every block
         const uint32_t m = bz / nblk, b = bz % nblk;
         *reinterpret_cast<float4*>(xs + (size_t)m * xstride + b * kXsBlock) = make_float4(0.f, 0.f, 0.f, 0.f);
     }
@@ -237,7 +250,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         if (lane == 63) ssq_part[wave] = v;
     }
     __syncthreads();
-    float yscale = 1.0f;
+    float yscale = XF == 3 ? out_scale : 1.0f;
     if (XF == 2) {
         const float tot = ((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) + ((ssq_part[4] + ssq_part[5]) + (ssq_part[6] + ssq_part[7]));
         yscale = 1.0f / sqrtf(tot / (float)cols + 1e-6f);
@@ -286,7 +299,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
             if (n + 1 < NL) lookup_load(wv[n + 1], lanebase, nxt);    // next load's table reads fly during these FMAs
             __builtin_amdgcn_sched_barrier(0);                        // keep them above the FMAs
             // the block's FP16 scale sits in the low half of its first lane's first dword
-            const float scale = __half2float(__ushort_as_half((unsigned short)(dpp_bcast8(wv[n].x) & 0xFFFFu)));
+            const float scale = XF == 3 ? 1.0f : __half2float(__ushort_as_half((unsigned short)(dpp_bcast8(wv[n].x) & 0xFFFFu)));
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
                 float a0 = 0.0f, a1 = 0.0f;
@@ -329,7 +342,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
                 for (int it = 0; it < RPW; ++it)
 #pragma unroll
                     for (int m = 0; m < MB; ++m)
-                        if (cbase + it < r1 && m0 + m < M) y[(size_t)(m0 + m) * rows + cbase + it] = XF == 2 ? part[m][it] * yscale : part[m][it];
+                        if (cbase + it < r1 && m0 + m < M) y[(size_t)(m0 + m) * rows + cbase + it] = XF >= 2 ? part[m][it] * yscale : part[m][it];
             }
             continue;
         }
@@ -351,7 +364,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
                 const float* pr = red + (size_t)o * S;
                 float s = 0.0f;
                 for (uint32_t k = 0; k < S; ++k) s += pr[k];
-                y[(size_t)(m0 + m) * rows + r] = XF == 2 ? s * yscale : s;
+                y[(size_t)(m0 + m) * rows + r] = XF >= 2 ? s * yscale : s;
             }
         }
         __syncthreads();
@@ -366,7 +379,8 @@ struct Oil4Plan {
 };
 
 template <int CS, int RPW, int MB, int MAXT, int XF, bool ROLL>
-int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
+int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p,
+           float out_scale = 1.0f) {
     static bool attr_done = false;
     auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT, XF, ROLL>;
     if (!attr_done) {
@@ -380,7 +394,7 @@ int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* 
     for (int m0 = 0; m0 < M; m0 += MB) {
         hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_xw, d_y,
                            (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M,
-                           (uint32_t)w.rows / J, (uint32_t)w.rows % J, wave_groups);
+                           (uint32_t)w.rows / J, (uint32_t)w.rows % J, wave_groups, out_scale);
         OILHIP_HIP(hipGetLastError());
     }
     return OILHIP_OK;
@@ -432,11 +446,12 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
 }
 
 template <int MB, int XF = 0>
-int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p) {
+int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p,
+             float out_scale = 1.0f) {
 #define OIL4_CASE(CS_, RPW_) \
     if (p.cs == CS_ && p.rpw == RPW_) \
-        return p.nchunks > 1 ? launch<CS_, RPW_, MB, 512, XF, true>(w, d_x, d_xw, d_y, M, s, p) \
-                             : launch<CS_, RPW_, MB, 512, XF, false>(w, d_x, d_xw, d_y, M, s, p);
+        return p.nchunks > 1 ? launch<CS_, RPW_, MB, 512, XF, true>(w, d_x, d_xw, d_y, M, s, p, out_scale) \
+                             : launch<CS_, RPW_, MB, 512, XF, false>(w, d_x, d_xw, d_y, M, s, p, out_scale);
     OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
     if constexpr (MB == 1) {
         OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)
@@ -474,6 +489,19 @@ int launch_gemv_oil4_rmsnorm(const oilhip_weights& w, const float* d_x, const fl
     Oil4Plan p;
     if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, 8, &p)) return 1;
     return dispatch<1, 2>(w, d_x, d_xw, d_y, 1, s, p);
+}
+
+// gemv_oil4 of src/kernel_production.cpp for one activation row: y[r] = scale * sum_k f16(cb16[code(r, k)]) * x[k], rows
+// of K/2 bytes, low nibble first.  Returns 1 when the shape is not covered (K must be a multiple of 256).
+int launch_gemv_flat4(const uint8_t* d_w, const uint16_t* d_cb16, float scale, const float* d_x, float* d_y, int rows, int K,
+                      hipStream_t s) {
+    if (rows < 1 || K < 256 || (K & 255) || (reinterpret_cast<uintptr_t>(d_w) & 15u)) return 1;
+    oilhip_weights w;                                             // a view: rows of K/2 bytes
+    w.d_payload = const_cast<uint8_t*>(d_w);
+    w.rows = (uint64_t)rows; w.cols = (uint64_t)K;
+    Oil4Plan p;
+    if (!make_plan((uint32_t)rows, (uint32_t)K, 1, 8, &p)) return 1;
+    return dispatch<1, 3>(w, d_x, reinterpret_cast<const float*>(d_cb16), d_y, 1, s, p, scale);
 }
 
 }  // namespace oilhip

@@ -69,7 +69,8 @@ def test_oil4_gemm_against_oracle(M, N, K):
     assert rel_l2(got, O.oil4_gemm(packed, cb16, act, M, N, K, order=2)) <= TOL
 
 
-@pytest.mark.parametrize("M,K,batch", [(1000, 4096, 1), (50, 333, 5), (7, 2, 3)])
+@pytest.mark.parametrize("M,K,batch", [(1000, 4096, 1), (50, 333, 5), (7, 2, 3), (4096, 11008, 1), (300, 256, 2), (40000, 512, 1),
+                                       (77, 2304, 2)])
 def test_production_gemv_batch_against_oracle(M, K, batch):
     rng = np.random.default_rng(M + K + batch)
     X = rng.standard_normal((batch, K)).astype(np.float32)
