@@ -3,6 +3,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <algorithm>
 #include <vector>
 
 #include "common.h"
@@ -131,6 +132,21 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
         if ((e = hipMalloc(&w->d_blocks, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(blocks)");
         if ((e = hipMemcpy(w->d_blocks, db.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
             return bail(e, "hipMemcpy(blocks)");
+        const uint64_t bpr = cols / 256;
+        if (all_full && !uniform && (cols & 255) == 0 && bpr >= 2 && bpr <= 0xFFFFFFFFull && (uint64_t)nblocks == rows * bpr) {
+            // The all-format GEMV takes 8 consecutive descriptors per step and runs every format present among them;
+            // with each row's blocks ordered by format most steps see one format only.  Order within a format stays
+            // by column (stable), so the result does not depend on anything but the tensor.
+            std::vector<DevBlock> sorted(db);
+            for (uint64_t r = 0; r < rows; ++r) {
+                DevBlock* row = sorted.data() + r * bpr;
+                for (uint64_t c = 0; c < bpr; ++c) row[c].nw = (uint32_t)c;
+                std::stable_sort(row, row + bpr, [](const DevBlock& a, const DevBlock& b) { return a.fmt < b.fmt; });
+            }
+            if ((e = hipMalloc(&w->d_sorted, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(sorted blocks)");
+            if ((e = hipMemcpy(w->d_sorted, sorted.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
+                return bail(e, "hipMemcpy(sorted blocks)");
+        }
         if (!all_full) {
             if ((e = hipMalloc(&w->d_out_off, 8 * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(out_off)");
             if ((e = hipMemcpy(w->d_out_off, out_off.data(), 8 * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
@@ -213,6 +229,7 @@ int oilhip_weights_destroy(oilhip_weights* w) {
     if (!w) return OILHIP_OK;
     if (w->d_payload) (void)hipFree(w->d_payload);
     if (w->d_blocks) (void)hipFree(w->d_blocks);
+    if (w->d_sorted) (void)hipFree(w->d_sorted);
     if (w->d_out_off) (void)hipFree(w->d_out_off);
     delete w;
     return OILHIP_OK;

@@ -32,6 +32,8 @@ struct oilhip_weights {
     int device = 0;
     uint8_t* d_payload = nullptr;           // block payloads, each 16-byte aligned
     oilhip::DevBlock* d_blocks = nullptr;   // one descriptor per block
+    oilhip::DevBlock* d_sorted = nullptr;   // mixed-format tensors of full blocks: each row's descriptors ordered by format,
+                                            // the block's column index in `nw` (rows keep their place)
     uint64_t* d_out_off = nullptr;          // first output index per block (only when nw varies)
     uint64_t alloc_bytes = 0;               // size of d_payload
     uint64_t payload_bytes = 0;             // sum of cb_bytes + idx_bytes

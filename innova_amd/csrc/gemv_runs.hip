@@ -170,7 +170,8 @@ template <int MB>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
 gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__ blocks, const DecodeTables* __restrict__ T,
                  const float* __restrict__ x, float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M,
-                 int uniform_fmt, uint32_t uniform_stride, uint32_t uniform_cb, uint32_t uniform_idx, uint32_t uniform_base) {
+                 int uniform_fmt, uint32_t uniform_stride, uint32_t uniform_cb, uint32_t uniform_idx, uint32_t uniform_base,
+                 int sorted) {
     extern __shared__ __align__(16) float smem[];
     const uint32_t bpr = cols >> 8, nruns = cols >> 5;
     const uint32_t xpad = nruns * kRunPad;
@@ -210,6 +211,7 @@ gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict
             if (blk < bpr) {
                 const size_t b = (size_t)row * bpr + blk;
                 Run R;
+                uint32_t colblk = blk;
                 if (uniform_fmt >= 0) {
                     R.cb = payload + uniform_base + b * uniform_stride;
                     R.cb_bytes = uniform_cb; R.idx_bytes = uniform_idx; R.fmt = (uint32_t)uniform_fmt;
@@ -217,9 +219,10 @@ gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict
                     const DevBlock d = blocks[b];
                     R.cb = payload + (size_t)d.off16 * 16;
                     R.cb_bytes = d.cb_bytes; R.idx_bytes = d.idx_bytes; R.fmt = d.fmt;
+                    if (sorted) colblk = d.nw;             // descriptors ordered by format: the block's column travels with it
                 }
                 R.r = r;
-                const uint32_t run = blk * 8u + r;
+                const uint32_t run = colblk * 8u + r;
                 float w[32], mean = 0.f;
                 if (decode_run(R, T, L, w, &mean)) {
 #pragma unroll
@@ -268,8 +271,10 @@ int launch_runs(const oilhip_weights& w, const DecodeTables* T, const float* d_x
     const uint32_t need = ((uint32_t)w.rows + 3u) / 4u;
     if (grid > need) grid = need;
     const bool uni = w.uniform_fmt >= 0 && w.uniform_stride > 0;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w.d_payload, w.d_blocks, T, d_x, d_y, (uint32_t)w.rows,
-                       (uint32_t)w.cols, m0, M, uni ? w.uniform_fmt : -1, w.uniform_stride, w.uniform_cb, w.uniform_idx, w.uniform_base);
+    const bool sorted = !uni && w.d_sorted != nullptr;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w.d_payload, sorted ? w.d_sorted : w.d_blocks, T, d_x, d_y, (uint32_t)w.rows,
+                       (uint32_t)w.cols, m0, M, uni ? w.uniform_fmt : -1, w.uniform_stride, w.uniform_cb, w.uniform_idx, w.uniform_base,
+                       sorted ? 1 : 0);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }
