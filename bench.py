@@ -346,6 +346,45 @@ def bench_prefill(torch, ia, payload, blocks):
     return out
 
 
+def bench_dequant_and_engine(torch, ia, payload, blocks):
+    """dequantize_block_all over the whole headline tensor (180 MB of FP32 written) and OIL8Engine::quant_gemm at M=1
+    (B laid out [K][N], k-ordered FMA chain per output: bit-identical to the reference loop)."""
+    L = ia._lib.lib()
+    out = {}
+    with ia.DeviceWeights.from_blocks(payload, blocks, ROWS, COLS) as d:
+        o = torch.empty(ROWS * COLS, dtype=torch.float32, device="cuda")
+        for _ in range(3):
+            ia._lib.check(L.oilhip_dequant_f32(d.handle, o.data_ptr(), ia._lib.current_stream()))
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            ia._lib.check(L.oilhip_dequant_f32(d.handle, o.data_ptr(), ia._lib.current_stream()))
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) * 1e-3 / 20
+        out["dequant_oil4_11008x4096_us"] = round(t * 1e6, 1)
+        out["dequant_oil4_11008x4096_written_GBps"] = round(ROWS * COLS * 4 / t / 1e9, 1)
+        del o
+    N = K = 4096
+    b = torch.randint(0, 256, (K * N,), dtype=torch.uint8, device="cuda")
+    cb = torch.linspace(-8, 8, 256, device="cuda")
+    a = torch.randn(K, device="cuda")
+    c = torch.empty(N, device="cuda")
+    call = lambda: ia._lib.check(L.oilhip_engine_quant_gemm(8, a.data_ptr(), b.data_ptr(), cb.data_ptr(), c.data_ptr(),  # noqa: E731
+                                                             1, N, K, ia._lib.current_stream()))
+    call()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        call()
+    e1.record()
+    torch.cuda.synchronize()
+    out["engine_oil8_quant_gemm_M1_4096x4096_us"] = round(e0.elapsed_time(e1) * 1e2, 1)
+    return out
+
+
 def bench_moe(torch, ia):
     """MoE step: 8 OIL4 experts (gate/up 14336x4096, down 4096x14336: 704.6 MB of payload), 64 tokens, top-2.
     One expert is quantized on the host and uploaded 8 times (distinct device copies, same bytes)."""
@@ -482,6 +521,7 @@ def main():
         extra.update(bench_fused_layer(torch, ia, 32 * per_layer))
         extra.update(bench_tall(torch, ia))
         extra.update(bench_oil8(torch, ia))
+        extra.update(bench_dequant_and_engine(torch, ia, payload, blocks))
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))
         extra.update(bench_moe(torch, ia))
