@@ -2,21 +2,25 @@
 // (2..16 tokens per pass): Qwen35Engine::gemm with small B (src/adapters/tools/qwen35_engine.cpp:47-85)
 // and the per-expert batches of moe_dispatch_batched (src/moe_variants.cpp:767-827).
 //
-// Every weight is decoded once (dequant_lattice: level * FP16 scale in FP32, bit-identical to the
-// reference decode) and multiplied into all tokens on the matrix cores with the FP32 instruction
-// v_mfma_f32_16x16x4_f32 (A = 16 weight rows x 4 positions, B = 4 positions x 16 tokens).
-// Lane l = 16*kq + i supplies row i of a group of 16 rows; of a 128-byte block it owns the
-// 16-byte chunks kq and kq+4 (64 nibbles), one nibble per instruction.  Lane 16*kq + j supplies
-// token j at the same nibble positions, and accumulator register v of that lane collects
-// row 4*kq + v x token j.
+// The products run on the matrix cores in FP16 with both operands split in two: a level L of the table is
+// Lh + Ll (Lh = fp16(L), Ll = fp16(L - Lh)), an activation x is xh + xl the same way, and
+// L x = Lh xh + Lh xl + Ll xh up to 2^-22 relative (the Ll xl term is dropped); every product of two FP16 values is
+// exact in the FP32 accumulator of v_mfma_f32_16x16x32_f16, so three matrix instructions stand for one FP32 one at
+// a quarter of its cost per flop.  The FP16 block scale multiplies the block's 16 x 16 partial sums afterwards.
+// Lane l = 16*kq + i supplies row i of a group of 16 rows; of a 128-byte block it owns the 16-byte chunks kq and
+// kq+4 (64 nibbles), one dword (8 nibbles) per matrix instruction.  Lane 16*kq + j supplies token j at the same
+// nibble positions, and accumulator register v of that lane collects row 4*kq + v x token j.
 //
-// A wavefront owns two blocks of the row per K-pass (8 wavefronts = 16 blocks = 4096 columns) and
-// keeps the activations of those blocks in registers (2 x 64 per lane), so the main loop is:
-// two 16-byte loads per lane and unit (16 rows x 1 block), 32 byte-pair table lookups, 64
-// multiplies by the block scale, 64 MFMAs.  The activations pass through a wave-private LDS
-// staging area in natural order; each lane gathers the values of its nibble positions from it.
-// Partial sums of the wavefronts are added through LDS once per tile of 64 rows.
+// A wavefront owns two blocks of the row per K-pass (8 wavefronts = 16 blocks = 4096 columns) and keeps the split
+// activations of those blocks in registers (2 x 64 FP16 pairs per lane), so the main loop is: two 16-byte loads per
+// lane and unit (16 rows x 1 block), 32 byte-pair table lookups (each returns the two high and the two low halves
+// of a byte's levels, already packed as matrix operands), 24 matrix instructions, 4 scale multiplies.  The
+// activations are split and laid out in this operand order once per launch by pack_x_kernel (every workgroup needs
+// all of them), so the main kernel fetches its 128 operand dwords with plain 16-byte loads.  Partial sums of the
+// wavefronts are added through LDS once per tile of 64 rows.
 #include <hip/hip_fp16.h>
+
+#include <mutex>
 
 #include "common.h"
 #include "oil4_lds.h"
@@ -27,19 +31,61 @@ namespace {
 using namespace oil4;
 
 typedef float v4f __attribute__((ext_vector_type(4)));
+typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+typedef __attribute__((address_space(3))) const u32x2 lds_cu32x2;
+
+// L -> fp16(L) in the low half, fp16(L - fp16(L)) in the high half
+__device__ __forceinline__ uint32_t split_level(float L) {
+    const __half h = __float2half_rn(L);
+    const __half l = __float2half_rn(L - __half2float(h));
+    return (uint32_t)__half_as_ushort(h) | ((uint32_t)__half_as_ushort(l) << 16);
+}
 
 constexpr int kGroups = 4;                // groups of 16 rows per tile
-constexpr int kTokStride = 132;           // floats per token in the staging area: half a block plus the overlap
-constexpr int kStageBytes = 16 * kTokStride * 4;   // per wavefront: 16 tokens x 132 weights, natural order
-constexpr int kStageBase = kTabBytes;     // staging areas follow the level table
+constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
+constexpr int kRedBytes = 8 * kGroups * 64 * 16;
+
+// Packed activations of one pass of 16 tokens: for block blk of the row, half h and lane l = 16*kq + t (token t) 32
+// dwords: the high FP16 parts of the lane's 32 nibble positions (positions 2c, 2c+1 in dword c, c = 0..15), then the
+// low parts.  Piece j (dwords 4j .. 4j+3 of the 32) of all 64 lanes is one contiguous KB at
+// ((blk*2 + h)*8 + j)*1024 + l*16 bytes, so that a wavefront fetches it with one coalesced 16-byte load per lane.  Nibble p = 32*(kq + 4h) + s of a block holds weight
+// i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
+__global__ void __launch_bounds__(256)
+pack_x_kernel(const float* __restrict__ x, const int* __restrict__ tok, uint32_t* __restrict__ xp, uint32_t cols, int m0, int M,
+              uint32_t ldx, uint32_t xrows) {
+    const uint32_t id = blockIdx.x * 256u + threadIdx.x;            // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
+    const uint32_t bpr = cols >> 8;
+    if (id >= bpr * 2048u) return;
+    const uint32_t c = id & 15u, lane = (id >> 4) & 63u, h = (id >> 10) & 1u, blk = id >> 11;
+    const uint32_t t = lane & 15u, kq = lane >> 4;
+    const int m = m0 + (int)t;
+    const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
+    float v[2] = {0.0f, 0.0f};
+    if (src < xrows) {
+        const float* row = x + (size_t)src * ldx + (size_t)blk * 256u;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint32_t pn = 32u * (kq + 4u * h) + 2u * c + e;
+            if (pn >= 4u) {
+                const uint32_t q = pn - 4u;
+                v[e] = row[q + q / 63u];
+            }
+        }
+    }
+    const auto ph = __builtin_amdgcn_cvt_pkrtz(v[0], v[1]);           // x = xh + xl, both FP16 (round toward zero)
+    const auto pl = __builtin_amdgcn_cvt_pkrtz(v[0] - (float)ph[0], v[1] - (float)ph[1]);
+    uint32_t* o = xp + ((size_t)(id >> 10) * 8u * 64u + lane) * 4u + (c & 3u);     // piece 0 of this lane, element c & 3
+    o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
+    o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+}
 
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const int* __restrict__ tok,
-                       float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t ldy,
-                       uint32_t xrows, uint32_t g_base, uint32_t g_rem) {
+gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, float* __restrict__ y,
+                       uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
-    float* red = reinterpret_cast<float*>(lds + kStageBase);               // [8 waves][kGroups][64 lanes][4], over the staging areas
+    float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][64 lanes][4]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, kq = lane >> 4;
@@ -53,14 +99,12 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
     const uint64_t remain = (uint64_t)(rows - g0 * 16u) * row_bytes;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(W + (size_t)g0 * 16u * row_bytes), 0, (int)(remain < 0x80000000ull ? remain : 0x80000000ull), 0x00020000);
-    const uint64_t xbytes = (uint64_t)xrows * ldx * 4u;
-    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)x, 0, (int)(xbytes < 0x80000000ull ? xbytes : 0x80000000ull), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xp, 0, (int)(bpr * 128u * 128u), 0x00020000);
 
-    float* stage = reinterpret_cast<float*>(lds + kStageBase + wave * kStageBytes);
-
-    float breg[2][64];                     // activations of this wavefront's two blocks, token li, chunks kq and kq+4
-    v4f acc[kGroups][2];                   // two accumulation chains per group: consecutive MFMAs do not wait for each other
+    // activations of this wavefront's two blocks, token li, chunks kq and kq+4: FP16 pairs (positions 2c, 2c+1),
+    // high parts and low parts
+    uint32_t bh[2][2][16], bl[2][2][16];
+    v4f acc[kGroups];
     const uint32_t lanebase = (lane & 31u) * 8u;
 
     u32x4 wv[2][2][2];                     // [buffer][block of the pair][half]
@@ -76,26 +120,17 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
         }
     };
 
-    // Nibble p = 32*(kq + 4h) + s of a block holds weight i = q + q/63 with q = p - 4 (p < 4: the scale).
-    // Inside a chunk q/63 steps at most once, at s = thr[h]; below it the weight index is base[h] + s.
-    int32_t gbase[2], gthr[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const int32_t q0 = 32 * (int32_t)(kq + 4u * h) - 4;
-        const int32_t c0 = q0 >= 0 ? q0 / 63 : 0;
-        const int32_t t = 63 * (c0 + 1) - q0;                              // first s with q/63 == c0 + 1
-        gbase[h] = q0 + c0;
-        gthr[h] = t < 32 ? t : 32;
-    }
-
     issue_group(0, g0, 0);                 // weights of the first group fly during the set-up
-    {   // pair table from literals (see gemv_oil4.hip)
-        const float lv_lane = level_literal(lane & 15u);
-        const float lo_fix = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+    {   // pair table from literals: entry of byte v = (b << 4 | a), lane copy c at byte v*256 + c*8 =
+        // { Lh[a] | Lh[b] << 16, Ll[a] | Ll[b] << 16 }; thread tid writes float4 number tid + 512*k (two copies of
+        // one entry): a = (tid >> 4) & 15 is fixed, b = (tid >> 8) + 2k is uniform across the wavefront
+        const uint32_t lv_lane = split_level(level_literal(lane & 15u));
+        const uint32_t pa = split_level(level_literal((tid >> 4) & 15u));
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((tid >> 8) + 2u * k)));
-            reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
+            const uint32_t pb = (uint32_t)__builtin_amdgcn_readlane((int)lv_lane, (int)((tid >> 8) + 2u * k));
+            const uint32_t e_hi = (pa & 0xFFFFu) | (pb << 16), e_lo = (pa >> 16) | (pb & 0xFFFF0000u);
+            reinterpret_cast<uint4*>(tab)[tid + 512u * k] = make_uint4(e_hi, e_lo, e_hi, e_lo);
         }
     }
     bool table_synced = false;
@@ -103,59 +138,29 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
     for (uint32_t tile = 0; tile < ntiles; ++tile) {
         const uint32_t tg0 = g0 + tile * kGroups;
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) { acc[g][0] = v4f{0.f, 0.f, 0.f, 0.f}; acc[g][1] = v4f{0.f, 0.f, 0.f, 0.f}; }
+        for (int g = 0; g < kGroups; ++g) acc[g] = v4f{0.f, 0.f, 0.f, 0.f};
         for (uint32_t pass = 0; pass < npass; ++pass) {
             if (tile > 0 || pass > 0) issue_group(0, tg0, pass);
             if (npass > 1 || tile == 0) {
-                // ---- activations of this wavefront's two blocks -> registers.  The wavefront copies them in natural
-                // order (one 16-byte store per lane and token) into its own staging area, half a block at a time,
-                // and every lane then picks the 32 values of its token and chunk, skipping slot weights.
-                if (tile > 0) __syncthreads();                             // partial sums of the previous tile have been read
+                // ---- split activations of this wavefront's two blocks -> registers: 8 loads of 16 bytes per block half
 #pragma unroll
                 for (int b2 = 0; b2 < 2; ++b2) {
                     const uint32_t blk = pass * 16u + wave * 2u + b2;
 #pragma unroll
-                    for (int h = 0; h < 2; ++h) {                          // weights 0..131 and 124..255 of the block
-                        u32x4 xv[16];
+                    for (int h = 0; h < 2; ++h) {
+                        const uint32_t off = blk < bpr ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
 #pragma unroll
-                        for (int t = 0; t < 16; ++t) {
-                            const int m = m0 + t;
-                            const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
-                            xv[t] = __builtin_amdgcn_raw_buffer_load_b128(
-                                xrsrc, (lane < 33u && blk < bpr && src < xrows) ? src * ldx * 4u + (blk * 256u + h * 124u + lane * 4u) * 4u : kOobOffset, 0, 0);
+                        for (int j = 0; j < 4; ++j) {
+                            const u32x4 vh = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 1024u * j, 0, 0);
+                            const u32x4 vl = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 4096u + 1024u * j, 0, 0);
+                            bh[b2][h][4 * j] = vh.x; bh[b2][h][4 * j + 1] = vh.y; bh[b2][h][4 * j + 2] = vh.z; bh[b2][h][4 * j + 3] = vh.w;
+                            bl[b2][h][4 * j] = vl.x; bl[b2][h][4 * j + 1] = vl.y; bl[b2][h][4 * j + 2] = vl.z; bl[b2][h][4 * j + 3] = vl.w;
                         }
-                        if (lane < 33u) {
-#pragma unroll
-                            for (int t = 0; t < 16; ++t)
-                                *reinterpret_cast<u32x4*>(stage + t * kTokStride + lane * 4u) = xv[t];
-                        }
-                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                        __builtin_amdgcn_wave_barrier();
-                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                        {
-                            // LDS byte address of the value below the step of q/63; from the step on it is one float
-                            // further.  The address is made opaque so that the 64 element addresses are formed here,
-                            // next to their reads, instead of being precomputed for the whole kernel.
-                            uint32_t lo = (uint32_t)(kStageBase + wave * kStageBytes) + (li * kTokStride + (uint32_t)(gbase[h] - h * 124)) * 4u;
-                            asm volatile("" : "+v"(lo));
-                            const uint32_t thr = (uint32_t)gthr[h];
-#pragma unroll
-                            for (int sI = 0; sI < 32; ++sI) {
-                                const uint32_t a = ((uint32_t)sI >= thr ? lo + 4u : lo) + 4u * sI;
-                                const float v = *(lds_cfloat*)(uintptr_t)a;
-                                if (h == 0 && sI < 4) breg[b2][sI] = kq == 0u ? 0.f : v;        // nibbles 0..3 of a block: its scale
-                                else breg[b2][32 * h + sI] = v;
-                            }
-                        }
-                        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                        __builtin_amdgcn_wave_barrier();
-                        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                     }
                 }
             }
             if (!table_synced) { __syncthreads(); table_synced = true; }   // the level table is complete
             // ---- main loop: groups of the tile, two blocks each -------------------------------------------
-            LevelPair lv[16];
 #pragma unroll
             for (int g = 0; g < kGroups; ++g) {
                 if (g + 1 < kGroups) issue_group((g + 1) & 1, tg0 + g + 1, pass);
@@ -165,18 +170,40 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
                     const bool on = g_on && pass * 16u + wave * 2u + b2 < bpr;     // wave-uniform
                     if (!on) continue;
                     const u32x4 w0 = wv[g & 1][b2][0], w1 = wv[g & 1][b2][1];
-                    const uint32_t sbits = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(li * 4u), (int)w0.x) & 0xFFFFu;
-                    const float scale = __half2float(__ushort_as_half((unsigned short)sbits));
+                    v4f t0 = v4f{0.f, 0.f, 0.f, 0.f}, t1 = v4f{0.f, 0.f, 0.f, 0.f};   // this block: Lh xh, and Lh xl + Ll xh
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {
-                        lookup_load(h == 0 ? w0 : w1, lanebase, lv);
-                        __builtin_amdgcn_sched_barrier(0);                 // all 16 table reads in flight before the first multiply
+                        const u32x4 wh = h == 0 ? w0 : w1;
+                        const uint32_t wd[4] = {wh.x, wh.y, wh.z, wh.w};
+                        uint32_t ah[16], al[16];
 #pragma unroll
-                        for (int k = 0; k < 16; ++k) {
-                            acc[g][0] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].lo * scale, breg[b2][32 * h + 2 * k], acc[g][0], 0, 0, 0);
-                            acc[g][1] = __builtin_amdgcn_mfma_f32_16x16x4f32(lv[k].hi * scale, breg[b2][32 * h + 2 * k + 1], acc[g][1], 0, 0, 0);
+                        for (int d = 0; d < 4; ++d) {
+#pragma unroll
+                            for (int J = 0; J < 4; ++J) {
+                                const uint32_t addr = __builtin_amdgcn_perm(wd[d], lanebase, 0x0C0C0000u | ((4u + J) << 8));
+                                const u32x2 e = *(lds_cu32x2*)(uintptr_t)addr;
+                                ah[4 * d + J] = e.x; al[4 * d + J] = e.y;
+                            }
+                        }
+                        __builtin_amdgcn_sched_barrier(0);                 // all 16 table reads in flight before the first product
+#pragma unroll
+                        for (int d = 0; d < 4; ++d) {
+                            const h8 Ah = __builtin_bit_cast(h8, u32x4{ah[4 * d], ah[4 * d + 1], ah[4 * d + 2], ah[4 * d + 3]});
+                            const h8 Al = __builtin_bit_cast(h8, u32x4{al[4 * d], al[4 * d + 1], al[4 * d + 2], al[4 * d + 3]});
+                            const h8 Bh = __builtin_bit_cast(h8, u32x4{bh[b2][h][4 * d], bh[b2][h][4 * d + 1], bh[b2][h][4 * d + 2], bh[b2][h][4 * d + 3]});
+                            const h8 Bl = __builtin_bit_cast(h8, u32x4{bl[b2][h][4 * d], bl[b2][h][4 * d + 1], bl[b2][h][4 * d + 2], bl[b2][h][4 * d + 3]});
+                            t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bh, t0, 0, 0, 0);
+                            t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bl, t1, 0, 0, 0);
+                            t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, Bh, t1, 0, 0, 0);
                         }
                         __builtin_amdgcn_sched_barrier(0);
+                    }
+                    // the block's FP16 scale of row r sits in the low half of the first dword of lane r (kq = 0)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const uint32_t sbits = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((4u * kq + v) * 4u), (int)w0.x) & 0xFFFFu;
+                        const float scale = __half2float(__ushort_as_half((unsigned short)sbits));
+                        acc[g][v] = __fmaf_rn(t0[v] + t1[v], scale, acc[g][v]);
                     }
                 }
             }
@@ -185,7 +212,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
         __syncthreads();
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) {
-            const v4f d = acc[g][0] + acc[g][1];
+            const v4f d = acc[g];
             *reinterpret_cast<float4*>(red + (((size_t)wave * kGroups + g) * 64 + lane) * 4) = make_float4(d[0], d[1], d[2], d[3]);
         }
         __syncthreads();
@@ -201,8 +228,25 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
                 y[(size_t)(m0 + j) * ldy + r] = s;
             }
         }
-        if (tile + 1 < ntiles && npass == 1) __syncthreads();              // red is rewritten by the next tile
+        if (tile + 1 < ntiles) __syncthreads();                            // red is rewritten by the next tile
     }
+}
+
+
+// device scratch for the packed activations of one pass (one per process and device; calls that overlap on one
+// device race on it, like the prefill GEMM's)
+std::mutex g_xp_mu;
+uint32_t* g_xp[64] = {};
+constexpr uint32_t kMaxPackCols = 32768;
+
+int get_pack_buffer(uint32_t** out) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_xp_mu);
+    if (!g_xp[dev]) OILHIP_HIP(hipMalloc(&g_xp[dev], (size_t)(kMaxPackCols >> 8) * 128u * 128u));
+    *out = g_xp[dev];
+    return OILHIP_OK;
 }
 
 }  // namespace
@@ -211,22 +255,27 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const float* __restrict__ 
 // Returns 1 when the shape is outside what this kernel covers.
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s) {
-    if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
+    if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
     static bool attr_done = false;
     if (!attr_done) {
         OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
-    const size_t lds_bytes = (size_t)kStageBase + 8 * (size_t)kStageBytes + 64;   // table, then staging areas / partial sums
-    static_assert(8 * kStageBytes >= 8 * kGroups * 64 * 16, "the staging areas must cover the partial sums");
+    uint32_t* xp = nullptr;
+    if (int rc = get_pack_buffer(&xp)) return rc;
+    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
     const uint32_t groups = ((uint32_t)w.rows + 15u) / 16u;
     uint32_t grid = (uint32_t)device_cu_count();
     if (grid > groups) grid = groups;
+    const uint32_t bpr = (uint32_t)(w.cols >> 8);
     for (int m0 = 0; m0 < M; m0 += 16) {          // passes of at most 16 tokens
         const int m1 = M - m0 < 16 ? M : m0 + 16;
-        hipLaunchKernelGGL(gemv_oil4_multi_kernel, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, d_x, d_tok, d_y,
-                           (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldx, ldy, xrows, groups / grid, groups % grid);
+        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_tok, xp, (uint32_t)w.cols, m0, m1,
+                           ldx, xrows);
+        OILHIP_HIP(hipGetLastError());
+        hipLaunchKernelGGL(gemv_oil4_multi_kernel, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
+                           (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
         OILHIP_HIP(hipGetLastError());
     }
     return OILHIP_OK;
