@@ -343,6 +343,32 @@ def bench_prefill(torch, ia, payload, blocks):
                 torch.cuda.synchronize()
                 t = e0.elapsed_time(e1) * 1e-3 / 20
                 out[f"prefill_M{M}_N{rows}_TFLOPs"] = round(2.0 * M * rows * cols / t / 1e12, 1)
+    # what this box reaches with a plain bf16 GEMM of the largest shape (rocBLAS / hipBLASLt through torch), and with a
+    # plain device-to-device copy: the practical ceilings next to the vendor peaks
+    a = torch.randn(2048, 4096, device="cuda").to(torch.bfloat16)
+    b = torch.randn(11008, 4096, device="cuda").to(torch.bfloat16)
+    for _ in range(3):
+        torch.matmul(a, b.t())
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(20):
+        torch.matmul(a, b.t())
+    e1.record()
+    torch.cuda.synchronize()
+    out["plain_bf16_gemm_M2048_N11008_TFLOPs"] = round(2.0 * 2048 * 11008 * 4096 / (e0.elapsed_time(e1) * 1e-3 / 20) / 1e12, 1)
+    src = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()
+    dst = torch.empty_like(src)
+    for _ in range(2):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(5):
+        dst.copy_(src)
+    e1.record()
+    torch.cuda.synchronize()
+    out["plain_copy_1GiB_read_plus_write_GBps"] = round(2.0 * src.numel() * 4 / (e0.elapsed_time(e1) * 1e-3 / 5) / 1e9, 1)
     return out
 
 
