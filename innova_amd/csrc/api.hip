@@ -301,10 +301,13 @@ int oilhip_dequant_f32(const oilhip_weights* w, float* d_out, void* stream) {
 int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
     if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
     if (w->uniform_fmt == OILHIP_OIL4 && w->uniform_stride == 128) {
-        int rc = M <= 4 ? launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream) : 1;      // 1: shape not covered
+        // one or two rows: the register-resident kernel; from three on the matrix-core kernel (16 rows per pass) is faster
+        int rc = 1;                                                                          // 1: shape not covered
+        if (M <= 2) rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
         if (rc == 1 && M >= 2)
             rc = launch_gemv_oil4_multi(*w, d_x, nullptr, d_y, M, (uint32_t)w->cols, (uint32_t)w->rows, (uint32_t)M,
                                         (hipStream_t)stream);
+        if (rc == 1 && M > 2 && M <= 4) rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
     if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256 && M <= 4) {

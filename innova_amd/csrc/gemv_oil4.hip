@@ -422,7 +422,7 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     if (grid == 0) grid = 1;
     const uint32_t Jn = grid * G;
     const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
-    const int budget = MB >= 4 ? 3 : 12 / best_cs;                 // wave-loads in flight per wave (register budget)
+    const int budget = 12 / best_cs;                               // wave-loads in flight per wave (register budget)
     int rpw = 1;
     if (max_rows <= (uint32_t)budget) {                            // one chunk: the smallest that holds every row
         for (int cand : {1, 2, 3, 4, 6, 12}) if ((uint32_t)cand >= max_rows) { rpw = cand; break; }
@@ -465,14 +465,10 @@ int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float
 
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || M > 16) return 1;
-    Oil4Plan p;
-    const int MB = M == 1 ? 1 : (M == 2 ? 2 : 4);
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) {
-        if (MB != 4 || !make_plan((uint32_t)w.rows, (uint32_t)w.cols, 2, 8, &p)) return 1;
-        return dispatch<2>(w, d_x, nullptr, d_y, M, s, p);
-    }
-    return MB == 1 ? dispatch<1>(w, d_x, nullptr, d_y, M, s, p)
-         : MB == 2 ? dispatch<2>(w, d_x, nullptr, d_y, M, s, p) : dispatch<4>(w, d_x, nullptr, d_y, M, s, p);
+    Oil4Plan p;                                   // rows beyond two go in passes of two (the matrix-core kernel is the
+    const int MB = M == 1 ? 1 : 2;                // better choice there and the caller tries it first)
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) return 1;
+    return MB == 1 ? dispatch<1>(w, d_x, nullptr, d_y, M, s, p) : dispatch<2>(w, d_x, nullptr, d_y, M, s, p);
 }
 
 // y = W . (silu(h[0..K)) * h[K..2K)) for one activation row h of 2K floats.  Returns 1 when the shape is not covered.
