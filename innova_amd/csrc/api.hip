@@ -7,6 +7,7 @@
 #include <vector>
 
 #include "common.h"
+#include "run_decode.h"
 
 namespace oilhip {
 
@@ -101,6 +102,111 @@ int oilhip_probe(int* gfx, uint64_t* hbm_bytes, int* compute_units, char* name, 
     return OILHIP_OK;
 }
 
+// Mixed-format tensors of full blocks: rewrite `pay` as the window streams the segmented GEMV reads (layout in
+// common.h, SegLayout) and point the descriptors at the blocks' new places.  Leaves everything as it is when the
+// tensor does not fit the scheme.
+static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, uint64_t rows, uint64_t cols,
+                                SegLayout& g) {
+    const uint64_t bpr = cols / 256, nblocks = db.size();
+    if ((cols & 255) || bpr < 1 || bpr > 4096 || nblocks != rows * bpr || rows > 0x7FFFFFFFull) return;
+    int slot_of[OILHIP_NUM_FORMATS];
+    for (int& v : slot_of) v = -1;
+    bool present[OILHIP_NUM_FORMATS] = {};
+    for (const DevBlock& d : db) present[d.fmt] = true;
+    uint32_t nf = 0;
+    for (int f = 0; f < OILHIP_NUM_FORMATS; ++f)
+        if (present[f]) {
+            if (nf == (uint32_t)kSegMaxFormats) return;
+            slot_of[f] = (int)nf;
+            g.fmt[nf++] = (uint32_t)f;
+        }
+    bool seen[kSegMaxFormats] = {};
+    for (const DevBlock& d : db) {                     // a format's full blocks must all have the same channel sizes
+        const int s = slot_of[d.fmt];
+        if (!seen[s]) {
+            seen[s] = true;
+            g.cb_bytes[s] = d.cb_bytes;
+            g.idx_bytes[s] = d.idx_bytes;
+            g.stride[s] = ((uint32_t)d.cb_bytes + d.idx_bytes + 15u) & ~15u;
+            if (g.stride[s] + 64u > kSegWindow) return;
+        } else if (g.cb_bytes[s] != d.cb_bytes || g.idx_bytes[s] != d.idx_bytes) {
+            return;
+        }
+    }
+    const uint32_t ns = (uint32_t)std::min<uint64_t>(rows, (uint64_t)device_cu_count() * 8);   // streams: two per SIMD
+    struct Entry { uint32_t slot, flags, nblk, data_off, tag_off, row0, nrows; };
+    struct Window { std::vector<Entry> ent; std::vector<uint16_t> tags; std::vector<uint32_t> src; uint32_t data = 0; };
+    auto bytes_of = [](size_t ne, size_t nb, uint32_t data) { return 16 + 16 * ne + ((2 * nb + 15) & ~(size_t)15) + data; };
+    std::vector<std::vector<Window>> streams(ns);
+    for (uint32_t st = 0; st < ns; ++st) {
+        std::vector<Window>& ws = streams[st];
+        ws.emplace_back();
+        // the stream's rows in tiles of at most kSegTileRows, as even as they come
+        const uint64_t ra = (uint64_t)st * rows / ns, rb = (uint64_t)(st + 1) * rows / ns;
+        const uint64_t nt = (rb - ra + kSegTileRows - 1) / kSegTileRows;
+        for (uint64_t t = 0; t < nt; ++t) {
+            const uint64_t r0 = ra + t * (rb - ra) / nt, r1 = ra + (t + 1) * (rb - ra) / nt;
+            Entry* last = nullptr;
+            for (uint32_t s = 0; s < nf; ++s) {
+                bool open = false;                     // an entry of this tile and slot is open in the current window
+                for (uint64_t r = r0; r < r1; ++r)
+                    for (uint64_t c = 0; c < bpr; ++c) {
+                        const uint32_t b = (uint32_t)(r * bpr + c);
+                        if (slot_of[db[b].fmt] != (int)s) continue;
+                        Window* w = &ws.back();
+                        if (bytes_of(w->ent.size() + (open ? 0 : 1), w->tags.size() + 1, w->data + g.stride[s]) > kSegWindow) {
+                            ws.emplace_back();
+                            w = &ws.back();
+                            open = false;
+                        }
+                        if (!open) {
+                            w->ent.push_back(Entry{s, 0u, 0u, w->data, (uint32_t)w->tags.size(), (uint32_t)r0, (uint32_t)(r1 - r0)});
+                            open = true;
+                        }
+                        last = &w->ent.back();
+                        ++last->nblk;
+                        w->tags.push_back((uint16_t)(((r - r0) << 12) | c));
+                        w->src.push_back(b);
+                        w->data += g.stride[s];
+                    }
+            }
+            last->flags |= 1u;                         // every tile has blocks: its last entry closes it
+        }
+    }
+    size_t maxw = 1;
+    for (const auto& ws : streams) maxw = std::max(maxw, ws.size());
+    const uint64_t stride = (uint64_t)maxw * kSegWindow, total = stride * ns;
+    if ((total >> 4) > 0xFFFFFFFFull) return;
+    std::vector<uint8_t> out(total, 0);
+    for (uint32_t st = 0; st < ns; ++st)
+        for (size_t wi = 0; wi < streams[st].size(); ++wi) {
+            const Window& w = streams[st][wi];
+            uint8_t* base = out.data() + st * stride + wi * kSegWindow;
+            const uint32_t tag_base = 16u + 16u * (uint32_t)w.ent.size();
+            const uint32_t data_base = tag_base + (uint32_t)((2 * w.tags.size() + 15) & ~(size_t)15);
+            const uint32_t hdr[4] = {(uint32_t)w.ent.size(), (uint32_t)streams[st].size(), 0u, 0u};
+            std::memcpy(base, hdr, 16);
+            for (size_t i = 0; i < w.ent.size(); ++i) {
+                const Entry& e = w.ent[i];
+                const uint32_t rec[4] = {e.slot | (g.fmt[e.slot] << 4) | (e.flags << 8) | (e.nblk << 16),
+                                         (data_base + e.data_off) | ((tag_base + 2u * e.tag_off) << 16), e.row0, e.nrows};
+                std::memcpy(base + 16 + 16 * i, rec, 16);
+            }
+            std::memcpy(base + tag_base, w.tags.data(), 2 * w.tags.size());
+            uint32_t at = data_base;
+            for (uint32_t b : w.src) {
+                DevBlock& d = db[b];
+                std::memcpy(base + at, pay.data() + (size_t)d.off16 * 16, (size_t)d.cb_bytes + d.idx_bytes);
+                d.off16 = (uint32_t)((st * stride + wi * kSegWindow + at) >> 4);
+                at += g.stride[slot_of[d.fmt]];
+            }
+        }
+    pay.swap(out);
+    g.nf = nf;
+    g.nstreams = ns;
+    g.stream_bytes = stride;
+}
+
 static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vector<uint64_t>& out_off,
                   uint64_t algo_bytes, uint64_t rows, uint64_t cols, oilhip_weights** out) {
     const uint32_t nblocks = (uint32_t)db.size();
@@ -122,6 +228,7 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
     };
     hipError_t e;
     if ((e = hipGetDevice(&w->device)) != hipSuccess) return bail(e, "hipGetDevice");
+    if (all_full && !uniform) pack_window_streams(pay, db, rows, cols, w->seg);
     // 64 spare bytes so vector loads that straddle the end of the last block stay in bounds
     w->alloc_bytes = pay.size() + 64;
     if ((e = hipMalloc(&w->d_payload, w->alloc_bytes)) != hipSuccess) return bail(e, "hipMalloc(payload)");
@@ -132,21 +239,6 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
         if ((e = hipMalloc(&w->d_blocks, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(blocks)");
         if ((e = hipMemcpy(w->d_blocks, db.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
             return bail(e, "hipMemcpy(blocks)");
-        const uint64_t bpr = cols / 256;
-        if (all_full && !uniform && (cols & 255) == 0 && bpr >= 2 && bpr <= 0xFFFFFFFFull && (uint64_t)nblocks == rows * bpr) {
-            // The all-format GEMV takes 8 consecutive descriptors per step and runs every format present among them;
-            // with each row's blocks ordered by format most steps see one format only.  Order within a format stays
-            // by column (stable), so the result does not depend on anything but the tensor.
-            std::vector<DevBlock> sorted(db);
-            for (uint64_t r = 0; r < rows; ++r) {
-                DevBlock* row = sorted.data() + r * bpr;
-                for (uint64_t c = 0; c < bpr; ++c) row[c].nw = (uint32_t)c;
-                std::stable_sort(row, row + bpr, [](const DevBlock& a, const DevBlock& b) { return a.fmt < b.fmt; });
-            }
-            if ((e = hipMalloc(&w->d_sorted, sizeof(DevBlock) * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(sorted blocks)");
-            if ((e = hipMemcpy(w->d_sorted, sorted.data(), sizeof(DevBlock) * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
-                return bail(e, "hipMemcpy(sorted blocks)");
-        }
         if (!all_full) {
             if ((e = hipMalloc(&w->d_out_off, 8 * (size_t)nblocks)) != hipSuccess) return bail(e, "hipMalloc(out_off)");
             if ((e = hipMemcpy(w->d_out_off, out_off.data(), 8 * (size_t)nblocks, hipMemcpyHostToDevice)) != hipSuccess)
@@ -229,7 +321,6 @@ int oilhip_weights_destroy(oilhip_weights* w) {
     if (!w) return OILHIP_OK;
     if (w->d_payload) (void)hipFree(w->d_payload);
     if (w->d_blocks) (void)hipFree(w->d_blocks);
-    if (w->d_sorted) (void)hipFree(w->d_sorted);
     if (w->d_out_off) (void)hipFree(w->d_out_off);
     delete w;
     return OILHIP_OK;
@@ -312,6 +403,10 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
     }
     if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256 && M <= 4) {
         const int rc = launch_gemv_oil8(*w, d_x, d_y, M, (hipStream_t)stream);
+        if (rc <= 0) return rc;
+    }
+    if (w->seg.nstreams) {
+        const int rc = launch_gemv_seg(*w, d_x, d_y, M, (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
     const int rc = launch_gemv_runs(*w, d_x, d_y, M, (hipStream_t)stream);

@@ -25,6 +25,22 @@ int fail(int code, const std::string& msg);
 int get_tables(const DecodeTables** out);
 int device_cu_count();
 
+// Tensors whose rows mix formats are stored as `nstreams` streams of 4 KB windows, stream s at byte s * stream_bytes
+// of the payload buffer, one wavefront per stream (gemv_seg.hip).  A stream covers a contiguous range of rows in tiles
+// of at most kSegTileRows; inside a tile the blocks are ordered by format (in the order of `fmt`), inside a format by
+// row and column.  Window: 4 dwords {entries, windows of the stream, 0, 0}; per entry 4 dwords
+// {slot | format << 4 | closes its tile << 8 | blocks << 16, byte offset of the blocks | byte offset of their tags << 16,
+// first row of the tile, rows of the tile}; the tags (per block: row of the tile << 12 | column block); the blocks,
+// 16-byte aligned, whole.
+constexpr int kSegMaxFormats = 15;
+constexpr uint32_t kSegWindow = 4096;
+constexpr int kSegTileRows = 4;
+struct SegLayout {
+    uint32_t nf = 0, nstreams = 0;
+    uint64_t stream_bytes = 0;
+    uint32_t fmt[kSegMaxFormats] = {}, cb_bytes[kSegMaxFormats] = {}, idx_bytes[kSegMaxFormats] = {}, stride[kSegMaxFormats] = {};
+};
+
 }  // namespace oilhip
 
 // The handle behind oilhip_weights*.
@@ -32,8 +48,7 @@ struct oilhip_weights {
     int device = 0;
     uint8_t* d_payload = nullptr;           // block payloads, each 16-byte aligned
     oilhip::DevBlock* d_blocks = nullptr;   // one descriptor per block
-    oilhip::DevBlock* d_sorted = nullptr;   // mixed-format tensors of full blocks: each row's descriptors ordered by format,
-                                            // the block's column index in `nw` (rows keep their place)
+    oilhip::SegLayout seg;                  // mixed-format tensors of full blocks: tile- and format-ordered storage
     uint64_t* d_out_off = nullptr;          // first output index per block (only when nw varies)
     uint64_t alloc_bytes = 0;               // size of d_payload
     uint64_t payload_bytes = 0;             // sum of cb_bytes + idx_bytes
@@ -62,7 +77,9 @@ int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_ac
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s);
-// every format and mixed rows, a lane per run of 32 weights
+// rows that mix formats, stored tile by tile and format by format
+int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
+// every format, a lane per run of 32 weights
 int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
 }  // namespace oilhip

@@ -13,20 +13,12 @@
 // in format diverge by 8-lane group only.  Formats without a short routine go through the
 // general per-weight decoder.
 #include "common.h"
+#include "run_decode.h"
 
 namespace oilhip {
 namespace {
 
 constexpr int kRunPad = 36;                // floats per run of 32 activations in LDS
-
-__device__ __forceinline__ float f16_bits(uint32_t h) { return half_bits_to_float(h & 0xFFFFu); }
-
-// 32-bit window starting `sh` bits into the dword pair (lo, hi)
-__device__ __forceinline__ uint32_t funnel(uint32_t lo, uint32_t hi, uint32_t sh) {
-    return __builtin_amdgcn_alignbit(hi, lo, sh);       // (hi:lo >> (sh & 31)) low dword
-}
-
-struct LdsTables { const float* lv2; const float* lv4; const float* lv8; const float* t255; };   // copies in LDS
 
 struct Run {                                // what a lane needs to know about its run
     const uint8_t* cb;                      // block payload: codebook channel, then index channel
@@ -34,132 +26,36 @@ struct Run {                                // what a lane needs to know about i
     uint32_t fmt, r;                        // format id, run 0..7 inside the block
 };
 
-// Decodes the lane's 32 weights.  Returns false when the run was handled as OIL1 (w untouched,
-// *mean set).  Bit layouts follow dequantize_block_all for full 256-weight blocks.
+template <int FMT>
+__device__ __forceinline__ void decode_one(const Run& R, const DecodeTables* __restrict__ T, const LdsTables& L, float (&w)[32]) {
+    uint32_t raw[run_raw_dwords(FMT)];
+    fetch_run<FMT>(R.cb, R.cb_bytes, R.r, raw);
+    expand_run<FMT>(raw, R.cb, R.cb_bytes, R.idx_bytes, R.r, T, L, w);
+}
+
+// Decodes the lane's 32 weights.  Returns false when the run was handled as OIL1 (w untouched, *mean set).
 __device__ __forceinline__ bool decode_run(const Run& R, const DecodeTables* __restrict__ T, const LdsTables& L, float (&w)[32], float* mean) {
-    const uint8_t* idx = R.cb + R.cb_bytes;
-    const uint32_t r = R.r;
     switch (R.fmt) {
-        case 0: {   // OIL1: FP16 mean of the run (:615-626)
-            *mean = f16_bits(*reinterpret_cast<const uint16_t*>(R.cb + 2 * r));
+        case 0: {
+            uint32_t raw[1];
+            fetch_run<0>(R.cb, R.cb_bytes, R.r, raw);
+            *mean = oil1_mean(raw);
             return false;
         }
-        case 1: {   // SPARK_Q0: FP16 scale + 32 sign bits per run (:643-654)
-            const uint16_t* p = reinterpret_cast<const uint16_t*>(idx + 6 * r);
-            const uint32_t sbits = __float_as_uint(f16_bits(p[0]));
-            const uint32_t neg = ~((uint32_t)p[1] | ((uint32_t)p[2] << 16));       // bit set -> weight is -scale
-#pragma unroll
-            for (int k = 0; k < 32; ++k)    // magnitude of the scale, sign from bit k
-                w[k] = __uint_as_float((sbits & 0x7FFFFFFFu) | (((neg << (31 - k)) & 0x80000000u) ^ (sbits & 0x80000000u)));
-            return true;
-        }
-        case 2: case 3: case 4: {   // OIL2 / OIL4 / OIL8: block scale, fixed-width indices, slots own no bits (:173-182)
-            const uint32_t bits = R.fmt == 2 ? 2u : (R.fmt == 3 ? 4u : 8u);
-            const uint32_t period = 16u * bits;                                    // one slot per `period` weights
-            const uint32_t b0 = 16u + bits * (32u * r - (32u * r) / period);
-            const bool last_is_slot = ((32u * (r + 1)) % period) == 0u;
-            const float scale = f16_bits(*reinterpret_cast<const uint16_t*>(idx));
-            const uint32_t* q = reinterpret_cast<const uint32_t*>(idx) + (b0 >> 5);
-            const uint32_t sh = b0 & 31u;
-            if (bits == 4u) {
-                uint32_t d[5];
-#pragma unroll
-                for (int j = 0; j < 5; ++j) d[j] = q[j];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t v = funnel(d[j], d[j + 1], sh);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) w[8 * j + e] = L.lv4[(v >> (4 * e)) & 15u] * scale;
-                }
-            } else if (bits == 2u) {
-                uint32_t d[3];
-#pragma unroll
-                for (int j = 0; j < 3; ++j) d[j] = q[j];
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t v = funnel(d[j], d[j + 1], sh);
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) w[16 * j + e] = L.lv2[(v >> (2 * e)) & 3u] * scale;
-                }
-            } else {
-                uint32_t d[9];
-#pragma unroll
-                for (int j = 0; j < 9; ++j) d[j] = q[j];
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t v = funnel(d[j], d[j + 1], sh);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) w[4 * j + e] = L.lv8[(v >> (8 * e)) & 255u] * scale;
-                }
-            }
-            if (last_is_slot) w[31] = 0.0f;
-            return true;
-        }
-        case 9: case 10: case 11: {   // grouped lattice: per 64 weights FP16 zero point + FP16 scale (:308-331)
-            const uint32_t bits = R.fmt == 9 ? 2u : (R.fmt == 10 ? 4u : 8u);
-            const uint32_t gbytes = 4u + 8u * bits;
-            const uint8_t* g = idx + (r >> 1) * gbytes;
-            const uint32_t hdr = *reinterpret_cast<const uint32_t*>(g);
-            const float zp = f16_bits(hdr), sc = f16_bits(hdr >> 16);
-            const uint32_t* q = reinterpret_cast<const uint32_t*>(g + 4 + (r & 1u) * 4u * bits);
-            if (sc == 0.0f) {
-#pragma unroll
-                for (int k = 0; k < 32; ++k) w[k] = zp;
-            } else if (bits == 4u) {
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const uint32_t v = q[j];
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) w[8 * j + e] = __fmaf_rn(L.lv4[(v >> (4 * e)) & 15u], sc, zp);
-                }
-            } else if (bits == 2u) {
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const uint32_t v = q[j];
-#pragma unroll
-                    for (int e = 0; e < 16; ++e) w[16 * j + e] = __fmaf_rn(L.lv2[(v >> (2 * e)) & 3u], sc, zp);
-                }
-            } else {
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const uint32_t v = q[j];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) w[4 * j + e] = __fmaf_rn(L.t255[(v >> (8 * e)) & 255u], sc, zp);
-                }
-            }
-            return true;
-        }
-        case 5: case 12: {   // OIL16 / OIL16_GRP: FP16 weights (:588-596)
-            const uint32_t* q = reinterpret_cast<const uint32_t*>(idx + 64 * r);
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const uint32_t v = q[j];
-                w[2 * j] = f16_bits(v);
-                w[2 * j + 1] = f16_bits(v >> 16);
-            }
-            return true;
-        }
-        case 6: {   // OIL32: raw FP32 (:585-587)
-            const uint32_t* q = reinterpret_cast<const uint32_t*>(idx + 128 * r);
-#pragma unroll
-            for (int k = 0; k < 32; ++k) w[k] = __uint_as_float(q[k]);
-            return true;
-        }
-        case 7: {   // OIL1_GRP: block scale, sign bits, every 16th weight is a slot (:627-642)
-            const float scale = f16_bits(*reinterpret_cast<const uint16_t*>(idx));
-            const uint32_t b0 = 16u + 30u * r;                                     // 30 coded weights per run
-            const uint32_t* q = reinterpret_cast<const uint32_t*>(idx) + (b0 >> 5);
-            const uint32_t v = funnel(q[0], q[1], b0 & 31u);
-#pragma unroll
-            for (int k = 0; k < 32; ++k) {
-                const int code = k - (k >= 15 ? 1 : 0);                            // weights 15 and 31 of a run are slots
-                w[k] = (k == 15 || k == 31) ? 0.0f : (((v >> code) & 1u) ? scale : -scale);
-            }
-            return true;
-        }
+        case 1: decode_one<1>(R, T, L, w); return true;
+        case 2: decode_one<2>(R, T, L, w); return true;
+        case 3: decode_one<3>(R, T, L, w); return true;
+        case 4: decode_one<4>(R, T, L, w); return true;
+        case 5: decode_one<5>(R, T, L, w); return true;
+        case 6: decode_one<6>(R, T, L, w); return true;
+        case 7: decode_one<7>(R, T, L, w); return true;
+        case 9: decode_one<9>(R, T, L, w); return true;
+        case 10: decode_one<10>(R, T, L, w); return true;
+        case 11: decode_one<11>(R, T, L, w); return true;
+        case 12: decode_one<12>(R, T, L, w); return true;
         default: {  // SPARK_Q0_GRP, sparse formats: the general decoder, weight by weight
             for (int k = 0; k < 32; ++k)
-                w[k] = decode_weight(R.fmt, R.cb, R.cb_bytes, idx, R.idx_bytes, 256u, 32u * r + (uint32_t)k, T);
+                w[k] = decode_weight(R.fmt, R.cb, R.cb_bytes, R.cb + R.cb_bytes, R.idx_bytes, 256u, 32u * R.r + (uint32_t)k, T);
             return true;
         }
     }
@@ -170,8 +66,7 @@ template <int MB>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3)))
 gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__ blocks, const DecodeTables* __restrict__ T,
                  const float* __restrict__ x, float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M,
-                 int uniform_fmt, uint32_t uniform_stride, uint32_t uniform_cb, uint32_t uniform_idx, uint32_t uniform_base,
-                 int sorted) {
+                 int uniform_fmt, uint32_t uniform_stride, uint32_t uniform_cb, uint32_t uniform_idx, uint32_t uniform_base) {
     extern __shared__ __align__(16) float smem[];
     const uint32_t bpr = cols >> 8, nruns = cols >> 5;
     const uint32_t xpad = nruns * kRunPad;
@@ -211,7 +106,6 @@ gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict
             if (blk < bpr) {
                 const size_t b = (size_t)row * bpr + blk;
                 Run R;
-                uint32_t colblk = blk;
                 if (uniform_fmt >= 0) {
                     R.cb = payload + uniform_base + b * uniform_stride;
                     R.cb_bytes = uniform_cb; R.idx_bytes = uniform_idx; R.fmt = (uint32_t)uniform_fmt;
@@ -219,10 +113,9 @@ gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict
                     const DevBlock d = blocks[b];
                     R.cb = payload + (size_t)d.off16 * 16;
                     R.cb_bytes = d.cb_bytes; R.idx_bytes = d.idx_bytes; R.fmt = d.fmt;
-                    if (sorted) colblk = d.nw;             // descriptors ordered by format: the block's column travels with it
                 }
                 R.r = r;
-                const uint32_t run = colblk * 8u + r;
+                const uint32_t run = blk * 8u + r;
                 float w[32], mean = 0.f;
                 if (decode_run(R, T, L, w, &mean)) {
 #pragma unroll
@@ -271,10 +164,8 @@ int launch_runs(const oilhip_weights& w, const DecodeTables* T, const float* d_x
     const uint32_t need = ((uint32_t)w.rows + 3u) / 4u;
     if (grid > need) grid = need;
     const bool uni = w.uniform_fmt >= 0 && w.uniform_stride > 0;
-    const bool sorted = !uni && w.d_sorted != nullptr;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w.d_payload, sorted ? w.d_sorted : w.d_blocks, T, d_x, d_y, (uint32_t)w.rows,
-                       (uint32_t)w.cols, m0, M, uni ? w.uniform_fmt : -1, w.uniform_stride, w.uniform_cb, w.uniform_idx, w.uniform_base,
-                       sorted ? 1 : 0);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, s, w.d_payload, w.d_blocks, T, d_x, d_y, (uint32_t)w.rows,
+                       (uint32_t)w.cols, m0, M, uni ? w.uniform_fmt : -1, w.uniform_stride, w.uniform_cb, w.uniform_idx, w.uniform_base);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }

@@ -1,0 +1,150 @@
+// run_decode.h -- one run of 32 consecutive weights of a full 256-weight block, per wire format, in two halves:
+// fetch_run<FMT> issues the loads of the run's bytes into a few registers, expand_run<FMT> turns them into 32
+// FP32 weights.  Keeping the halves apart lets a kernel fetch several runs before it expands the first.  Bit
+// layouts follow dequantize_block_all for nw = 256 (src/block_codec.cpp:576-720): dequant_lattice (:173-182),
+// dequant_grouped_lattice (:308-331), OIL1 (:615-626), OIL1_GRP (:627-642), SPARK_Q0 (:643-654), OIL16 / OIL32
+// (:585-596).  SPARK_Q0_GRP and the sparse formats go through decode_weight, weight by weight.
+#pragma once
+#include "block_decode.h"
+
+namespace oilhip {
+
+struct LdsTables { const float* lv2; const float* lv4; const float* lv8; const float* t255; };   // copies in LDS
+
+__device__ __forceinline__ float f16_bits(uint32_t h) { return half_bits_to_float(h & 0xFFFFu); }
+
+// 32-bit window starting `sh` bits into the dword pair (lo, hi)
+__device__ __forceinline__ uint32_t funnel(uint32_t lo, uint32_t hi, uint32_t sh) {
+    return __builtin_amdgcn_alignbit(hi, lo, sh);       // (hi:lo >> (sh & 31)) low dword
+}
+
+// registers a fetched run occupies
+__host__ __device__ constexpr int run_raw_dwords(int fmt) {
+    return fmt == 0 ? 1 : fmt == 1 ? 2 : fmt == 2 ? 4 : fmt == 3 ? 6 : fmt == 4 ? 10 : fmt == 5 || fmt == 12 ? 16
+         : fmt == 6 ? 32 : fmt == 7 ? 3 : fmt == 9 ? 3 : fmt == 10 ? 5 : fmt == 11 ? 9 : 1;
+}
+
+// steps of 8 blocks the segmented GEMV fetches together for a format (few registers per run: more steps)
+__host__ __device__ constexpr int seg_batch_steps(int fmt) {
+    return run_raw_dwords(fmt) <= 3 ? 4 : (run_raw_dwords(fmt) <= 10 ? 2 : 1);
+}
+
+__host__ __device__ constexpr int lattice_bits(int fmt) { return fmt == 2 || fmt == 9 ? 2 : (fmt == 3 || fmt == 10 ? 4 : 8); }
+
+// cb: start of the block's payload (codebook channel, then index channel); r: run 0..7 of the block
+template <int FMT>
+__device__ __forceinline__ void fetch_run(const uint8_t* __restrict__ cb, uint32_t cb_bytes, uint32_t r,
+                                          uint32_t (&raw)[run_raw_dwords(FMT)]) {
+    const uint8_t* idx = cb + cb_bytes;
+    if constexpr (FMT == 0) {
+        raw[0] = *reinterpret_cast<const uint16_t*>(cb + 2 * r);
+    } else if constexpr (FMT == 1) {
+        const uint16_t* p = reinterpret_cast<const uint16_t*>(idx + 6 * r);
+        raw[0] = p[0];
+        raw[1] = (uint32_t)p[1] | ((uint32_t)p[2] << 16);
+    } else if constexpr (FMT == 2 || FMT == 3 || FMT == 4) {
+        constexpr uint32_t bits = lattice_bits(FMT), period = 16u * bits;
+        const uint32_t b0 = 16u + bits * (32u * r - (32u * r) / period);
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(idx) + (b0 >> 5);
+        raw[0] = *reinterpret_cast<const uint16_t*>(idx);
+#pragma unroll
+        for (int j = 0; j < run_raw_dwords(FMT) - 1; ++j) raw[1 + j] = q[j];
+    } else if constexpr (FMT == 9 || FMT == 10 || FMT == 11) {
+        constexpr uint32_t bits = lattice_bits(FMT), gbytes = 4u + 8u * bits;
+        const uint8_t* g = idx + (r >> 1) * gbytes;
+        raw[0] = *reinterpret_cast<const uint32_t*>(g);
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(g + 4 + (r & 1u) * 4u * bits);
+#pragma unroll
+        for (int j = 0; j < (int)bits; ++j) raw[1 + j] = q[j];
+    } else if constexpr (FMT == 5 || FMT == 12) {
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(idx + 64 * r);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) raw[j] = q[j];
+    } else if constexpr (FMT == 6) {
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(idx + 128 * r);
+#pragma unroll
+        for (int j = 0; j < 32; ++j) raw[j] = q[j];
+    } else if constexpr (FMT == 7) {
+        const uint32_t b0 = 16u + 30u * r;                                     // 30 coded weights per run
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(idx) + (b0 >> 5);
+        raw[0] = *reinterpret_cast<const uint16_t*>(idx);
+        raw[1] = q[0];
+        raw[2] = q[1];
+    } else {
+        raw[0] = 0;
+    }
+}
+
+// OIL1 has no per-weight form: the caller multiplies the run's mean with the sum of the run's activations.
+__device__ __forceinline__ float oil1_mean(const uint32_t (&raw)[1]) { return f16_bits(raw[0]); }
+
+template <int FMT>
+__device__ __forceinline__ void expand_run(const uint32_t (&raw)[run_raw_dwords(FMT)], const uint8_t* __restrict__ cb,
+                                           uint32_t cb_bytes, uint32_t idx_bytes, uint32_t r,
+                                           const DecodeTables* __restrict__ T, const LdsTables& L, float (&w)[32]) {
+    static_assert(FMT != 0, "OIL1 runs are a mean, see oil1_mean");
+    if constexpr (FMT == 1) {
+        const uint32_t sbits = __float_as_uint(f16_bits(raw[0]));
+        const uint32_t neg = ~raw[1];                                              // bit set -> weight is -scale
+#pragma unroll
+        for (int k = 0; k < 32; ++k)    // magnitude of the scale, sign from bit k
+            w[k] = __uint_as_float((sbits & 0x7FFFFFFFu) | (((neg << (31 - k)) & 0x80000000u) ^ (sbits & 0x80000000u)));
+    } else if constexpr (FMT == 2 || FMT == 3 || FMT == 4) {
+        constexpr uint32_t bits = lattice_bits(FMT), period = 16u * bits;
+        const uint32_t b0 = 16u + bits * (32u * r - (32u * r) / period);
+        const bool last_is_slot = ((32u * (r + 1)) % period) == 0u;
+        const float scale = f16_bits(raw[0]);
+        const uint32_t sh = b0 & 31u;
+        constexpr int per = 32 / (int)bits;                                        // weights per dword
+#pragma unroll
+        for (int j = 0; j < run_raw_dwords(FMT) - 2; ++j) {
+            const uint32_t v = funnel(raw[1 + j], raw[2 + j], sh);
+#pragma unroll
+            for (int e = 0; e < per; ++e) {
+                const uint32_t q = (v >> (bits * e)) & ((1u << bits) - 1u);
+                w[per * j + e] = (bits == 2u ? L.lv2[q] : bits == 4u ? L.lv4[q] : L.lv8[q]) * scale;
+            }
+        }
+        if (last_is_slot) w[31] = 0.0f;
+    } else if constexpr (FMT == 9 || FMT == 10 || FMT == 11) {
+        constexpr uint32_t bits = lattice_bits(FMT);
+        const float zp = f16_bits(raw[0]), sc = f16_bits(raw[0] >> 16);
+        constexpr int per = 32 / (int)bits;
+        if (sc == 0.0f) {
+#pragma unroll
+            for (int k = 0; k < 32; ++k) w[k] = zp;
+        } else {
+#pragma unroll
+            for (int j = 0; j < (int)bits; ++j) {
+                const uint32_t v = raw[1 + j];
+#pragma unroll
+                for (int e = 0; e < per; ++e) {
+                    const uint32_t q = (v >> (bits * e)) & ((1u << bits) - 1u);
+                    w[per * j + e] = __fmaf_rn(bits == 2u ? L.lv2[q] : bits == 4u ? L.lv4[q] : L.t255[q], sc, zp);
+                }
+            }
+        }
+    } else if constexpr (FMT == 5 || FMT == 12) {
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            w[2 * j] = f16_bits(raw[j]);
+            w[2 * j + 1] = f16_bits(raw[j] >> 16);
+        }
+    } else if constexpr (FMT == 6) {
+#pragma unroll
+        for (int k = 0; k < 32; ++k) w[k] = __uint_as_float(raw[k]);
+    } else if constexpr (FMT == 7) {
+        const float scale = f16_bits(raw[0]);
+        const uint32_t v = funnel(raw[1], raw[2], (16u + 30u * r) & 31u);
+#pragma unroll
+        for (int k = 0; k < 32; ++k) {
+            const int code = k - (k >= 15 ? 1 : 0);                                // weights 15 and 31 of a run are slots
+            w[k] = (k == 15 || k == 31) ? 0.0f : (((v >> code) & 1u) ? scale : -scale);
+        }
+    } else {
+        for (int k = 0; k < 32; ++k)
+            w[k] = decode_weight((uint32_t)FMT, cb, cb_bytes, cb + cb_bytes, idx_bytes, 256u, 32u * r + (uint32_t)k, T);
+    }
+}
+
+}  // namespace oilhip

@@ -65,6 +65,35 @@ def test_mixed_format_rows():
     assert err <= TOL
 
 
+# rows that mix formats run on the tile- and format-ordered layout: the planner's half-and-half SPARK_Q0 / OIL1 plan,
+# the four-format stress plan, the grouped mixes and all fifteen formats at once; row counts that are not a multiple
+# of the tile, single-block rows, one to five activation rows
+@pytest.mark.parametrize("fmt_ids", [(0, 1), (0, 1, 2, 3), (7, 9, 10, 11), (6, 11, 9, 7), tuple(range(15))])
+@pytest.mark.parametrize("rows,cols,M", [(4, 256, 1), (7, 512, 2), (33, 4096, 1), (130, 2816, 3), (61, 1024, 5), (1, 1536, 4)])
+def test_mixed_format_tiles(fmt_ids, rows, cols, M):
+    rng = np.random.default_rng(rows * 7 + cols + M + len(fmt_ids))
+    fmts = rng.choice(np.array(fmt_ids, dtype=np.uint8), size=rows * cols // 256)
+    if fmts.min() == fmts.max():
+        fmts[0] = fmt_ids[0] if fmts[0] != fmt_ids[0] else fmt_ids[1]
+    err, payload, blocks, X, want = run_case(fmts, rows, cols, M=M, seed=57 + rows)
+    assert err <= TOL
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:      # the reordered payload decodes as before
+        got = dw.dequant().cpu().numpy()
+    ref = O.dequant_blocks(payload, to_orc_blocks(blocks))
+    assert np.array_equal(got.view(np.uint32).ravel(), ref.view(np.uint32).ravel())
+
+
+def test_mixed_format_skewed_tiles():
+    """Tiles in which a format is absent, or holds a single block, or fills every block."""
+    rows, cols = 24, 2048
+    fmts = np.zeros(rows * cols // 256, dtype=np.uint8)          # OIL1 everywhere ...
+    fmts[8 * 8: 12 * 8] = 1                                      # ... rows 8-11 all SPARK_Q0 (one whole tile)
+    fmts[5] = 3                                                  # a single OIL4 block in tile 0
+    fmts[-1] = 11                                                # a single OIL8_GRP block in the last row
+    err, *_ = run_case(fmts, rows, cols, M=1, seed=77)
+    assert err <= TOL
+
+
 # the fast OIL4 kernel: every slab width (cols/256 = 16 -> 8 blocks per slab, 43 -> 4,
 # 6 -> 2, 3 -> 1, 56 -> 8), ragged row counts, chunked rows, M up to 16
 @pytest.mark.parametrize("rows,cols", [(64, 4096), (1000, 4096), (37, 11008), (300, 11008),
