@@ -124,6 +124,12 @@ int oilhip_weights_destroy(oilhip_weights* w);
 int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols,
                         uint32_t* nblocks, uint64_t* payload_bytes, int* uniform_fmt);
 
+/* Device memory the tensor occupies: block bytes as stored (padding, and for a tensor that mixes formats the window
+ * headers and block tags of its streams), and the 16-byte per-block descriptors.  The difference between stored_bytes
+ * and payload_bytes is what a GEMV reads on top of the algorithmic bytes.  No counterpart in the reference, whose
+ * tensors live in host memory (include/oil/qwen35_engine.h:29).  Either out pointer may be NULL. */
+int oilhip_weights_device_bytes(const oilhip_weights* w, uint64_t* stored_bytes, uint64_t* descriptor_bytes);
+
 /* ------------------------------------------------------------- .oil container
  * OILReader (include/oil/oil_format.h:66-108, src/oil_format.cpp:289-527) and OILWriter
  * (src/oil_format.cpp:189-283).  A file handle maps the file and indexes its block records once.
@@ -214,10 +220,12 @@ int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const 
                              float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
 
 /* ------------------------------------------------------------ decode-step pieces
- * oilhip_weights_stack_rows : several uploaded tensors of one format, width and regular block layout as one
- *                             tensor of their rows in order (device copy; the parts stay valid).  Lets the gate
- *                             and up projections (or q, k, v) run as one launch.  No reference counterpart: the
- *                             reference walks each tensor separately.
+ * oilhip_weights_stack_rows : several uploaded tensors of one width (full 256-weight blocks only) as one tensor of
+ *                             their rows in order; the parts stay valid.  Parts of one format and regular layout
+ *                             are copied on the device; parts that mix formats, or differ in format, are fetched
+ *                             back and laid out afresh as one mixed tensor.  Lets the gate and up projections (or
+ *                             q, k, v) run as one launch.  No reference counterpart: the reference walks each
+ *                             tensor separately.
  * oilhip_rmsnorm_f32        : Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:39-44) over `rows` rows of
  *                             n floats: out = x * r * (1 + w), r = 1 / sqrt(mean(x^2) + 1e-6)
  * oilhip_gemv_rmsnorm_f32   : y[M][rows] = W . rmsnorm(x; normw), the rmsnorm + gemm pair in front of every projection

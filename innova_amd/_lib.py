@@ -42,6 +42,7 @@ _SIGNATURES = {
     "oilhip_weights_create": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
     "oilhip_weights_create_from_records": (C.c_int, [vp, C.c_uint64, vp, C.c_uint32, C.c_uint64, C.c_uint64, C.POINTER(vp)]),
     "oilhip_weights_destroy": (C.c_int, [vp]),
+    "oilhip_weights_device_bytes": (C.c_int, [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
     "oilhip_weights_info": (C.c_int, [vp, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint32),
                                       C.POINTER(C.c_uint64), C.POINTER(C.c_int)]),
     "oilhip_file_open": (C.c_int, [C.c_char_p, C.POINTER(vp)]),

@@ -138,6 +138,14 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
     struct Window { std::vector<Entry> ent; std::vector<uint16_t> tags; std::vector<uint32_t> src; uint32_t data = 0; };
     auto bytes_of = [](size_t ne, size_t nb, uint32_t data) { return 16 + 16 * ne + ((2 * nb + 15) & ~(size_t)15) + data; };
     std::vector<std::vector<Window>> streams(ns);
+    // The first window of every stream is fetched blind at the size of the fullest one, so its capacity is held near
+    // the average stream: what does not fit goes to a second window, fetched while the first is worked on.
+    uint64_t all_bytes = 0, widest = 0;
+    for (const DevBlock& d : db) {
+        all_bytes += g.stride[slot_of[d.fmt]] + 2u;
+        widest = std::max<uint64_t>(widest, g.stride[slot_of[d.fmt]]);
+    }
+    const uint64_t first_cap = std::min<uint64_t>(kSegWindow, std::max((all_bytes / ns * 9 / 8 + 96 + 63) & ~63ull, (widest + 64 + 63) & ~63ull));
     for (uint32_t st = 0; st < ns; ++st) {
         std::vector<Window>& ws = streams[st];
         ws.emplace_back();
@@ -154,7 +162,8 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
                         const uint32_t b = (uint32_t)(r * bpr + c);
                         if (slot_of[db[b].fmt] != (int)s) continue;
                         Window* w = &ws.back();
-                        if (bytes_of(w->ent.size() + (open ? 0 : 1), w->tags.size() + 1, w->data + g.stride[s]) > kSegWindow) {
+                        if (bytes_of(w->ent.size() + (open ? 0 : 1), w->tags.size() + 1, w->data + g.stride[s]) >
+                            (ws.size() == 1 ? first_cap : kSegWindow)) {
                             ws.emplace_back();
                             w = &ws.back();
                             open = false;
@@ -173,18 +182,33 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
             last->flags |= 1u;                         // every tile has blocks: its last entry closes it
         }
     }
-    size_t maxw = 1;
-    for (const auto& ws : streams) maxw = std::max(maxw, ws.size());
-    const uint64_t stride = (uint64_t)maxw * kSegWindow, total = stride * ns;
+    // first windows at a fixed stride (the fullest of them decides it), so that a wavefront finds its own from its
+    // number alone; the windows after them packed one behind the other, each found through its predecessor's header
+    auto used = [&](const Window& w) { return bytes_of(w.ent.size(), w.tags.size(), w.data); };
+    size_t first_used = 0;
+    for (const auto& ws : streams) first_used = std::max(first_used, used(ws[0]));
+    const uint64_t stride = (first_used + 63) & ~(size_t)63;
+    uint64_t total = stride * ns;
+    std::vector<std::vector<uint64_t>> at_of(ns);
+    for (uint32_t st = 0; st < ns; ++st) {
+        at_of[st].push_back(st * stride);
+        for (size_t wi = 1; wi < streams[st].size(); ++wi) {
+            at_of[st].push_back(total);
+            total += (used(streams[st][wi]) + 63) & ~(size_t)63;
+        }
+    }
     if ((total >> 4) > 0xFFFFFFFFull) return;
     std::vector<uint8_t> out(total, 0);
     for (uint32_t st = 0; st < ns; ++st)
         for (size_t wi = 0; wi < streams[st].size(); ++wi) {
             const Window& w = streams[st][wi];
-            uint8_t* base = out.data() + st * stride + wi * kSegWindow;
+            uint8_t* base = out.data() + at_of[st][wi];
             const uint32_t tag_base = 16u + 16u * (uint32_t)w.ent.size();
             const uint32_t data_base = tag_base + (uint32_t)((2 * w.tags.size() + 15) & ~(size_t)15);
-            const uint32_t hdr[4] = {(uint32_t)w.ent.size(), (uint32_t)streams[st].size(), 0u, 0u};
+            const bool more = wi + 1 < streams[st].size();
+            const uint32_t hdr[4] = {(uint32_t)w.ent.size(), more ? 1u : 0u,
+                                     more ? (uint32_t)((used(streams[st][wi + 1]) + 15) >> 4) : 0u,
+                                     more ? (uint32_t)(at_of[st][wi + 1] >> 4) : 0u};
             std::memcpy(base, hdr, 16);
             for (size_t i = 0; i < w.ent.size(); ++i) {
                 const Entry& e = w.ent[i];
@@ -197,13 +221,14 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
             for (uint32_t b : w.src) {
                 DevBlock& d = db[b];
                 std::memcpy(base + at, pay.data() + (size_t)d.off16 * 16, (size_t)d.cb_bytes + d.idx_bytes);
-                d.off16 = (uint32_t)((st * stride + wi * kSegWindow + at) >> 4);
+                d.off16 = (uint32_t)((at_of[st][wi] + at) >> 4);
                 at += g.stride[slot_of[d.fmt]];
             }
         }
     pay.swap(out);
     g.nf = nf;
     g.nstreams = ns;
+    g.blind16 = (uint32_t)((first_used + 15) >> 4);
     g.stream_bytes = stride;
 }
 
@@ -333,12 +358,40 @@ int oilhip_weights_stack_rows(const oilhip_weights* const* parts, int n, oilhip_
     *out = nullptr;
     const oilhip_weights* p0 = parts[0];
     uint64_t rows = 0, nblocks = 0, bytes = 0, algo = 0;
+    bool regular = true;
     for (int i = 0; i < n; ++i) {
         const oilhip_weights* p = parts[i];
-        if (!p || !p->uniform_stride || p->uniform_fmt != p0->uniform_fmt || p->uniform_stride != p0->uniform_stride ||
-            p->cols != p0->cols || !p->all_full || p->uniform_cb != p0->uniform_cb || p->uniform_idx != p0->uniform_idx)
-            return fail(OILHIP_E_ARG, "stack_rows: parts must share one format, width and regular block layout");
+        if (!p || !p0 || p->cols != p0->cols || !p->all_full)
+            return fail(OILHIP_E_ARG, "stack_rows: parts must share one width and hold full 256-weight blocks only");
+        regular &= p->uniform_stride && p->uniform_fmt == p0->uniform_fmt && p->uniform_stride == p0->uniform_stride &&
+                   p->uniform_cb == p0->uniform_cb && p->uniform_idx == p0->uniform_idx;
         rows += p->rows; nblocks += p->nblocks; bytes += (uint64_t)p->nblocks * p->uniform_stride; algo += p->payload_bytes;
+    }
+    if (!regular) {
+        // parts that mix formats (or differ in format): fetch their blocks back and upload the concatenation, which
+        // lays the rows out afresh (window streams for a mix)
+        if (nblocks > 0xFFFFFFFFull) return fail(OILHIP_E_ARG, "stack_rows: too large");
+        std::vector<uint8_t> pay;
+        std::vector<DevBlock> db;
+        std::vector<uint64_t> off;
+        db.reserve((size_t)nblocks);
+        for (int i = 0; i < n; ++i) {
+            const oilhip_weights* p = parts[i];
+            std::vector<uint8_t> hp((size_t)p->alloc_bytes);
+            std::vector<DevBlock> hb(p->nblocks);
+            OILHIP_HIP(hipMemcpy(hp.data(), p->d_payload, hp.size(), hipMemcpyDeviceToHost));
+            OILHIP_HIP(hipMemcpy(hb.data(), p->d_blocks, sizeof(DevBlock) * hb.size(), hipMemcpyDeviceToHost));
+            for (DevBlock d : hb) {
+                const size_t nb = (size_t)d.cb_bytes + d.idx_bytes, at = pay.size();
+                if ((at >> 4) > 0xFFFFFFFFull) return fail(OILHIP_E_ARG, "stack_rows: too large");
+                pay.resize((at + nb + 15) & ~(size_t)15, 0);
+                std::memcpy(pay.data() + at, hp.data() + (size_t)d.off16 * 16, nb);
+                d.off16 = (uint32_t)(at >> 4);
+                off.push_back((uint64_t)db.size() * 256u);
+                db.push_back(d);
+            }
+        }
+        return upload(pay, db, off, algo, rows, p0->cols, out);
     }
     if (nblocks > 0xFFFFFFFFull || bytes / 16 > 0xFFFFFFFFull) return fail(OILHIP_E_ARG, "stack_rows: too large");
     auto* w = new (std::nothrow) oilhip_weights();
@@ -381,6 +434,13 @@ int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols,
     if (nblocks) *nblocks = w->nblocks;
     if (payload_bytes) *payload_bytes = w->payload_bytes;
     if (uniform_fmt) *uniform_fmt = w->uniform_fmt;
+    return OILHIP_OK;
+}
+
+int oilhip_weights_device_bytes(const oilhip_weights* w, uint64_t* stored_bytes, uint64_t* descriptor_bytes) {
+    if (!w) return fail(OILHIP_E_ARG, "null weights");
+    if (stored_bytes) *stored_bytes = w->alloc_bytes;
+    if (descriptor_bytes) *descriptor_bytes = (uint64_t)w->nblocks * sizeof(DevBlock);
     return OILHIP_OK;
 }
 

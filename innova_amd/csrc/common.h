@@ -25,18 +25,20 @@ int fail(int code, const std::string& msg);
 int get_tables(const DecodeTables** out);
 int device_cu_count();
 
-// Tensors whose rows mix formats are stored as `nstreams` streams of 4 KB windows, stream s at byte s * stream_bytes
-// of the payload buffer, one wavefront per stream (gemv_seg.hip).  A stream covers a contiguous range of rows in tiles
+// Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream
+// (gemv_seg.hip).  The first window of stream s sits at byte s * stream_bytes of the payload buffer, the later ones
+// behind all first windows, each found through its predecessor.  A stream covers a contiguous range of rows in tiles
 // of at most kSegTileRows; inside a tile the blocks are ordered by format (in the order of `fmt`), inside a format by
-// row and column.  Window: 4 dwords {entries, windows of the stream, 0, 0}; per entry 4 dwords
-// {slot | format << 4 | closes its tile << 8 | blocks << 16, byte offset of the blocks | byte offset of their tags << 16,
-// first row of the tile, rows of the tile}; the tags (per block: row of the tile << 12 | column block); the blocks,
-// 16-byte aligned, whole.
+// row and column.  Window: 4 dwords {entries, 1 if another window follows, 16-byte pieces that window fills, its byte
+// offset / 16 in the buffer}; per entry 4 dwords {slot | format << 4 | closes its tile << 8 | blocks << 16, byte offset
+// of the blocks | byte offset of their tags << 16, first row of the tile, rows of the tile}; the tags (per block: row
+// of the tile << 12 | column block); the blocks, 16-byte aligned, whole.  `blind16` = 16-byte pieces the fullest first
+// window fills.
 constexpr int kSegMaxFormats = 15;
 constexpr uint32_t kSegWindow = 4096;
 constexpr int kSegTileRows = 4;
 struct SegLayout {
-    uint32_t nf = 0, nstreams = 0;
+    uint32_t nf = 0, nstreams = 0, blind16 = 0;
     uint64_t stream_bytes = 0;
     uint32_t fmt[kSegMaxFormats] = {}, cb_bytes[kSegMaxFormats] = {}, idx_bytes[kSegMaxFormats] = {}, stride[kSegMaxFormats] = {};
 };

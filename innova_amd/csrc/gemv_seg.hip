@@ -4,9 +4,9 @@
 // (src/adapters/tools/qwen35_engine.cpp:47-85) fused with dequantize_block_all (src/block_codec.cpp:576-720).
 //
 // Such a tensor is a few MB of small blocks (16 bytes for OIL1, 48 for SPARK_Q0), so the launch is bound by
-// dependent memory round trips, not by bandwidth.  The upload therefore stores it as one stream of 4 KB windows per
-// wavefront, at an address that follows from the wavefront's number alone: the first window is fetched blind together
-// with the activations, and a window describes itself (entries: format, block count, where the blocks and their tags
+// dependent memory round trips, not by bandwidth.  The upload therefore stores it as one stream of windows (at most
+// 4 KB each) per wavefront, the first at an address that follows from the wavefront's number alone: it is fetched
+// blind together with the activations, and a window describes itself and says where the next one is (entries: format, block count, where the blocks and their tags
 // sit in the window, which rows they belong to).  A stream covers a contiguous range of rows in tiles of up to four;
 // inside a tile the blocks are ordered by format, inside a format by row and column, so a step of 8 blocks has one
 // format for all 64 lanes.  The wavefront copies a window to LDS with plain 16-byte loads, fetches the next one while it works,
@@ -31,7 +31,7 @@ typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct SegArgs {
-    uint32_t nstreams;
+    uint32_t nstreams, blind16;
     uint64_t stream_bytes;
     uint32_t cb_bytes[kSegMaxFormats], idx_bytes[kSegMaxFormats], stride[kSegMaxFormats];
 };
@@ -58,32 +58,30 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
     constexpr int N = run_raw_dwords(FMT);
     const uint32_t steps = (nblk + 7u) >> 3, r = lane & 7u, g = lane >> 3;
     if constexpr (FMT == 0) {
-        // no arithmetic to hide the LDS round trips behind: several steps side by side
-        constexpr int U = MB >= 4 ? 2 : 4;
-        for (uint32_t st0 = 0; st0 < steps; st0 += U) {
-            uint32_t tag[U], raw[U][1];
-            bool live[U];
+        // a block is 8 FP16 run means: a lane takes a whole block, 16 bytes of means against 8 run sums
+        for (uint32_t b0 = 0; b0 < nblk; b0 += 64u) {
+            const uint32_t blk = b0 + lane;
+            const bool live = blk < nblk;
+            const uint32_t bc = live ? blk : nblk - 1u;
+            const uint32_t tag = tags[bc];
+            const u32x4 mv = *reinterpret_cast<const u32x4*>(data + bc * stride);
+            const float mean[8] = {f16_bits(mv.x), f16_bits(mv.x >> 16), f16_bits(mv.y), f16_bits(mv.y >> 16),
+                                   f16_bits(mv.z), f16_bits(mv.z >> 16), f16_bits(mv.w), f16_bits(mv.w >> 16)};
+            float part[MB];
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const uint32_t blk = (st0 + u) * 8u + g;
-                live[u] = blk < nblk;
-                const uint32_t bc = live[u] ? blk : nblk - 1u;
-                tag[u] = tags[bc];
-                fetch_run<0>(data + bc * stride, cb_bytes, r, raw[u]);
+            for (int m = 0; m < MB; ++m) {
+                const float4* sp = reinterpret_cast<const float4*>(rs + (size_t)m * nruns + (tag & 0xFFFu) * 8u);
+                const float4 s0 = sp[0], s1 = sp[1];
+                float a0 = mean[0] * s0.x, a1 = mean[1] * s0.y;
+                a0 = __fmaf_rn(mean[2], s0.z, a0);
+                a1 = __fmaf_rn(mean[3], s0.w, a1);
+                a0 = __fmaf_rn(mean[4], s1.x, a0);
+                a1 = __fmaf_rn(mean[5], s1.y, a1);
+                a0 = __fmaf_rn(mean[6], s1.z, a0);
+                a1 = __fmaf_rn(mean[7], s1.w, a1);
+                part[m] = live ? a0 + a1 : 0.f;
             }
-            float sum[U][MB];
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-#pragma unroll
-                for (int m = 0; m < MB; ++m) sum[u][m] = rs[(size_t)m * nruns + (tag[u] & 0xFFFu) * 8u + r];
-#pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const float mean = live[u] ? oil1_mean(raw[u]) : 0.f;
-                float part[MB];
-#pragma unroll
-                for (int m = 0; m < MB; ++m) part[m] = mean * sum[u][m];
-                add_to_row<MB>(acc, tag[u] >> 12, part);
-            }
+            add_to_row<MB>(acc, tag >> 12, part);
         }
     } else {
     for (uint32_t st = 0; st < steps; ++st) {
@@ -177,8 +175,11 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     const bool active = sid < A.nstreams;
     const uint8_t* sp = streams + (active ? (size_t)sid * A.stream_bytes : 0);
     u32x4 wreg[4];                                     // a window in flight: 4 x 16 bytes per lane
+    // the first window is fetched before anything is known about it: as many 16-byte pieces as the fullest first
+    // window of the tensor has
 #pragma unroll
-    for (int j = 0; j < 4; ++j) wreg[j] = *reinterpret_cast<const u32x4*>(sp + ((size_t)j * 64u + lane) * 16u);
+    for (int j = 0; j < 4; ++j)
+        wreg[j] = j * 64u + lane < A.blind16 ? *reinterpret_cast<const u32x4*>(sp + ((size_t)j * 64u + lane) * 16u) : u32x4{0, 0, 0, 0};
 
     for (uint32_t i = tid; i < 532u; i += 64u * kWaves)
         tb[i] = i < 256u ? T->lv8[i] : i < 512u ? T->t255[i - 256u] : i < 528u ? kLv4[i - 512u] : kLv2[i - 528u];
@@ -220,16 +221,18 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     for (int m = 0; m < MB; ++m)
 #pragma unroll
         for (int j = 0; j < TR; ++j) acc[m][j] = 0.f;
-    const uint32_t nwin = uniform(reinterpret_cast<const uint32_t*>(win)[1]);
-    for (uint32_t wi = 0; wi < nwin; ++wi) {
+    for (uint32_t wi = 0;; ++wi) {
         const uint8_t* cur = win + (wi & 1u) * kSegWindow;
-        const bool more = wi + 1u < nwin;
-        if (more) {
+        const uint32_t* hdr = reinterpret_cast<const uint32_t*>(cur);
+        const bool more = uniform(hdr[1]) != 0u;
+        if (more) {                                    // the next window: its size and place are in this one's header
+            const uint32_t used16 = uniform(hdr[2]);
+            const uint8_t* np = streams + (size_t)uniform(hdr[3]) * 16u;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                wreg[j] = *reinterpret_cast<const u32x4*>(sp + (size_t)(wi + 1u) * kSegWindow + ((size_t)j * 64u + lane) * 16u);
+                if (j * 64u + lane < used16) wreg[j] = *reinterpret_cast<const u32x4*>(np + ((size_t)j * 64u + lane) * 16u);
         }
-        const uint32_t ne = uniform(reinterpret_cast<const uint32_t*>(cur)[0]);
+        const uint32_t ne = uniform(hdr[0]);
         for (uint32_t i = 0; i < ne; ++i) {
             const uint32_t* rec = reinterpret_cast<const uint32_t*>(cur) + 4u + 4u * i;
             const uint32_t r0 = uniform(rec[0]), r1 = uniform(rec[1]), row0 = uniform(rec[2]), nrows = uniform(rec[3]);
@@ -265,6 +268,8 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 #pragma unroll
             for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(nxt + ((size_t)j * 64u + lane) * 16u) = wreg[j];
             __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");       // other lanes read what this lane wrote
+        } else {
+            break;
         }
     }
 }
@@ -286,7 +291,7 @@ int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x,
         attr_done = true;
     }
     SegArgs A{};
-    A.nstreams = g.nstreams; A.stream_bytes = g.stream_bytes;
+    A.nstreams = g.nstreams; A.blind16 = g.blind16; A.stream_bytes = g.stream_bytes;
     for (uint32_t i = 0; i < g.nf; ++i) { A.cb_bytes[i] = g.cb_bytes[i]; A.idx_bytes[i] = g.idx_bytes[i]; A.stride[i] = g.stride[i]; }
     hipLaunchKernelGGL(kern, dim3((g.nstreams + kWaves - 1) / kWaves), dim3(64 * kWaves), lds, s, w.d_payload, T, d_x, d_y,
                        (uint32_t)w.rows, (uint32_t)w.cols, m0, M, A);

@@ -5,13 +5,17 @@
 // dequant_grouped_lattice (:308-331), OIL1 (:615-626), OIL1_GRP (:627-642), SPARK_Q0 (:643-654), OIL16 / OIL32
 // (:585-596).  SPARK_Q0_GRP and the sparse formats go through decode_weight, weight by weight.
 #pragma once
+#include <hip/hip_fp16.h>
+
 #include "block_decode.h"
 
 namespace oilhip {
 
 struct LdsTables { const float* lv2; const float* lv4; const float* lv8; const float* t255; };   // copies in LDS
 
-__device__ __forceinline__ float f16_bits(uint32_t h) { return half_bits_to_float(h & 0xFFFFu); }
+// FP16 bits -> FP32 through the hardware conversion: the same value as f16_to_f32 (src/block_codec.cpp:61-84) for
+// every finite input and infinity (NaN payloads, which the bit-exact dequantization keeps, do not matter in a dot product)
+__device__ __forceinline__ float f16_bits(uint32_t h) { return __half2float(__ushort_as_half((unsigned short)(h & 0xFFFFu))); }
 
 // 32-bit window starting `sh` bits into the dword pair (lo, hi)
 __device__ __forceinline__ uint32_t funnel(uint32_t lo, uint32_t hi, uint32_t sh) {

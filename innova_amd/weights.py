@@ -83,8 +83,10 @@ class DeviceWeights:
         nb, uf = C.c_uint32(0), C.c_int(0)
         _lib.check(_lib.lib().oilhip_weights_info(self.handle, C.byref(rows), C.byref(cols), C.byref(nb),
                                                   C.byref(pb), C.byref(uf)))
+        stored, desc = C.c_uint64(0), C.c_uint64(0)
+        _lib.check(_lib.lib().oilhip_weights_device_bytes(self.handle, C.byref(stored), C.byref(desc)))
         return {"rows": rows.value, "cols": cols.value, "nblocks": nb.value, "payload_bytes": pb.value,
-                "uniform_fmt": uf.value}
+                "uniform_fmt": uf.value, "stored_bytes": stored.value, "descriptor_bytes": desc.value}
 
     # ---- compute ----------------------------------------------------------------
     def dequant(self, out=None):

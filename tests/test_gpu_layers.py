@@ -112,7 +112,28 @@ def test_embed_rows():
 def test_stack_rows_rejects_mismatched_parts():
     a = ia.DeviceWeights.quantize(gaussian_weights(4 * 512, 1), ia.Format.OIL4, 4, 512)
     b = ia.DeviceWeights.quantize(gaussian_weights(4 * 256, 2), ia.Format.OIL4, 4, 256)
-    c = ia.DeviceWeights.quantize(gaussian_weights(4 * 512, 3), ia.Format.OIL8, 4, 512)
-    for bad in ([a, b], [a, c]):
-        with pytest.raises(ia.OilHipError):
-            ia.DeviceWeights.stack_rows(bad)
+    with pytest.raises(ia.OilHipError):
+        ia.DeviceWeights.stack_rows([a, b])
+
+
+def test_stack_rows_of_mixed_and_different_formats():
+    """Parts that mix formats, or differ in format, stack into one mixed tensor: GEMV and dequantization of the
+    stack equal those of the parts one after the other."""
+    rng = np.random.default_rng(12)
+    cols, parts, ys, dq = 1024, [], [], []
+    X = rng.standard_normal((2, cols)).astype(np.float32)
+    for i, (rows, fm) in enumerate([(9, (0, 1)), (5, (3,)), (14, (0, 1, 10))]):
+        w = gaussian_weights(rows * cols, 40 + i)
+        fmts = rng.choice(np.array(fm, dtype=np.uint8), size=rows * cols // 256)
+        payload, blocks = ia.block_codec.quantize_tensor(w, fmts)
+        parts.append(ia.DeviceWeights.from_blocks(payload, blocks, rows, cols))
+        ys.append(O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True))
+        dq.append(O.dequant_blocks(payload, to_orc_blocks(blocks)))
+    with ia.DeviceWeights.stack_rows(parts) as st:
+        assert st.info()["rows"] == 28 and st.info()["uniform_fmt"] == -1
+        got = st.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
+        deq = st.dequant().cpu().numpy()
+    assert rel_l2(got, np.concatenate(ys, axis=1)) <= 1e-5
+    assert np.array_equal(deq.view(np.uint32), np.concatenate(dq).view(np.uint32))
+    for p in parts:
+        p.close()
