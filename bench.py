@@ -277,11 +277,12 @@ STACK = [("q", 4096, 4096), ("k", 4096, 4096), ("v", 4096, 4096), ("o", 4096, 40
 def bench_mixed_stack(torch, ia):
     """The 1.50-bpw stack: 7 matrices of a Llama-7B layer, 1 % of blocks scaled x8, importance = mean |w|
     per block, formats from the planner at target 1.50 (half SPARK_Q0, half OIL1), and a stress plan that is
-    NOT reference-derived (importance quartiles -> OIL4 / OIL2 / SPARK_Q0 / OIL1)."""
+    NOT reference-derived (importance quartiles -> OIL4 / OIL2 / SPARK_Q0 / OIL1); and the registry's grouped mix
+    SPARK_MIX_Q0 (1.925 bpw: OIL8_GRP / OIL4_GRP / OIL2_GRP / OIL1_GRP per block by FormatRegistry::allocate_mix_blocks)."""
     import numpy as np
-    from innova_amd.format_planner import FormatPlanner
+    from innova_amd.format_planner import FormatPlanner, allocate_mix_blocks
     rng = np.random.default_rng(33)
-    plans = {"planner_1p50": [], "stress_quartiles": []}
+    plans = {"planner_1p50": [], "stress_quartiles": [], "spark_mix_q0": []}
     for name, rows, cols in STACK:
         w = make_weights(rows, cols, seed=100 + len(name) + rows % 97)
         nb = rows * cols // 256
@@ -293,7 +294,8 @@ def bench_mixed_stack(torch, ia):
         sc = pl.importance_scores()
         q = np.argsort(np.argsort(-sc, kind="stable"), kind="stable") * 4 // nb          # quartile by descending importance
         stress = np.array([int(ia.Format.OIL4), int(ia.Format.OIL2), int(ia.Format.SPARK_Q0), int(ia.Format.OIL1)], np.uint8)[q]
-        for key, fm in (("planner_1p50", plan.formats), ("stress_quartiles", stress)):
+        mix = allocate_mix_blocks("SPARK_MIX_Q0", w, 256, (rows, cols))[0]
+        for key, fm in (("planner_1p50", plan.formats), ("stress_quartiles", stress), ("spark_mix_q0", mix)):
             payload, blocks = ia.block_codec.quantize_tensor(w, fm)
             plans[key].append((rows, cols, payload, blocks))
         del w

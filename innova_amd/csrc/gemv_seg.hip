@@ -127,6 +127,23 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
                 }
                 part[m] = a0 + a1;
             }
+        } else if constexpr (has_dot_run(FMT)) {
+            constexpr int MH = MB > 2 ? 2 : MB;          // activation rows per pass: 32 registers of x each
+#pragma unroll
+            for (int h = 0; h < MB; h += MH) {
+                f32x4_t xv[MH][8];
+                float xsum[MH], sub[MH];
+#pragma unroll
+                for (int m = 0; m < MH; ++m) {
+                    const float* xr = xs + (size_t)(h + m) * xpad + run * kRunPad;
+#pragma unroll
+                    for (int c = 0; c < 8; ++c) xv[m][c] = *reinterpret_cast<const f32x4_t*>(xr + 4 * c);
+                    xsum[m] = rs[(size_t)(h + m) * nruns + run];
+                }
+                dot_run<FMT, MH>(raw, r, xv, xsum, sub);
+#pragma unroll
+                for (int m = 0; m < MH; ++m) part[h + m] = sub[m];
+            }
         } else {
             float w[32];
             expand_run<FMT>(raw, cb, cb_bytes, idx_bytes, r, T, L, w);
@@ -156,20 +173,19 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
 
 #define OILHIP_SEG_FORMATS(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14)
 
-// MB activation rows per launch.  Dynamic LDS: MB * (padded x + run sums), level tables, two windows per wavefront.
+// MB activation rows per launch.  Dynamic LDS: byte tables, MB * (padded x + run sums), two windows per wavefront.
 template <int MB>
 __global__ void __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restrict__ T, const float* __restrict__ x,
                 float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M, const SegArgs A) {
     extern __shared__ __align__(16) float smem[];
     const uint32_t nruns = cols >> 5, xpad = nruns * kRunPad;
-    float* xs = smem;                                  // [MB][nruns][36]
-    float* rs = smem + (size_t)MB * xpad;              // [MB][nruns] run sums
-    float* tb = rs + (size_t)MB * nruns;               // level tables: lv8[256] t255[256] lv4[16] lv2[4]
+    float* xs = smem + kByteTabBytes / 4;              // [MB][nruns][36], behind the byte tables of dot_run
+    float* rs = xs + (size_t)MB * xpad;                // [MB][nruns] run sums
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = uniform(tid >> 6);
-    uint8_t* win = reinterpret_cast<uint8_t*>(tb + 532) + (size_t)wave * 2u * kSegWindow;
-    const LdsTables L{tb + 528, tb + 512, tb, tb + 256};
+    uint8_t* win = reinterpret_cast<uint8_t*>(rs + (size_t)MB * nruns) + (size_t)wave * 2u * kSegWindow;
+    const LdsTables L{nullptr, nullptr, nullptr, nullptr};      // the formats that expand weight by weight here use no level table
 
     const uint32_t sid = blockIdx.x * kWaves + wave;
     const bool active = sid < A.nstreams;
@@ -181,8 +197,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     for (int j = 0; j < 4; ++j)
         wreg[j] = j * 64u + lane < A.blind16 ? *reinterpret_cast<const u32x4*>(sp + ((size_t)j * 64u + lane) * 16u) : u32x4{0, 0, 0, 0};
 
-    for (uint32_t i = tid; i < 532u; i += 64u * kWaves)
-        tb[i] = i < 256u ? T->lv8[i] : i < 512u ? T->t255[i - 256u] : i < 528u ? kLv4[i - 512u] : kLv2[i - 528u];
+    build_byte_tables(smem, tid, 64u * kWaves);
     // x -> LDS, 36 floats per run; 8 consecutive threads hold one run and add it up on the way
     const uint32_t nq = cols >> 2;
 #pragma unroll
@@ -276,7 +291,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 
 template <int MB>
 size_t seg_lds_bytes(const oilhip_weights& w) {
-    return ((size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) + 532) * 4 + (size_t)kWaves * 2 * kSegWindow;
+    return kByteTabBytes + (size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) * 4 + (size_t)kWaves * 2 * kSegWindow;
 }
 
 template <int MB>
