@@ -1,7 +1,6 @@
-// gemv_runs.hip -- decode GEMV for every wire format and for rows that mix formats (the 1.50-bpw
-// stacks FormatPlanner::allocate produces, src/format_planner.cpp:133-315): Qwen35Engine::gemm
-// (src/adapters/tools/qwen35_engine.cpp:47-85) fused with dequantize_block_all
-// (src/block_codec.cpp:576-720).
+// gemv_runs.hip -- decode GEMV for uniform tensors of every wire format that has no kernel of its own (all but OIL4
+// and OIL8), and the fallback for mixed tensors the window-stream kernel does not take: Qwen35Engine::gemm
+// (src/adapters/tools/qwen35_engine.cpp:47-85) fused with dequantize_block_all (src/block_codec.cpp:576-720).
 //
 // A lane owns one run of 32 consecutive weights: 8 lanes cover a 256-weight block and a
 // wavefront-step covers 8 consecutive blocks of a row.  Each lane fetches only the bytes of its
@@ -9,8 +8,9 @@
 // short routine into 32 registers and multiplies them with its 32 activations, which sit in LDS
 // with 4 floats of padding per run so that the 16-byte reads of neighbouring lanes fall into
 // different banks.  OIL1 needs no per-weight work at all: its run contributes mean * sum(x over
-// the run), and the run sums are computed once per launch.  Lanes of a step whose blocks differ
-// in format diverge by 8-lane group only.  Formats without a short routine go through the
+// the run), and the run sums are computed once per launch.  Block addresses follow from the constant
+// stride of a uniform tensor, or from the 16-byte descriptors otherwise (lanes of a step whose blocks
+// differ in format then diverge by 8-lane group).  Formats without a short routine go through the
 // general per-weight decoder.
 #include "common.h"
 #include "run_decode.h"

@@ -173,14 +173,14 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
 
 #define OILHIP_SEG_FORMATS(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14)
 
-// MB activation rows per launch.  Dynamic LDS: byte tables, MB * (padded x + run sums), two windows per wavefront.
+// MB activation rows per launch.  Dynamic LDS: level tables, MB * (padded x + run sums), two windows per wavefront.
 template <int MB>
 __global__ void __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restrict__ T, const float* __restrict__ x,
                 float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M, const SegArgs A) {
     extern __shared__ __align__(16) float smem[];
     const uint32_t nruns = cols >> 5, xpad = nruns * kRunPad;
-    float* xs = smem + kByteTabBytes / 4;              // [MB][nruns][36], behind the byte tables of dot_run
+    float* xs = smem + kLevelTabBytes / 4;              // [MB][nruns][36], behind the level tables of dot_run
     float* rs = xs + (size_t)MB * xpad;                // [MB][nruns] run sums
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = uniform(tid >> 6);
@@ -197,7 +197,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     for (int j = 0; j < 4; ++j)
         wreg[j] = j * 64u + lane < A.blind16 ? *reinterpret_cast<const u32x4*>(sp + ((size_t)j * 64u + lane) * 16u) : u32x4{0, 0, 0, 0};
 
-    build_byte_tables(smem, tid, 64u * kWaves);
+    build_level_tables(smem, tid);
     // x -> LDS, 36 floats per run; 8 consecutive threads hold one run and add it up on the way
     const uint32_t nq = cols >> 2;
 #pragma unroll
@@ -291,7 +291,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 
 template <int MB>
 size_t seg_lds_bytes(const oilhip_weights& w) {
-    return kByteTabBytes + (size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) * 4 + (size_t)kWaves * 2 * kSegWindow;
+    return kLevelTabBytes + (size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) * 4 + (size_t)kWaves * 2 * kSegWindow;
 }
 
 template <int MB>

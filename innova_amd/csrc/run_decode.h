@@ -162,13 +162,13 @@ __device__ __forceinline__ void expand_run(const uint32_t (&raw)[run_raw_dwords(
 // expand_run / decode_weight.  The two tables sit at the start of the kernel's LDS.
 constexpr uint32_t kLv4Off = 0;            // 16 floats
 constexpr uint32_t kLv2Off = 64;           // 4 floats
-constexpr uint32_t kByteTabBytes = 128;
+constexpr uint32_t kLevelTabBytes = 128;
 
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) const float lds_cf;
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ void build_byte_tables(float* lds0, uint32_t tid, uint32_t) {
+__device__ __forceinline__ void build_level_tables(float* lds0, uint32_t tid) {
     if (tid < 16u) lds0[kLv4Off / 4 + tid] = kLv4[tid];
     if (tid < 4u) lds0[kLv2Off / 4 + tid] = kLv2[tid];
 }

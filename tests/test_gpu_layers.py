@@ -130,7 +130,11 @@ def test_stack_rows_of_mixed_and_different_formats():
         ys.append(O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True))
         dq.append(O.dequant_blocks(payload, to_orc_blocks(blocks)))
     with ia.DeviceWeights.stack_rows(parts) as st:
-        assert st.info()["rows"] == 28 and st.info()["uniform_fmt"] == -1
+        info = st.info()
+        assert info["rows"] == 28 and info["uniform_fmt"] == -1
+        # stored as window streams: block bytes plus tags and window headers, never less than the payload
+        assert info["payload_bytes"] <= info["stored_bytes"] <= 2 * info["payload_bytes"] + 4096
+        assert info["descriptor_bytes"] == 16 * info["nblocks"]
         got = st.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
         deq = st.dequant().cpu().numpy()
     assert rel_l2(got, np.concatenate(ys, axis=1)) <= 1e-5
