@@ -53,13 +53,15 @@ constexpr int kRedBytes = 8 * kGroups * 64 * 16;
 // i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const int* __restrict__ tok, uint32_t* __restrict__ xp, uint32_t cols, int m0, int M,
-              uint32_t ldx, uint32_t xrows) {
+              uint32_t ldx, uint32_t xrows, int half) {
     const uint32_t id = blockIdx.x * 256u + threadIdx.x;            // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
     const uint32_t bpr = cols >> 8;
     if (id >= bpr * 2048u) return;
     const uint32_t c = id & 15u, lane = (id >> 4) & 63u, h = (id >> 10) & 1u, blk = id >> 11;
     const uint32_t t = lane & 15u, kq = lane >> 4;
-    const int m = m0 + (int)t;
+    // passes of 8 tokens: columns 0..7 carry the high parts of tokens 0..7, columns 8..15 their low parts, in the
+    // pieces that otherwise hold the high parts of 16 tokens; the low-part pieces are not used
+    const int m = m0 + (int)(half ? (t & 7u) : t);
     const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
     float v[2] = {0.0f, 0.0f};
     if (src < xrows) {
@@ -76,10 +78,18 @@ pack_x_kernel(const float* __restrict__ x, const int* __restrict__ tok, uint32_t
     const auto ph = __builtin_amdgcn_cvt_pkrtz(v[0], v[1]);           // x = xh + xl, both FP16 (round toward zero)
     const auto pl = __builtin_amdgcn_cvt_pkrtz(v[0] - (float)ph[0], v[1] - (float)ph[1]);
     uint32_t* o = xp + ((size_t)(id >> 10) * 8u * 64u + lane) * 4u + (c & 3u);     // piece 0 of this lane, element c & 3
-    o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
-    o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+    if (half) {
+        o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, t < 8u ? ph : pl);
+    } else {
+        o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
+        o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+    }
 }
 
+// HALF: passes of 8 tokens.  The activation operand then holds high parts (columns 0..7) and low parts (columns 8..15)
+// at once, so L x = (Lh + Ll)(xh + xl) takes two matrix instructions per 32 columns instead of three, the activations
+// are half as many bytes, and an output is the sum of accumulator columns j and j + 8.
+template <bool HALF>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, float* __restrict__ y,
                        uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem) {
@@ -103,7 +113,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 
     // activations of this wavefront's two blocks, token li, chunks kq and kq+4: FP16 pairs (positions 2c, 2c+1),
     // high parts and low parts
-    uint32_t bh[2][2][16], bl[2][2][16];
+    uint32_t bh[2][2][16], bl[HALF ? 1 : 2][HALF ? 1 : 2][HALF ? 1 : 16];
     v4f acc[kGroups];
     const uint32_t lanebase = (lane & 31u) * 8u;
 
@@ -120,6 +130,27 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         }
     };
 
+    // split activations of this wavefront's two blocks of K-pass `pass` -> registers: 8 (4 for passes of 8 tokens)
+    // loads of 16 bytes per block half
+    auto load_b = [&](uint32_t pass) {
+#pragma unroll
+        for (int b2 = 0; b2 < 2; ++b2) {
+            const uint32_t blk = pass * 16u + wave * 2u + b2;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t off = blk < bpr ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const u32x4 vh = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 1024u * j, 0, 0);
+                    bh[b2][h][4 * j] = vh.x; bh[b2][h][4 * j + 1] = vh.y; bh[b2][h][4 * j + 2] = vh.z; bh[b2][h][4 * j + 3] = vh.w;
+                    if constexpr (!HALF) {
+                        const u32x4 vl = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 4096u + 1024u * j, 0, 0);
+                        bl[b2][h][4 * j] = vl.x; bl[b2][h][4 * j + 1] = vl.y; bl[b2][h][4 * j + 2] = vl.z; bl[b2][h][4 * j + 3] = vl.w;
+                    }
+                }
+            }
+        }
+    };
     issue_group(0, g0, 0);                 // weights of the first group fly during the set-up
     {   // pair table from literals: entry of byte v = (b << 4 | a), lane copy c at byte v*256 + c*8 =
         // { Lh[a] | Lh[b] << 16, Ll[a] | Ll[b] << 16 }; thread tid writes float4 number tid + 512*k (two copies of
@@ -141,24 +172,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         for (int g = 0; g < kGroups; ++g) acc[g] = v4f{0.f, 0.f, 0.f, 0.f};
         for (uint32_t pass = 0; pass < npass; ++pass) {
             if (tile > 0 || pass > 0) issue_group(0, tg0, pass);
-            if (npass > 1 || tile == 0) {
-                // ---- split activations of this wavefront's two blocks -> registers: 8 loads of 16 bytes per block half
-#pragma unroll
-                for (int b2 = 0; b2 < 2; ++b2) {
-                    const uint32_t blk = pass * 16u + wave * 2u + b2;
-#pragma unroll
-                    for (int h = 0; h < 2; ++h) {
-                        const uint32_t off = blk < bpr ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const u32x4 vh = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 1024u * j, 0, 0);
-                            const u32x4 vl = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 4096u + 1024u * j, 0, 0);
-                            bh[b2][h][4 * j] = vh.x; bh[b2][h][4 * j + 1] = vh.y; bh[b2][h][4 * j + 2] = vh.z; bh[b2][h][4 * j + 3] = vh.w;
-                            bl[b2][h][4 * j] = vl.x; bl[b2][h][4 * j + 1] = vl.y; bl[b2][h][4 * j + 2] = vl.z; bl[b2][h][4 * j + 3] = vl.w;
-                        }
-                    }
-                }
-            }
+            if (npass > 1 || tile == 0) load_b(pass);
             if (!table_synced) { __syncthreads(); table_synced = true; }   // the level table is complete
             // ---- main loop: groups of the tile, two blocks each -------------------------------------------
 #pragma unroll
@@ -191,9 +205,11 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                             const h8 Ah = __builtin_bit_cast(h8, u32x4{ah[4 * d], ah[4 * d + 1], ah[4 * d + 2], ah[4 * d + 3]});
                             const h8 Al = __builtin_bit_cast(h8, u32x4{al[4 * d], al[4 * d + 1], al[4 * d + 2], al[4 * d + 3]});
                             const h8 Bh = __builtin_bit_cast(h8, u32x4{bh[b2][h][4 * d], bh[b2][h][4 * d + 1], bh[b2][h][4 * d + 2], bh[b2][h][4 * d + 3]});
-                            const h8 Bl = __builtin_bit_cast(h8, u32x4{bl[b2][h][4 * d], bl[b2][h][4 * d + 1], bl[b2][h][4 * d + 2], bl[b2][h][4 * d + 3]});
                             t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bh, t0, 0, 0, 0);
-                            t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bl, t1, 0, 0, 0);
+                            if constexpr (!HALF) {
+                                const h8 Bl = __builtin_bit_cast(h8, u32x4{bl[b2][h][4 * d], bl[b2][h][4 * d + 1], bl[b2][h][4 * d + 2], bl[b2][h][4 * d + 3]});
+                                t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bl, t1, 0, 0, 0);
+                            }
                             t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, Bh, t1, 0, 0, 0);
                         }
                         __builtin_amdgcn_sched_barrier(0);
@@ -220,11 +236,13 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
             const uint32_t rl = o & 63u, j = o >> 6;                       // row of the tile, token of the pass
             const uint32_t g = rl >> 4, i = rl & 15u;
             const uint32_t r = (tg0 + g) * 16u + i;
-            if (tg0 + g < g1 && r < rows && m0 + (int)j < M) {
+            if (tg0 + g < g1 && r < rows && m0 + (int)j < M && (!HALF || j < 8u)) {
                 float s = 0.f;
 #pragma unroll
-                for (uint32_t w8 = 0; w8 < 8; ++w8)
+                for (uint32_t w8 = 0; w8 < 8; ++w8) {
                     s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j) * 4 + (i & 3u)];
+                    if (HALF) s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j + 8u) * 4 + (i & 3u)];
+                }
                 y[(size_t)(m0 + j) * ldy + r] = s;
             }
         }
@@ -258,7 +276,9 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
     static bool attr_done = false;
     if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel),
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
@@ -269,14 +289,20 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     uint32_t grid = (uint32_t)device_cu_count();
     if (grid > groups) grid = groups;
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
-    for (int m0 = 0; m0 < M; m0 += 16) {          // passes of at most 16 tokens
-        const int m1 = M - m0 < 16 ? M : m0 + 16;
+    for (int m0 = 0; m0 < M;) {                   // passes of 16 tokens; the last 8 or fewer as a pass of 8
+        const bool half = M - m0 <= 8;
+        const int m1 = half || M - m0 < 16 ? M : m0 + 16;
         hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_tok, xp, (uint32_t)w.cols, m0, m1,
-                           ldx, xrows);
+                           ldx, xrows, half ? 1 : 0);
         OILHIP_HIP(hipGetLastError());
-        hipLaunchKernelGGL(gemv_oil4_multi_kernel, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
-                           (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
+        if (half)
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
+                               (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
+        else
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
+                               (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
         OILHIP_HIP(hipGetLastError());
+        m0 = m1;
     }
     return OILHIP_OK;
 }
