@@ -110,7 +110,7 @@ def test_oil4_fast_kernel_shapes(rows, cols, M):
     assert rel_l2(ref32, want) <= TOL
 
 
-# the multi-token kernel: every pass width (1..4 token groups), a ragged last pass, several
+# the multi-token kernel: passes of 16 tokens and of 8 or fewer (alone and as the last pass of a batch), several
 # row tiles per workgroup (rows > 48 * 256), several K-slabs, an odd number of blocks per row
 @pytest.mark.parametrize("rows,cols", [(130, 4096), (61, 11008), (13000, 512), (47, 14336), (3, 256)])
 @pytest.mark.parametrize("M", [3, 5, 8, 9, 13, 17, 40])
