@@ -193,9 +193,12 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     u32x4 wreg[4];                                     // a window in flight: 4 x 16 bytes per lane
     // the first window is fetched before anything is known about it: as many 16-byte pieces as the fullest first
     // window of the tensor has
+    // (pieces past that size repeat the last one: every lane loads, unconditionally, so that nothing waits here)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-        wreg[j] = j * 64u + lane < A.blind16 ? *reinterpret_cast<const u32x4*>(sp + ((size_t)j * 64u + lane) * 16u) : u32x4{0, 0, 0, 0};
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t piece = j * 64u + lane < A.blind16 ? j * 64u + lane : A.blind16 - 1u;
+        wreg[j] = *reinterpret_cast<const u32x4*>(sp + (size_t)piece * 16u);
+    }
 
     build_level_tables(smem, tid);
     // x -> LDS, 36 floats per run; 8 consecutive threads hold one run and add it up on the way
@@ -244,8 +247,10 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
             const uint32_t used16 = uniform(hdr[2]);
             const uint8_t* np = streams + (size_t)uniform(hdr[3]) * 16u;
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (j * 64u + lane < used16) wreg[j] = *reinterpret_cast<const u32x4*>(np + ((size_t)j * 64u + lane) * 16u);
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t piece = j * 64u + lane < used16 ? j * 64u + lane : used16 - 1u;
+                wreg[j] = *reinterpret_cast<const u32x4*>(np + (size_t)piece * 16u);
+            }
         }
         const uint32_t ne = uniform(hdr[0]);
         for (uint32_t i = 0; i < ne; ++i) {
