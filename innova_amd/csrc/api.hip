@@ -253,7 +253,11 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
     };
     hipError_t e;
     if ((e = hipGetDevice(&w->device)) != hipSuccess) return bail(e, "hipGetDevice");
-    if (all_full && !uniform) pack_window_streams(pay, db, rows, cols, w->seg);
+    // window streams for every tensor of full blocks but the uniform OIL4 and OIL8 ones, which have kernels of their own
+    // that read the blocks back to back
+    const bool own_kernel = uniform && regular && nblocks && (db[0].fmt == OILHIP_OIL4 || db[0].fmt == OILHIP_OIL8);
+    if (all_full && nblocks && !own_kernel) pack_window_streams(pay, db, rows, cols, w->seg);
+    if (w->seg.nstreams) regular = false;
     // 64 spare bytes so vector loads that straddle the end of the last block stay in bounds
     w->alloc_bytes = pay.size() + 64;
     if ((e = hipMalloc(&w->d_payload, w->alloc_bytes)) != hipSuccess) return bail(e, "hipMalloc(payload)");

@@ -26,14 +26,15 @@ dequant_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__
     }
 }
 
-// Full OIL2 / OIL4 / OIL8 blocks laid out back to back (one format, regular stride): a wavefront per block, lane l decodes
+// Full OIL2 / OIL4 / OIL8 blocks of one format, laid out back to back at a regular stride (`blocks` null) or wherever
+// their descriptors say (tensors stored as window streams): a wavefront per block, lane l decodes
 // weights 4l .. 4l+3 from two dwords and stores one float4, so a block is one coalesced 1 KB store.  Values are
 // formed exactly as decode_weight forms them: level (literal table / host-built table) times the FP16 scale widened
 // by the integer rule; slot weights are 0.
 template <int BITS>
 __global__ void __launch_bounds__(256)
-dequant_lattice_kernel(const uint8_t* __restrict__ base, uint32_t stride, const DecodeTables* __restrict__ T,
-                       float* __restrict__ out, uint32_t nblocks) {
+dequant_lattice_kernel(const uint8_t* __restrict__ base, uint32_t stride, const DevBlock* __restrict__ blocks,
+                       const DecodeTables* __restrict__ T, float* __restrict__ out, uint32_t nblocks) {
     __shared__ float lv[256];
     if (BITS == 8) lv[threadIdx.x] = T->lv8[threadIdx.x];
     else if (BITS == 4 && threadIdx.x < 16) lv[threadIdx.x] = kLv4[threadIdx.x];
@@ -41,7 +42,7 @@ dequant_lattice_kernel(const uint8_t* __restrict__ base, uint32_t stride, const 
     __syncthreads();
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     for (uint32_t b = blockIdx.x * 4u + wave; b < nblocks; b += gridDim.x * 4u) {
-        const uint32_t* q = reinterpret_cast<const uint32_t*>(base + (size_t)b * stride);
+        const uint32_t* q = reinterpret_cast<const uint32_t*>(base + (blocks ? (size_t)blocks[b].off16 * 16u : (size_t)b * stride));
         const float scale = half_bits_to_float(q[0] & 0xFFFFu);
         // first code bit of weight 4l: 16 + BITS * (4l - slots before it); one slot per 16*BITS weights
         const uint32_t i0 = 4u * lane;
@@ -65,14 +66,15 @@ dequant_lattice_kernel(const uint8_t* __restrict__ base, uint32_t stride, const 
 }
 
 // Full OIL1 (FMT 0: eight FP16 run means, 16 bytes) and SPARK_Q0 (FMT 1: per run of 32 an FP16 scale and 32 sign
-// bits, 48 bytes) blocks laid out back to back; lane l stores weights 4l .. 4l+3 of its wavefront's block.
+// bits, 48 bytes) blocks, back to back or by descriptor as above; lane l stores weights 4l .. 4l+3 of its wavefront's block.
 template <int FMT>
 __global__ void __launch_bounds__(256)
-dequant_runs_kernel(const uint8_t* __restrict__ base, uint32_t stride, float* __restrict__ out, uint32_t nblocks) {
+dequant_runs_kernel(const uint8_t* __restrict__ base, uint32_t stride, const DevBlock* __restrict__ blocks,
+                    float* __restrict__ out, uint32_t nblocks) {
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
     const uint32_t run = lane >> 3, j0 = 4u * (lane & 7u);
     for (uint32_t b = blockIdx.x * 4u + wave; b < nblocks; b += gridDim.x * 4u) {
-        const uint16_t* h = reinterpret_cast<const uint16_t*>(base + (size_t)b * stride);
+        const uint16_t* h = reinterpret_cast<const uint16_t*>(base + (blocks ? (size_t)blocks[b].off16 * 16u : (size_t)b * stride));
         float4 o;
         if (FMT == 0) {
             const float m = half_bits_to_float(h[run]);
@@ -160,22 +162,27 @@ int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s) {
     const DecodeTables* T = nullptr;
     if (int rc = get_tables(&T)) return rc;
     if (w.nblocks == 0) return OILHIP_OK;
-    if (w.all_full && w.uniform_stride > 0 && !w.d_out_off && (w.uniform_base & 3u) == 0 && (w.uniform_stride & 3u) == 0) {
+    // one format, full blocks: regular stride, or (window streams) the place of every block from its descriptor
+    const bool by_stride = w.uniform_stride > 0 && (w.uniform_base & 3u) == 0 && (w.uniform_stride & 3u) == 0;
+    const bool by_desc = w.seg.nstreams > 0 && w.seg.nf == 1;
+    if (w.all_full && w.uniform_fmt >= 0 && !w.d_out_off && (by_stride || by_desc)) {
         const uint32_t g = std::min<uint32_t>((w.nblocks + 3u) / 4u, (uint32_t)device_cu_count() * 16u);
-        const uint8_t* base = w.d_payload + w.uniform_base;
+        const uint8_t* base = w.d_payload + (by_stride ? w.uniform_base : 0u);
+        const DevBlock* bl = by_stride ? nullptr : w.d_blocks;
         const int f = w.uniform_fmt;
-        const uint32_t st = w.uniform_stride;
+        const uint32_t st = by_stride ? w.uniform_stride : w.seg.stride[0];
+        const uint32_t cb = by_stride ? w.uniform_cb : w.seg.cb_bytes[0];
         bool done = true;
-        if (f == OILHIP_OIL4 && st == 128 && w.uniform_cb == 0)
-            hipLaunchKernelGGL(dequant_lattice_kernel<4>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
-        else if (f == OILHIP_OIL8 && st == 256 && w.uniform_cb == 0)
-            hipLaunchKernelGGL(dequant_lattice_kernel<8>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
-        else if (f == OILHIP_OIL2 && st == 64 && w.uniform_cb == 0)
-            hipLaunchKernelGGL(dequant_lattice_kernel<2>, dim3(g), dim3(256), 0, s, base, st, T, d_out, w.nblocks);
-        else if (f == OILHIP_OIL1 && st == 16 && w.uniform_cb == 16)
-            hipLaunchKernelGGL(dequant_runs_kernel<0>, dim3(g), dim3(256), 0, s, base, st, d_out, w.nblocks);
-        else if (f == OILHIP_SPARK_Q0 && st == 48 && w.uniform_cb == 0)
-            hipLaunchKernelGGL(dequant_runs_kernel<1>, dim3(g), dim3(256), 0, s, base, st, d_out, w.nblocks);
+        if (f == OILHIP_OIL4 && st == 128 && cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<4>, dim3(g), dim3(256), 0, s, base, st, bl, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL8 && st == 256 && cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<8>, dim3(g), dim3(256), 0, s, base, st, bl, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL2 && st == 64 && cb == 0)
+            hipLaunchKernelGGL(dequant_lattice_kernel<2>, dim3(g), dim3(256), 0, s, base, st, bl, T, d_out, w.nblocks);
+        else if (f == OILHIP_OIL1 && st == 16 && cb == 16)
+            hipLaunchKernelGGL(dequant_runs_kernel<0>, dim3(g), dim3(256), 0, s, base, st, bl, d_out, w.nblocks);
+        else if (f == OILHIP_SPARK_Q0 && st == 48 && cb == 0)
+            hipLaunchKernelGGL(dequant_runs_kernel<1>, dim3(g), dim3(256), 0, s, base, st, bl, d_out, w.nblocks);
         else
             done = false;
         if (done) {

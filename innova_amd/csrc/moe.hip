@@ -92,7 +92,7 @@ int expert_gemv(const oilhip_weights& w, const float* d_x, const int* d_tok, flo
         OILHIP_HIP(hipGetLastError());
         xin = d_gather;
     }
-    return launch_gemv_generic(w, xin, d_y, nt, s);
+    return oilhip_gemv_f32(&w, xin, d_y, nt, s);      // every other format and mixed rows: the decode GEMV's own routing
 }
 
 }  // namespace
