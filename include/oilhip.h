@@ -124,8 +124,8 @@ int oilhip_weights_destroy(oilhip_weights* w);
 int oilhip_weights_info(const oilhip_weights* w, uint64_t* rows, uint64_t* cols,
                         uint32_t* nblocks, uint64_t* payload_bytes, int* uniform_fmt);
 
-/* Device memory the tensor occupies: block bytes as stored (padding, and for a tensor that mixes formats the window
- * headers and block tags of its streams), and the 16-byte per-block descriptors.  The difference between stored_bytes
+/* Device memory the tensor occupies: block bytes as stored (padding, and for every tensor of full blocks except uniform
+ * OIL4 / OIL8 the window headers and block tags of its streams), and the 16-byte per-block descriptors.  The difference between stored_bytes
  * and payload_bytes is what a GEMV reads on top of the algorithmic bytes.  No counterpart in the reference, whose
  * tensors live in host memory (include/oil/qwen35_engine.h:29).  Either out pointer may be NULL. */
 int oilhip_weights_device_bytes(const oilhip_weights* w, uint64_t* stored_bytes, uint64_t* descriptor_bytes);
