@@ -476,8 +476,8 @@ def main():
                     help="only run plain 1 GiB device copies (reference for the FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build measures one GPU only (the path shards by output rows with no "
-                 "reduction; see DESIGN.md); run with --gpus 1")
+        sys.exit("bench.py: this build measures one GPU only (the path would shard by output rows, with no "
+                 "reduction between GPUs); run with --gpus 1")
 
     import numpy as np
     import torch
