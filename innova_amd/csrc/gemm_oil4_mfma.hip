@@ -19,6 +19,7 @@
 // block's FP16 scale in FP32 and rounded once to bf16.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <cstdlib>
 #include <mutex>
 
@@ -189,6 +190,11 @@ gemm_oil4_bf16_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict_
         }
 }
 
+// Y <- 0 in front of a launch whose workgroups add partial sums (a fill kernel, so that a caller may capture it in a graph)
+__global__ void __launch_bounds__(256) zero_y_kernel(float* __restrict__ y, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (size_t)gridDim.x * 256u) y[i] = 0.f;
+}
+
 // Pipelined kernel for larger M: 256 tokens x 128 weight rows per workgroup, 8 wavefronts (4 x 2, each
 // 64 x 64 outputs), 64 columns per step, two LDS tile buffers: while the matrix cores work on step kt, the
 // same wavefronts decode the weights of step kt+1 into the other buffer and the global loads of the
@@ -205,7 +211,7 @@ constexpr int PBM = 256, PBN = 128;
 
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
-                           uint32_t M, uint32_t N, uint32_t K) {
+                           uint32_t M, uint32_t N, uint32_t K, uint32_t ksplit) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);
     __bf16* As = reinterpret_cast<__bf16*>(lds + kTabBytes);                      // [2][PBM][PLD]
@@ -318,18 +324,21 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     // unconditionally (steps past the end are clamped to the last one and decoded into a buffer nobody reads):
     // the number of loads in flight is then a compile-time fact and each wait covers exactly the step it needs.
     static_assert(D == 2 || D == 4, "D must be even and divide 4");
-    const uint32_t last = KT - 1u;
+    // ksplit > 1: workgroup blockIdx.z takes the steps [kbeg, kend) of the row and adds its partial sums to a zeroed Y
+    // (two parts at most, so the sum does not depend on which arrives first)
+    const uint32_t kbeg = KT / ksplit * blockIdx.z, kend = blockIdx.z + 1u == ksplit ? KT : kbeg + KT / ksplit;
+    const uint32_t last = kend - 1u;
     auto clampk = [&](uint32_t k) { return k < last ? k : last; };
 #pragma unroll
-    for (int u = 0; u < D; ++u) load_regs(u, clampk((uint32_t)u));
+    for (int u = 0; u < D; ++u) load_regs(u, clampk(kbeg + (uint32_t)u));
     __syncthreads();                                   // table complete
     store_tiles(0, 0);
-    load_regs(0, clampk((uint32_t)D));
+    load_regs(0, clampk(kbeg + (uint32_t)D));
     __syncthreads();
     // register set s holds the steps congruent to s modulo D.  Iteration kt issues the table reads of step kt+1,
     // then the fragment reads of step kt (buffer kt & 1), multiplies, finishes the decode of step kt+1 into the
     // other buffer in the shadow of the MFMAs and refills that register set with step kt+1+D.
-    for (uint32_t kt0 = 0; kt0 < KT; kt0 += D) {
+    for (uint32_t kt0 = kbeg; kt0 < kend; kt0 += D) {
 #pragma unroll
         for (int u = 0; u < D; ++u) {
             const uint32_t kt = kt0 + u;
@@ -350,7 +359,10 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t row = m0 + (wm * 2 + i) * 32u + 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u);
-                if (row < M && col < N) Y[(size_t)row * N + col] = acc[i][j][v];
+                if (row < M && col < N) {
+                    if (ksplit > 1u) unsafeAtomicAdd(Y + (size_t)row * N + col, acc[i][j][v]);
+                    else Y[(size_t)row * N + col] = acc[i][j][v];
+                }
             }
         }
 }
@@ -420,8 +432,15 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
         }
         const uint32_t N = (uint32_t)w.rows;
         const size_t lds_bytes = (size_t)kTabBytes + 2ull * (PBM + PBN) * PLD * 2;
-        hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel, dim3((N + PBN - 1) / PBN, Mpad / PBM), dim3(512), lds_bytes, s,
-                           w.d_payload, xp, d_y, (uint32_t)M, N, K);
+        // a grid that leaves half of the compute units idle is cut in two along K (two partial sums into a zeroed Y)
+        const uint32_t tiles = (N + PBN - 1) / PBN * (Mpad / PBM);
+        const uint32_t ksplit = tiles * 2u <= (uint32_t)device_cu_count() && (K / PK) % 8u == 0u ? 2u : 1u;
+        if (ksplit > 1u) {
+            hipLaunchKernelGGL(zero_y_kernel, dim3((uint32_t)std::min<size_t>(((size_t)M * N + 255) / 256, 4096)), dim3(256), 0, s, d_y, (size_t)M * N);
+            OILHIP_HIP(hipGetLastError());
+        }
+        hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel, dim3((N + PBN - 1) / PBN, Mpad / PBM, ksplit), dim3(512), lds_bytes, s,
+                           w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
         OILHIP_HIP(hipGetLastError());
         return OILHIP_OK;
     }
