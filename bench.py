@@ -337,6 +337,42 @@ def bench_mixed_stack(torch, ia):
         out[f"stack_{key}_stacked_us_per_layer"] = round(ts * 1e6, 1)
         out[f"stack_{key}_stacked_GBps"] = round(payload_bytes / ts / 1e9, 1)
         out[f"stack_{key}_stacked_tok_per_s_32_layers"] = round(1.0 / (32 * ts), 1)
+        # ... and as the decode step runs it: both RMSNorms and the SwiGLU product inside the launches that consume them
+        L = _lib_handles(ia)
+        wn = torch.randn(4096, device="cuda") * 0.1
+        scratch = torch.empty(3 * 11008 + 4096, device="cuda")
+        cur = lambda: ia._lib.current_stream()  # noqa: E731
+
+        def layer(c):
+            qkv, gu = skeep[2 * c], skeep[2 * c + 1]
+            o, down = keep[7 * c + 3], keep[7 * c + 6]
+            ia._lib.check(L.oilhip_gemv_rmsnorm_f32(qkv.handle, xs[4096].data_ptr(), wn.data_ptr(), ysk[(4096, 12288)].data_ptr(),
+                                                    1, None, cur()))
+            o.gemv(xs[4096], out=ys[4096])                               # attention itself is not modelled
+            ia._lib.check(L.oilhip_mlp_step_f32(gu.handle, down.handle, ys[4096].data_ptr(), wn.data_ptr(),
+                                                ysk[(4096, 12288)].data_ptr(), 1, scratch.data_ptr(), cur()))
+
+        for c in range(copies):
+            layer(c)
+        torch.cuda.synchronize()
+        fstream, fgraph = torch.cuda.Stream(), torch.cuda.CUDAGraph()
+        with torch.cuda.stream(fstream):
+            with torch.cuda.graph(fgraph, stream=fstream):
+                for c in range(copies):
+                    layer(c)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(fstream):
+            fgraph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(fstream)
+            for _ in range(5):
+                fgraph.replay()
+            e1.record(fstream)
+            torch.cuda.synchronize()
+        tf = e0.elapsed_time(e1) * 1e-3 / (5 * copies)
+        out[f"stack_{key}_fused_layer_us"] = round(tf * 1e6, 1)
+        out[f"stack_{key}_fused_layer_tok_per_s_32_layers"] = round(1.0 / (32 * tf), 1)
         for d in keep + skeep:
             d.close()
     return out

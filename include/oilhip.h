@@ -229,14 +229,15 @@ int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const 
  * oilhip_rmsnorm_f32        : Qwen35Engine::rmsnorm (src/adapters/tools/qwen35_engine.cpp:39-44) over `rows` rows of
  *                             n floats: out = x * r * (1 + w), r = 1 / sqrt(mean(x^2) + 1e-6)
  * oilhip_gemv_rmsnorm_f32   : y[M][rows] = W . rmsnorm(x; normw), the rmsnorm + gemm pair in front of every projection
- *                             (:484-486 attention input, :611-614 MLP input).  With M = 1 and an OIL4 tensor the
- *                             norm is formed while the GEMV stages x (one launch, d_xn unused and may be NULL);
+ *                             (:484-486 attention input, :611-614 MLP input).  With M = 1 and an OIL4 or window-stream
+ *                             tensor the norm is formed while the GEMV stages x (one launch, d_xn unused and may be NULL);
  *                             otherwise d_xn[M][cols] receives the normalised rows and the GEMV reads them.
  * oilhip_mlp_step_f32       : Qwen35Engine::mlp_step (:611-621): y[M][D] = down(siluf(gate x) * up x), gate_up = the
  *                             gate and up projections stacked (2F x D, gate rows first), down = D x F.  A non-NULL
  *                             d_normw applies rmsnorm(x; d_normw) first, as the caller of mlp_step does.
- *                             d_scratch holds M * (3*F + D) floats.  With M = 1 and OIL4 tensors the norm rides on
- *                             the first GEMV and the SwiGLU product on the second: two launches for the whole step.
+ *                             d_scratch holds M * (3*F + D) floats.  With M = 1 and OIL4 or window-stream tensors the
+ *                             norm rides on the first GEMV and the SwiGLU product on the second: two launches for the
+ *                             whole step.
  * oilhip_embed_rows_f32     : the embedding lookup of Qwen35Engine::append_token (:756-760, decode_block :17-28):
  *                             rows d_ids[i] of a quantized [vocab][cols] tensor decoded to d_out[i][cols]; ids outside
  *                             the table give zero rows */

@@ -174,13 +174,20 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
 #define OILHIP_SEG_FORMATS(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14)
 
 // MB activation rows per launch.  Dynamic LDS: level tables, MB * (padded x + run sums), two windows per wavefront.
-template <int MB>
+// XF (one activation row only) transforms x while it is staged: 1 = the row holds 2 * cols floats h and the kernel
+// multiplies with siluf(h[k]) * h[cols + k] (the SwiGLU product of Qwen35Engine::mlp_step,
+// src/adapters/tools/qwen35_engine.cpp:611-621); 2 = x * (1 + xw[k]) is staged and every output is scaled by
+// 1 / sqrt(mean(x^2) + 1e-6), which each workgroup forms from the row it loads anyway (Qwen35Engine::rmsnorm, :39-44).
+template <int MB, int XF>
 __global__ void __launch_bounds__(64 * kWaves) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restrict__ T, const float* __restrict__ x,
-                float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M, const SegArgs A) {
+                const float* __restrict__ xw, float* __restrict__ y, uint32_t rows, uint32_t cols, int m0, int M,
+                const SegArgs A) {
+    static_assert(XF == 0 || MB == 1, "the fused input transforms serve one activation row");
     extern __shared__ __align__(16) float smem[];
     const uint32_t nruns = cols >> 5, xpad = nruns * kRunPad;
-    float* xs = smem + kLevelTabBytes / 4;              // [MB][nruns][36], behind the level tables of dot_run
+    float* ssq_part = smem + kLevelTabBytes / 4;       // XF = 2: sum(x^2) per wavefront
+    float* xs = ssq_part + 16;                         // [MB][nruns][36], behind the level tables of dot_run
     float* rs = xs + (size_t)MB * xpad;                // [MB][nruns] run sums
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = uniform(tid >> 6);
@@ -203,22 +210,35 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     build_level_tables(smem, tid);
     // x -> LDS, 36 floats per run; 8 consecutive threads hold one run and add it up on the way
     const uint32_t nq = cols >> 2;
+    float ssq = 0.f;
 #pragma unroll
     for (int m = 0; m < MB; ++m) {
         const bool on = m0 + m < M;
-        const float4* xrow = reinterpret_cast<const float4*>(x + (size_t)(on ? m0 + m : 0) * cols);
+        const float4* xrow = reinterpret_cast<const float4*>(x + (size_t)(on ? m0 + m : 0) * cols * (XF == 1 ? 2u : 1u));
         for (uint32_t c0 = tid; c0 < nq; c0 += 256u * kWaves) {
-            float4 v[4];
+            float4 v[4], b[XF ? 4 : 1];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t c4 = c0 + 64u * kWaves * j;
                 v[j] = xrow[c4 < nq ? c4 : c0];
+                if constexpr (XF == 1) b[j] = xrow[nq + (c4 < nq ? c4 : c0)];
+                if constexpr (XF == 2) b[j] = reinterpret_cast<const float4*>(xw)[c4 < nq ? c4 : c0];
             }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t c4 = c0 + 64u * kWaves * j;
                 if (c4 < nq) {
-                    const float4 t = on ? v[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    float4 t = on ? v[j] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    if constexpr (XF == 1) {
+                        t.x = (t.x * __builtin_amdgcn_rcpf(1.0f + __expf(-t.x))) * b[j].x;
+                        t.y = (t.y * __builtin_amdgcn_rcpf(1.0f + __expf(-t.y))) * b[j].y;
+                        t.z = (t.z * __builtin_amdgcn_rcpf(1.0f + __expf(-t.z))) * b[j].z;
+                        t.w = (t.w * __builtin_amdgcn_rcpf(1.0f + __expf(-t.w))) * b[j].w;
+                    }
+                    if constexpr (XF == 2) {
+                        ssq = __fmaf_rn(t.x, t.x, __fmaf_rn(t.y, t.y, __fmaf_rn(t.z, t.z, __fmaf_rn(t.w, t.w, ssq))));
+                        t.x *= 1.0f + b[j].x; t.y *= 1.0f + b[j].y; t.z *= 1.0f + b[j].z; t.w *= 1.0f + b[j].w;
+                    }
                     *reinterpret_cast<float4*>(xs + (size_t)m * xpad + (c4 >> 3) * kRunPad + (c4 & 7u) * 4) = t;
                     float s = (t.x + t.y) + (t.z + t.w);
                     s += oil4::dpp_quad_xor1(s);
@@ -229,10 +249,25 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
             }
         }
     }
+    if constexpr (XF == 2) {
+        float v = ssq;
+        v += oil4::dpp_quad_xor1(v);
+        v += oil4::dpp_quad_xor2(v);
+        v += oil4::dpp_half_mirror(v);
+        v += oil4::dpp_row_mirror(v);
+        v += oil4::dpp_row_bcast15(v);
+        v += oil4::dpp_row_bcast31(v);
+        if (lane == 63) ssq_part[wave] = v;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4*>(win + ((size_t)j * 64u + lane) * 16u) = wreg[j];
     __syncthreads();
     if (!active) return;
+    float yscale = 1.0f;
+    if constexpr (XF == 2) {
+        const float tot = ((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) + ((ssq_part[4] + ssq_part[5]) + (ssq_part[6] + ssq_part[7]));
+        yscale = 1.0f / sqrtf(tot / (float)cols + 1e-6f);
+    }
 
     float acc[MB][TR];
 #pragma unroll
@@ -279,7 +314,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
                         v += oil4::dpp_row_mirror(v);
                         v += oil4::dpp_row_bcast15(v);
                         v += oil4::dpp_row_bcast31(v);
-                        if (lane == 63 && (uint32_t)j < nrows && m0 + m < M) y[(size_t)(m0 + m) * rows + row0 + j] = v;
+                        if (lane == 63 && (uint32_t)j < nrows && m0 + m < M) y[(size_t)(m0 + m) * rows + row0 + j] = v * yscale;
                     }
             }
         }
@@ -296,13 +331,14 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 
 template <int MB>
 size_t seg_lds_bytes(const oilhip_weights& w) {
-    return kLevelTabBytes + (size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) * 4 + (size_t)kWaves * 2 * kSegWindow;
+    return kLevelTabBytes + 64 + (size_t)MB * ((w.cols >> 5) * (kRunPad + 1)) * 4 + (size_t)kWaves * 2 * kSegWindow;
 }
 
-template <int MB>
-int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x, float* d_y, int m0, int M, hipStream_t s) {
+template <int MB, int XF = 0>
+int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x, float* d_y, int m0, int M, hipStream_t s,
+               const float* d_xw = nullptr) {
     static bool attr_done = false;
-    auto kern = gemv_seg_kernel<MB>;
+    auto kern = gemv_seg_kernel<MB, XF>;
     const SegLayout& g = w.seg;
     const size_t lds = seg_lds_bytes<MB>(w);
     if (lds > 160 * 1024) return 1;
@@ -313,8 +349,8 @@ int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x,
     SegArgs A{};
     A.nstreams = g.nstreams; A.blind16 = g.blind16; A.stream_bytes = g.stream_bytes;
     for (uint32_t i = 0; i < g.nf; ++i) { A.cb_bytes[i] = g.cb_bytes[i]; A.idx_bytes[i] = g.idx_bytes[i]; A.stride[i] = g.stride[i]; }
-    hipLaunchKernelGGL(kern, dim3((g.nstreams + kWaves - 1) / kWaves), dim3(64 * kWaves), lds, s, w.d_payload, T, d_x, d_y,
-                       (uint32_t)w.rows, (uint32_t)w.cols, m0, M, A);
+    hipLaunchKernelGGL(kern, dim3((g.nstreams + kWaves - 1) / kWaves), dim3(64 * kWaves), lds, s, w.d_payload, T, d_x, d_xw,
+                       d_y, (uint32_t)w.rows, (uint32_t)w.cols, m0, M, A);
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }
@@ -337,6 +373,22 @@ int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M
         if (rc) return rc;
     }
     return OILHIP_OK;
+}
+
+// y = W . (siluf(h[0..K)) * h[K..2K)) for one activation row h of 2K floats.  Returns 1 when the tensor is not covered.
+int launch_gemv_seg_swiglu(const oilhip_weights& w, const float* d_h, float* d_y, hipStream_t s) {
+    if (!w.seg.nstreams || !w.all_full || (w.cols & 255u) || w.rows == 0 || seg_lds_bytes<1>(w) > 160 * 1024) return 1;
+    const DecodeTables* T = nullptr;
+    if (int rc = get_tables(&T)) return rc;
+    return launch_seg<1, 1>(w, T, d_h, d_y, 0, 1, s);
+}
+
+// y = W . rmsnorm(x; xw) for one activation row.  Returns 1 when the tensor is not covered.
+int launch_gemv_seg_rmsnorm(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, hipStream_t s) {
+    if (!w.seg.nstreams || !w.all_full || (w.cols & 255u) || w.rows == 0 || seg_lds_bytes<1>(w) > 160 * 1024) return 1;
+    const DecodeTables* T = nullptr;
+    if (int rc = get_tables(&T)) return rc;
+    return launch_seg<1, 2>(w, T, d_x, d_y, 0, 1, s, d_xw);
 }
 
 }  // namespace oilhip

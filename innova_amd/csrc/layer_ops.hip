@@ -8,6 +8,8 @@
 namespace oilhip {
 int launch_gemv_oil4_swiglu(const oilhip_weights& w, const float* d_h, float* d_y, hipStream_t s);
 int launch_gemv_oil4_rmsnorm(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, hipStream_t s);
+int launch_gemv_seg_swiglu(const oilhip_weights& w, const float* d_h, float* d_y, hipStream_t s);
+int launch_gemv_seg_rmsnorm(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, hipStream_t s);
 
 namespace {
 
@@ -102,6 +104,10 @@ int oilhip_gemv_rmsnorm_f32(const oilhip_weights* w, const float* d_x, const flo
         const int rc = launch_gemv_oil4_rmsnorm(*w, d_x, d_normw, d_y, (hipStream_t)stream);   // the norm rides on the staging of x
         if (rc <= 0) return rc;
     }
+    if (M == 1 && w->seg.nstreams) {
+        const int rc = launch_gemv_seg_rmsnorm(*w, d_x, d_normw, d_y, (hipStream_t)stream);    // likewise for window-stream tensors
+        if (rc <= 0) return rc;
+    }
     if (!d_xn) return fail(OILHIP_E_ARG, "gemv_rmsnorm: this shape needs the d_xn workspace");
     if (int rc = oilhip_rmsnorm_f32(d_x, d_normw, (int)w->cols, M, d_xn, stream)) return rc;
     return oilhip_gemv_f32(w, d_xn, d_y, M, stream);
@@ -121,6 +127,10 @@ int oilhip_mlp_step_f32(const oilhip_weights* gate_up, const oilhip_weights* dow
                          : oilhip_gemv_f32(gate_up, d_x, h2, M, stream)) return rc;
     if (M == 1 && down->uniform_fmt == OILHIP_OIL4 && down->uniform_stride == 128) {
         const int rc = launch_gemv_oil4_swiglu(*down, h2, d_y, s);      // SwiGLU formed while the activations are staged
+        if (rc <= 0) return rc;
+    }
+    if (M == 1 && down->seg.nstreams) {
+        const int rc = launch_gemv_seg_swiglu(*down, h2, d_y, s);
         if (rc <= 0) return rc;
     }
     const size_t n = (size_t)F * (size_t)M;

@@ -27,18 +27,30 @@ def test_rmsnorm():
         assert np.abs(got - want).max() <= 4e-6 * np.abs(want).max()
 
 
+def block_formats(fmt, nblocks, seed):
+    """A Format for a uniform tensor, or a tuple of format ids drawn per block (a tensor whose rows mix formats)."""
+    if not isinstance(fmt, tuple):
+        return fmt
+    return np.random.default_rng(seed).choice(np.array(fmt, dtype=np.uint8), size=nblocks)
+
+
+# OIL4 and window-stream tensors (mixed rows, other uniform formats) fuse the input transforms into one-row launches;
+# OIL8 and several activation rows take the separate kernels
 @pytest.mark.parametrize("M,D,F,fmt", [(1, 512, 768, ia.Format.OIL4), (1, 4096, 11008, ia.Format.OIL4),
-                                        (3, 512, 768, ia.Format.OIL4), (1, 256, 512, ia.Format.OIL8)])
+                                        (3, 512, 768, ia.Format.OIL4), (1, 256, 512, ia.Format.OIL8),
+                                        (1, 1024, 2816, (0, 1)), (1, 512, 768, ia.Format.SPARK_Q0),
+                                        (2, 512, 768, (0, 1, 3))])
 def test_mlp_step(M, D, F, fmt):
     rng = np.random.default_rng(D + F + M)
     mats = {}
     for name, (r, c) in (("gate", (F, D)), ("up", (F, D)), ("down", (D, F))):
         w = gaussian_weights(r * c, seed=len(name) + D) * np.float32(50.0 / np.sqrt(c))
-        mats[name] = (r, c) + ia.block_codec.quantize_tensor(w, fmt)
+        mats[name] = (r, c) + ia.block_codec.quantize_tensor(w, block_formats(fmt, r * c // 256, len(name)))
     x = rng.standard_normal((M, D)).astype(np.float32)
     dev = {k: ia.DeviceWeights.from_blocks(v[2], v[3], v[0], v[1]) for k, v in mats.items()}
     gu = ia.DeviceWeights.stack_rows([dev["gate"], dev["up"]])
-    assert (gu.rows, gu.cols) == (2 * F, D) and gu.info()["payload_bytes"] == 2 * dev["gate"].info()["payload_bytes"]
+    assert (gu.rows, gu.cols) == (2 * F, D)
+    assert gu.info()["payload_bytes"] == dev["gate"].info()["payload_bytes"] + dev["up"].info()["payload_bytes"]
     got = layers.mlp_step(gu, dev["down"], torch.from_numpy(x).cuda()).cpu().numpy()
     # oracle: the reference's steps with the matmuls in double precision
     g = O.block_gemm(mats["gate"][2], to_orc_blocks(mats["gate"][3]), F, D, x, wide=True)
@@ -57,11 +69,15 @@ def test_mlp_step(M, D, F, fmt):
 
 @pytest.mark.parametrize("M,rows,cols,fmt", [(1, 768, 512, ia.Format.OIL4), (1, 12288, 4096, ia.Format.OIL4),
                                               (1, 300, 11008, ia.Format.OIL4), (3, 768, 512, ia.Format.OIL4),
-                                              (1, 256, 512, ia.Format.OIL8)])
+                                              (1, 256, 512, ia.Format.OIL8), (1, 1000, 4096, (0, 1)),
+                                              (1, 300, 2816, (0, 1, 3, 10)), (1, 5000, 1024, ia.Format.OIL2_GRP),
+                                              (2, 300, 1024, (0, 1))])
 def test_gemv_rmsnorm(M, rows, cols, fmt):
-    """W . rmsnorm(x): one launch for one OIL4 row, norm kernel + GEMV otherwise; both against the oracle's two steps."""
+    """W . rmsnorm(x): one launch for one row of an OIL4 or window-stream tensor, norm kernel + GEMV otherwise; both
+    against the oracle's two steps."""
     rng = np.random.default_rng(rows + cols + M)
-    payload, blocks = ia.block_codec.quantize_tensor(gaussian_weights(rows * cols, seed=rows), fmt)
+    payload, blocks = ia.block_codec.quantize_tensor(gaussian_weights(rows * cols, seed=rows),
+                                                     block_formats(fmt, rows * cols // 256, rows))
     x = (rng.standard_normal((M, cols)) * 3.0).astype(np.float32)
     nw = (rng.standard_normal(cols) * 0.2).astype(np.float32)
     dw = ia.DeviceWeights.from_blocks(payload, blocks, rows, cols)
@@ -71,13 +87,14 @@ def test_gemv_rmsnorm(M, rows, cols, fmt):
     dw.close()
 
 
-def test_mlp_step_with_norm():
+@pytest.mark.parametrize("fmt", [ia.Format.OIL4, (0, 1)])
+def test_mlp_step_with_norm(fmt):
     M, D, F = 1, 1024, 2816
     rng = np.random.default_rng(9)
     mats = {}
     for name, (r, c) in (("gate", (F, D)), ("up", (F, D)), ("down", (D, F))):
         w = gaussian_weights(r * c, seed=len(name) + D) * np.float32(50.0 / np.sqrt(c))
-        mats[name] = (r, c) + ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+        mats[name] = (r, c) + ia.block_codec.quantize_tensor(w, block_formats(fmt, r * c // 256, len(name)))
     x = (rng.standard_normal((M, D)) * 2.0).astype(np.float32)
     nw = (rng.standard_normal(D) * 0.2).astype(np.float32)
     dev = {k: ia.DeviceWeights.from_blocks(v[2], v[3], v[0], v[1]) for k, v in mats.items()}
