@@ -89,10 +89,15 @@ def test_truncated_and_garbage_payloads_match_reference_rules():
 
 
 @pytest.mark.parametrize("fmt,nbytes", [(ia.Format.OIL4, 128), (ia.Format.OIL8, 256), (ia.Format.OIL2, 64),
-                                        (ia.Format.OIL1, 16), (ia.Format.SPARK_Q0, 48)])
+                                        (ia.Format.OIL1, 16), (ia.Format.SPARK_Q0, 48), (ia.Format.OIL16, 512),
+                                        (ia.Format.OIL32, 1024), (ia.Format.OIL1_GRP, 32), (ia.Format.SPARK_Q0_GRP, 48),
+                                        (ia.Format.OIL2_GRP, 80), (ia.Format.OIL4_GRP, 144), (ia.Format.OIL8_GRP, 272),
+                                        (ia.Format.OIL16_GRP, 512), (ia.Format.SPARK_SPARSE, 64),
+                                        (ia.Format.SPARK_SPARSE_GRP, 64)])
 def test_uniform_full_blocks_random_payload_bit_exact(fmt, nbytes):
-    """Tensors of full OIL1 / SPARK_Q0 / OIL2 / OIL4 / OIL8 blocks take the wavefront-per-block kernels: random payload bytes (every code, scales
-    including subnormals, infinities and NaNs) against the oracle, and quantized data against it as well."""
+    """Tensors of full blocks of one fixed-size format take the wavefront-per-block kernels: random payload bytes (every
+    code, scales and zero points including subnormals, infinities and NaNs, zero scales) against the oracle, and
+    quantized data against it as well."""
     rng = np.random.default_rng(int(fmt) + 40)
     nb = 3001
     payload = rng.integers(0, 256, nb * nbytes, dtype=np.uint8).astype(np.uint8)
