@@ -67,9 +67,11 @@ def test_mixed_format_rows():
 
 # rows that mix formats run on the tile- and format-ordered layout: the planner's half-and-half SPARK_Q0 / OIL1 plan,
 # the four-format stress plan, the grouped mixes and all fifteen formats at once; row counts that are not a multiple
-# of the tile, single-block rows, one to five activation rows
+# of the tile, single-block rows, one to nine activation rows, streams of several windows, and rows too wide for the
+# window-stream kernel's LDS (they fall back to the descriptor-driven kernel)
 @pytest.mark.parametrize("fmt_ids", [(0, 1), (0, 1, 2, 3), (7, 9, 10, 11), (6, 11, 9, 7), tuple(range(15))])
-@pytest.mark.parametrize("rows,cols,M", [(4, 256, 1), (7, 512, 2), (33, 4096, 1), (130, 2816, 3), (61, 1024, 5), (1, 1536, 4)])
+@pytest.mark.parametrize("rows,cols,M", [(4, 256, 1), (7, 512, 2), (33, 4096, 1), (130, 2816, 3), (61, 1024, 5), (1, 1536, 4),
+                                          (20, 768, 9), (3000, 512, 1), (9, 25600, 2)])
 def test_mixed_format_tiles(fmt_ids, rows, cols, M):
     rng = np.random.default_rng(rows * 7 + cols + M + len(fmt_ids))
     fmts = rng.choice(np.array(fmt_ids, dtype=np.uint8), size=rows * cols // 256)
