@@ -607,6 +607,25 @@ def main():
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))
         extra.update(bench_moe(torch, ia))
+        # the secondary legs against the same published peaks as the headline's roofline (HBM 8 TB/s, bf16 MFMA 2.5 PFLOP/s):
+        # payload GB/s for the memory-bound ones, TFLOP/s for the prefill GEMM
+        sec_roof = {}
+        for leg, key, bound in (("config1_oil8_block_gemv", "oil8_block_4096x4096_M1_GBps", "hbm"),
+                                ("config1_oil8_flat_gemv", "oil8_flat_4096x4096_M1_GBps", "hbm"),
+                                ("config2_oil4_gemv_M4", "up_gate_M4_GBps", "hbm"),
+                                ("config2_oil4_gemv_M16", "up_gate_M16_GBps", "hbm"),
+                                ("config3_planner_1p50_stack", "stack_planner_1p50_GBps", "hbm"),
+                                ("config3_planner_1p50_stack_stacked", "stack_planner_1p50_stacked_GBps", "hbm"),
+                                ("config3_spark_mix_q0_stack_stacked", "stack_spark_mix_q0_stacked_GBps", "hbm"),
+                                ("config4_prefill_M2048_N11008", "prefill_M2048_N11008_TFLOPs", "mfma"),
+                                ("config4_prefill_M512_N4096", "prefill_M512_N4096_TFLOPs", "mfma"),
+                                ("config5_moe_step", "moe_GBps", "hbm"),
+                                ("dequant_oil4_written", "dequant_oil4_11008x4096_written_GBps", "hbm")):
+            if key in extra:
+                peak = HBM_PEAK_GBS if bound == "hbm" else 2500.0
+                sec_roof[leg] = {"bound": bound, "achieved": extra[key], "peak": peak,
+                                 "unit": "GB/s" if bound == "hbm" else "TFLOP/s", "frac": round(extra[key] / peak, 4)}
+        extra["roofline_secondary"] = sec_roof
         out["extra"] = extra
     else:
         ring.close()
