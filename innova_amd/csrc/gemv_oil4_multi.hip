@@ -269,11 +269,15 @@ int get_pack_buffer(uint32_t** out) {
 
 }  // namespace
 
-// Y[m][r] for m < M: x row tok[m] (or m when tok is null) of an [xrows][ldx] activation matrix.
-// Returns 1 when the shape is outside what this kernel covers.
+// Y[m][r] for m < M: x row tok[m] (or m when tok is null) of an [xrows][ldx] activation matrix; with w2 the same
+// activations also go through a second tensor of the same width into d_y2 (the gate and up projections of an expert):
+// they are split and ordered once per pass for both.  Returns 1 when the shape is outside what this kernel covers.
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
-                           uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s) {
+                           uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2, float* d_y2,
+                           uint32_t ldy2) {
     if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
+    if (w2 && (w2->cols != w.cols || w2->rows == 0 || w2->rows > 0x7FFFFFFFull || w2->uniform_fmt != OILHIP_OIL4 ||
+               w2->uniform_stride != 128 || !d_y2)) return 1;
     static bool attr_done = false;
     if (!attr_done) {
         OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false>),
@@ -285,23 +289,30 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     uint32_t* xp = nullptr;
     if (int rc = get_pack_buffer(&xp)) return rc;
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
-    const uint32_t groups = ((uint32_t)w.rows + 15u) / 16u;
-    uint32_t grid = (uint32_t)device_cu_count();
-    if (grid > groups) grid = groups;
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
+    auto main_launch = [&](const oilhip_weights& t, float* y, uint32_t ld, bool half, int m0, int m1) {
+        const uint32_t groups = ((uint32_t)t.rows + 15u) / 16u;
+        uint32_t grid = (uint32_t)device_cu_count();
+        if (grid > groups) grid = groups;
+        if (half)
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(grid), dim3(512), lds_bytes, s, t.d_payload, xp, y,
+                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / grid, groups % grid);
+        else
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(grid), dim3(512), lds_bytes, s, t.d_payload, xp, y,
+                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / grid, groups % grid);
+    };
     for (int m0 = 0; m0 < M;) {                   // passes of 16 tokens; the last 8 or fewer as a pass of 8
         const bool half = M - m0 <= 8;
         const int m1 = half || M - m0 < 16 ? M : m0 + 16;
         hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_tok, xp, (uint32_t)w.cols, m0, m1,
                            ldx, xrows, half ? 1 : 0);
         OILHIP_HIP(hipGetLastError());
-        if (half)
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
-                               (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
-        else
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(grid), dim3(512), lds_bytes, s, w.d_payload, xp, d_y,
-                               (uint32_t)w.rows, (uint32_t)w.cols, m0, m1, ldy, groups / grid, groups % grid);
+        main_launch(w, d_y, ldy, half, m0, m1);
         OILHIP_HIP(hipGetLastError());
+        if (w2) {
+            main_launch(*w2, d_y2, ldy2, half, m0, m1);
+            OILHIP_HIP(hipGetLastError());
+        }
         m0 = m1;
     }
     return OILHIP_OK;

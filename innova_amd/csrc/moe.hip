@@ -178,8 +178,16 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
     for (int e = 0; e < E; ++e) {
         const int b = begin[(size_t)e], nt = begin[(size_t)e + 1] - b;
         if (nt == 0) continue;
-        if (int rc = expert_gemv(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)T, ws.xg, s)) return rc;
-        if (int rc = expert_gemv(*up[e], d_x, ws.tok + b, ws.u, nt, (uint32_t)T, ws.xg, s)) return rc;
+        // gate and up read the same gathered activations: uniform OIL4 experts split them once per pass for both
+        int both = 1;
+        if (gate[e]->uniform_fmt == OILHIP_OIL4 && gate[e]->uniform_stride == 128)
+            both = launch_gemv_oil4_multi(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)D, (uint32_t)F, (uint32_t)T, s, up[e], ws.u,
+                                          (uint32_t)F);
+        if (both < 0) return both;
+        if (both == 1) {
+            if (int rc = expert_gemv(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)T, ws.xg, s)) return rc;
+            if (int rc = expert_gemv(*up[e], d_x, ws.tok + b, ws.u, nt, (uint32_t)T, ws.xg, s)) return rc;
+        }
         const size_t n = (size_t)nt * (size_t)F;
         hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0, s, ws.g, ws.u, n);
         OILHIP_HIP(hipGetLastError());
