@@ -79,7 +79,7 @@ int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_ac
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2 = nullptr,
-                           float* d_y2 = nullptr, uint32_t ldy2 = 0);
+                           float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr);
 // rows that mix formats, stored tile by tile and format by format
 int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // every format, a lane per run of 32 weights

@@ -46,14 +46,14 @@ constexpr int kGroups = 4;                // groups of 16 rows per tile
 constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
 constexpr int kRedBytes = 8 * kGroups * 64 * 16;
 
-// Packed activations of one pass of 16 tokens: for block blk of the row, half h and lane l = 16*kq + t (token t) 32
+// Packed activations of one pass of 16 tokens (x, or silu(x) * x2 when x2 is given): for block blk of the row, half h and lane l = 16*kq + t (token t) 32
 // dwords: the high FP16 parts of the lane's 32 nibble positions (positions 2c, 2c+1 in dword c, c = 0..15), then the
 // low parts.  Piece j (dwords 4j .. 4j+3 of the 32) of all 64 lanes is one contiguous KB at
 // ((blk*2 + h)*8 + j)*1024 + l*16 bytes, so that a wavefront fetches it with one coalesced 16-byte load per lane.  Nibble p = 32*(kq + 4h) + s of a block holds weight
 // i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
 __global__ void __launch_bounds__(256)
-pack_x_kernel(const float* __restrict__ x, const int* __restrict__ tok, uint32_t* __restrict__ xp, uint32_t cols, int m0, int M,
-              uint32_t ldx, uint32_t xrows, int half) {
+pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
+              uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half) {
     const uint32_t id = blockIdx.x * 256u + threadIdx.x;            // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
     const uint32_t bpr = cols >> 8;
     if (id >= bpr * 2048u) return;
@@ -65,13 +65,16 @@ pack_x_kernel(const float* __restrict__ x, const int* __restrict__ tok, uint32_t
     const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
     float v[2] = {0.0f, 0.0f};
     if (src < xrows) {
-        const float* row = x + (size_t)src * ldx + (size_t)blk * 256u;
+        const size_t at = (size_t)src * ldx + (size_t)blk * 256u;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint32_t pn = 32u * (kq + 4u * h) + 2u * c + e;
             if (pn >= 4u) {
                 const uint32_t q = pn - 4u;
-                v[e] = row[q + q / 63u];
+                v[e] = x[at + q + q / 63u];
+                // x2: the activations are silu(x) * x2, the SwiGLU product in front of an expert's down projection
+                // (ExpertFFN::forward, src/moe_variants.cpp:77-91), formed here instead of in a kernel of its own
+                if (x2) v[e] = (v[e] / (1.0f + expf(-v[e]))) * x2[at + q + q / 63u];
             }
         }
     }
@@ -271,10 +274,11 @@ int get_pack_buffer(uint32_t** out) {
 
 // Y[m][r] for m < M: x row tok[m] (or m when tok is null) of an [xrows][ldx] activation matrix; with w2 the same
 // activations also go through a second tensor of the same width into d_y2 (the gate and up projections of an expert):
-// they are split and ordered once per pass for both.  Returns 1 when the shape is outside what this kernel covers.
+// they are split and ordered once per pass for both.  With d_x2 (same layout as d_x) the activations are silu(x) * x2.
+// Returns 1 when the shape is outside what this kernel covers.
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2, float* d_y2,
-                           uint32_t ldy2) {
+                           uint32_t ldy2, const float* d_x2) {
     if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
     if (w2 && (w2->cols != w.cols || w2->rows == 0 || w2->rows > 0x7FFFFFFFull || w2->uniform_fmt != OILHIP_OIL4 ||
                w2->uniform_stride != 128 || !d_y2)) return 1;
@@ -304,7 +308,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     for (int m0 = 0; m0 < M;) {                   // passes of 16 tokens; the last 8 or fewer as a pass of 8
         const bool half = M - m0 <= 8;
         const int m1 = half || M - m0 < 16 ? M : m0 + 16;
-        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_tok, xp, (uint32_t)w.cols, m0, m1,
+        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_x2, d_tok, xp, (uint32_t)w.cols, m0, m1,
                            ldx, xrows, half ? 1 : 0);
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, half, m0, m1);

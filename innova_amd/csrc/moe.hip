@@ -56,6 +56,26 @@ __global__ void __launch_bounds__(256) combine_kernel(const float* __restrict__ 
     if (threadIdx.x == 0) atomicAdd(zacc, (part[0] + part[1]) + (part[2] + part[3]));
 }
 
+// The same for a list without repeated tokens (what top-k routing produces): every (row, column) of the list has an
+// output element of its own, so the rows go side by side, blockIdx.y = list entry.
+__global__ void __launch_bounds__(256) combine_distinct_kernel(const float* __restrict__ o, const int* __restrict__ tok,
+                                                               const float* __restrict__ wgt, uint32_t D,
+                                                               float* __restrict__ out, double* __restrict__ zacc) {
+    __shared__ double part[4];
+    const uint32_t d = blockIdx.x * 256 + threadIdx.x, i = blockIdx.y;
+    const float w = wgt[i];
+    double z = 0.0;
+    if (d < D && w > 0.0f) {
+        const float v = w * o[(size_t)i * D + d];
+        out[(size_t)tok[i] * D + d] += v;
+        z = (double)v * (double)v;
+    }
+    for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = z;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(zacc, (part[0] + part[1]) + (part[2] + part[3]));
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
@@ -167,6 +187,11 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                 }
     }
     begin[(size_t)E] = (int)tok.size();
+    // a list is in ascending token order, so a token listed twice sits next to itself
+    std::vector<char> distinct((size_t)E, 1);
+    for (int e = 0; e < E; ++e)
+        for (int i = begin[(size_t)e] + 1; i < begin[(size_t)e + 1]; ++i)
+            if (tok[(size_t)i] == tok[(size_t)i - 1]) distinct[(size_t)e] = 0;
     if (!tok.empty()) {
         OILHIP_HIP(hipMemcpyAsync(ws.tok, tok.data(), tok.size() * 4, hipMemcpyHostToDevice, s));
         OILHIP_HIP(hipMemcpyAsync(ws.wgt, wgt.data(), wgt.size() * 4, hipMemcpyHostToDevice, s));
@@ -188,12 +213,24 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
             if (int rc = expert_gemv(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)T, ws.xg, s)) return rc;
             if (int rc = expert_gemv(*up[e], d_x, ws.tok + b, ws.u, nt, (uint32_t)T, ws.xg, s)) return rc;
         }
-        const size_t n = (size_t)nt * (size_t)F;
-        hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0, s, ws.g, ws.u, n);
-        OILHIP_HIP(hipGetLastError());
-        if (int rc = expert_gemv(*down[e], ws.g, nullptr, ws.o, nt, (uint32_t)nt, ws.xg, s)) return rc;
-        hipLaunchKernelGGL(combine_kernel, dim3((uint32_t)((D + 255) / 256)), dim3(256), 0, s, ws.o, ws.tok + b, ws.wgt + b, nt,
-                           (uint32_t)D, d_out, ws.z);
+        // silu(gate) * up: formed while the down projection's activations are split (uniform OIL4), or by a kernel of its own
+        int fused = 1;
+        if (down[e]->uniform_fmt == OILHIP_OIL4 && down[e]->uniform_stride == 128)
+            fused = launch_gemv_oil4_multi(*down[e], ws.g, nullptr, ws.o, nt, (uint32_t)F, (uint32_t)D, (uint32_t)nt, s, nullptr, nullptr, 0,
+                                           ws.u);
+        if (fused < 0) return fused;
+        if (fused == 1) {
+            const size_t n = (size_t)nt * (size_t)F;
+            hipLaunchKernelGGL(swiglu_kernel, dim3((uint32_t)std::min<size_t>((n + 255) / 256, 4096)), dim3(256), 0, s, ws.g, ws.u, n);
+            OILHIP_HIP(hipGetLastError());
+            if (int rc = expert_gemv(*down[e], ws.g, nullptr, ws.o, nt, (uint32_t)nt, ws.xg, s)) return rc;
+        }
+        if (distinct[(size_t)e])
+            hipLaunchKernelGGL(combine_distinct_kernel, dim3((uint32_t)((D + 255) / 256), (uint32_t)nt), dim3(256), 0, s, ws.o, ws.tok + b,
+                               ws.wgt + b, (uint32_t)D, d_out, ws.z);
+        else
+            hipLaunchKernelGGL(combine_kernel, dim3((uint32_t)((D + 255) / 256)), dim3(256), 0, s, ws.o, ws.tok + b, ws.wgt + b, nt,
+                               (uint32_t)D, d_out, ws.z);
         OILHIP_HIP(hipGetLastError());
     }
     if (dropped) *dropped = drop;
