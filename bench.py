@@ -587,6 +587,11 @@ def main():
         yd = torch.empty((1, COLS), dtype=torch.float32, device="cuda")
         s_d, _ = time_ring(torch, ring_d, xd, yd, 2000, 100)
         extra["down_M1_GBps"] = round(ring_d.payload_bytes / s_d / 1e9, 1)
+        for M in (4, 16):
+            xm = torch.randn(M, ROWS, device="cuda")
+            ym = torch.empty((M, COLS), dtype=torch.float32, device="cuda")
+            s_m, _ = time_ring(torch, ring_d, xm, ym, 400, 40)
+            extra[f"down_M{M}_GBps"] = round(ring_d.payload_bytes / s_m / 1e9, 1)
         ring_d.close()
         # weights-only decode rate of a Llama-7B-shaped stack: per layer 4 x (4096x4096), 2 x up/gate, 1 x down
         t_qkvo = None
