@@ -53,9 +53,15 @@ constexpr int kRedBytes = 8 * kGroups * 64 * 16;
 // i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
-              uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half) {
+              uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
+              float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld) {
     const uint32_t id = blockIdx.x * 256u + threadIdx.x;            // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
     const uint32_t bpr = cols >> 8;
+    // outputs that the main kernel accumulates into (rows cut along K between workgroups) start at zero
+    if (yc0)
+        for (uint32_t i = id; i < yc0_rows * (uint32_t)(M - m0); i += bpr * 2048u) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
+    if (yc1)
+        for (uint32_t i = id; i < yc1_rows * (uint32_t)(M - m0); i += bpr * 2048u) yc1[(size_t)(m0 + i / yc1_rows) * yc1_ld + i % yc1_rows] = 0.0f;
     if (id >= bpr * 2048u) return;
     const uint32_t c = id & 15u, lane = (id >> 4) & 63u, h = (id >> 10) & 1u, blk = id >> 11;
     const uint32_t t = lane & 15u, kq = lane >> 4;
@@ -95,7 +101,8 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
 template <bool HALF>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, float* __restrict__ y,
-                       uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem) {
+                       uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
+                       uint32_t ksplit) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][64 lanes][4]
@@ -103,11 +110,15 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, kq = lane >> 4;
     const uint32_t bpr = cols >> 8, row_bytes = bpr * 128u;
-    const uint32_t npass = (bpr + 15u) / 16u;
+    // ksplit > 1: workgroup blockIdx.x takes part blockIdx.x % ksplit of every row (at most 16 blocks, so its
+    // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit, and adds into y
+    const uint32_t slab = ksplit > 1u ? blockIdx.x / ksplit : blockIdx.x, part = ksplit > 1u ? blockIdx.x % ksplit : 0u;
+    const uint32_t blk_lo = bpr * part / ksplit, blk_hi = bpr * (part + 1u) / ksplit;
+    const uint32_t npass = (blk_hi - blk_lo + 15u) / 16u;
 
     // groups of 16 rows [g0, g1) of this workgroup
     auto group_begin = [&](uint32_t j) { return j * g_base + (j < g_rem ? j : g_rem); };
-    const uint32_t g0 = group_begin(blockIdx.x), g1 = group_begin(blockIdx.x + 1);
+    const uint32_t g0 = group_begin(slab), g1 = group_begin(slab + 1);
     const uint32_t ntiles = (g1 - g0 + kGroups - 1) / kGroups;
     const uint64_t remain = (uint64_t)(rows - g0 * 16u) * row_bytes;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -125,8 +136,8 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         const uint32_t r = g * 16u + li;
 #pragma unroll
         for (int b2 = 0; b2 < 2; ++b2) {
-            const uint32_t blk = pass * 16u + wave * 2u + b2;
-            const bool ok = g < g1 && r < rows && blk < bpr;
+            const uint32_t blk = blk_lo + pass * 16u + wave * 2u + b2;
+            const bool ok = g < g1 && r < rows && blk < blk_hi;
             const uint32_t off = (r - g0 * 16u) * row_bytes + blk * 128u + kq * 16u;
             wv[buf][b2][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off : kOobOffset, 0, 0);
             wv[buf][b2][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off + 64u : kOobOffset, 0, 0);
@@ -138,10 +149,10 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     auto load_b = [&](uint32_t pass) {
 #pragma unroll
         for (int b2 = 0; b2 < 2; ++b2) {
-            const uint32_t blk = pass * 16u + wave * 2u + b2;
+            const uint32_t blk = blk_lo + pass * 16u + wave * 2u + b2;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint32_t off = blk < bpr ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
+                const uint32_t off = blk < blk_hi ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const u32x4 vh = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 1024u * j, 0, 0);
@@ -184,7 +195,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                 const bool g_on = tg0 + g < g1;                            // wave-uniform
 #pragma unroll
                 for (int b2 = 0; b2 < 2; ++b2) {
-                    const bool on = g_on && pass * 16u + wave * 2u + b2 < bpr;     // wave-uniform
+                    const bool on = g_on && blk_lo + pass * 16u + wave * 2u + b2 < blk_hi;     // wave-uniform
                     if (!on) continue;
                     const u32x4 w0 = wv[g & 1][b2][0], w1 = wv[g & 1][b2][1];
                     v4f t0 = v4f{0.f, 0.f, 0.f, 0.f}, t1 = v4f{0.f, 0.f, 0.f, 0.f};   // this block: Lh xh, and Lh xl + Ll xh
@@ -246,7 +257,8 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                     s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j) * 4 + (i & 3u)];
                     if (HALF) s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j + 8u) * 4 + (i & 3u)];
                 }
-                y[(size_t)(m0 + j) * ldy + r] = s;
+                if (ksplit > 1u) unsafeAtomicAdd(y + (size_t)(m0 + j) * ldy + r, s);
+                else y[(size_t)(m0 + j) * ldy + r] = s;
             }
         }
         if (tile + 1 < ntiles) __syncthreads();                            // red is rewritten by the next tile
@@ -294,22 +306,32 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     if (int rc = get_pack_buffer(&xp)) return rc;
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
+    // rows wider than one K-pass (16 blocks): the row is cut into parts of at most 16 blocks that go to different
+    // workgroups, so that a workgroup fetches the split activations of its part once instead of once per pass and tile
+    // (the parts' sums meet through float atomics: with three or more parts the order of the additions, and with it the
+    // last bits of y, can differ between launches)
+    auto split_of = [&](const oilhip_weights&) -> uint32_t {
+        const uint32_t np = (bpr + 15u) / 16u;
+        return np >= 2u && np <= (uint32_t)device_cu_count() ? np : 1u;
+    };
     auto main_launch = [&](const oilhip_weights& t, float* y, uint32_t ld, bool half, int m0, int m1) {
         const uint32_t groups = ((uint32_t)t.rows + 15u) / 16u;
-        uint32_t grid = (uint32_t)device_cu_count();
-        if (grid > groups) grid = groups;
+        const uint32_t ks = split_of(t);
+        uint32_t slabs = (uint32_t)device_cu_count() / ks;
+        if (slabs > groups) slabs = groups;
         if (half)
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(grid), dim3(512), lds_bytes, s, t.d_payload, xp, y,
-                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / grid, groups % grid);
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y,
+                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
         else
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(grid), dim3(512), lds_bytes, s, t.d_payload, xp, y,
-                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / grid, groups % grid);
+            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y,
+                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
     };
     for (int m0 = 0; m0 < M;) {                   // passes of 16 tokens; the last 8 or fewer as a pass of 8
         const bool half = M - m0 <= 8;
         const int m1 = half || M - m0 < 16 ? M : m0 + 16;
         hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_x2, d_tok, xp, (uint32_t)w.cols, m0, m1,
-                           ldx, xrows, half ? 1 : 0);
+                           ldx, xrows, half ? 1 : 0, split_of(w) > 1u ? d_y : nullptr, (uint32_t)w.rows, ldy,
+                           w2 && split_of(*w2) > 1u ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, half, m0, m1);
         OILHIP_HIP(hipGetLastError());

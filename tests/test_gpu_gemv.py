@@ -121,6 +121,21 @@ def test_oil4_multi_token_counts(rows, cols, M):
     assert err <= TOL
 
 
+# rows wider than 16 blocks are cut along K between workgroups that add into y: the output buffer is cleared by the
+# launch itself (it holds NaNs here), several row tiles per workgroup, parts of unequal length, both pass widths
+@pytest.mark.parametrize("rows,cols,M", [(9000, 8192, 5), (9000, 8192, 17), (5000, 11008, 16), (700, 8448, 24)])
+def test_oil4_multi_token_rows_cut_along_k(rows, cols, M):
+    w = gaussian_weights(rows * cols, rows + M)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    X = np.random.default_rng(rows + M + 1).standard_normal((M, cols)).astype(np.float32)
+    want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        out = torch.full((M, rows), float("nan"), device="cuda")
+        for _ in range(2):                                   # the second call finds the first call's sums in y
+            got = dw.gemv(torch.from_numpy(X).cuda(), out=out).cpu().numpy()
+            assert rel_l2(got, want) <= TOL
+
+
 # the OIL8 kernel: one and several slabs per row, rows not a multiple of the wave count, several chunks per
 # wavefront (tall tensors), every activation-row grouping, a partial last column set
 @pytest.mark.parametrize("rows,cols", [(64, 4096), (1000, 4096), (37, 11008), (300, 1024), (5000, 256), (3, 256),
