@@ -44,7 +44,10 @@ __device__ __forceinline__ uint32_t split_level(float L) {
 
 constexpr int kGroups = 4;                // groups of 16 rows per tile
 constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
-constexpr int kRedBytes = 8 * kGroups * 64 * 16;
+// partial sums of a 16 x 16 tile, accumulator lane 16 q + j, element v at float q*68 + 4 j + v of 272: for one token j the
+// 64 (group, row) pairs of a tile fall into 64 different banks
+constexpr int kRedTile = 272;
+constexpr int kRedBytes = 8 * kGroups * kRedTile * 4;
 
 // Packed activations of one pass of 16 tokens (x, or silu(x) * x2 when x2 is given): for block blk of the row, half h and lane l = 16*kq + t (token t) 32
 // dwords: the high FP16 parts of the lane's 32 nibble positions (positions 2c, 2c+1 in dword c, c = 0..15), then the
@@ -105,7 +108,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                        uint32_t ksplit) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
-    float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][64 lanes][4]
+    float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, kq = lane >> 4;
@@ -243,7 +246,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 #pragma unroll
         for (int g = 0; g < kGroups; ++g) {
             const v4f d = acc[g];
-            *reinterpret_cast<float4*>(red + (((size_t)wave * kGroups + g) * 64 + lane) * 4) = make_float4(d[0], d[1], d[2], d[3]);
+            *reinterpret_cast<float4*>(red + ((size_t)wave * kGroups + g) * kRedTile + kq * 68u + li * 4u) = make_float4(d[0], d[1], d[2], d[3]);
         }
         __syncthreads();
         for (uint32_t o = tid; o < kGroups * 16u * 16u; o += 512u) {
@@ -254,8 +257,8 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                 float s = 0.f;
 #pragma unroll
                 for (uint32_t w8 = 0; w8 < 8; ++w8) {
-                    s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j) * 4 + (i & 3u)];
-                    if (HALF) s += red[(((size_t)w8 * kGroups + g) * 64 + (i >> 2) * 16u + j + 8u) * 4 + (i & 3u)];
+                    s += red[((size_t)w8 * kGroups + g) * kRedTile + (i >> 2) * 68u + j * 4u + (i & 3u)];
+                    if (HALF) s += red[((size_t)w8 * kGroups + g) * kRedTile + (i >> 2) * 68u + (j + 8u) * 4u + (i & 3u)];
                 }
                 if (ksplit > 1u) unsafeAtomicAdd(y + (size_t)(m0 + j) * ldy + r, s);
                 else y[(size_t)(m0 + j) * ldy + r] = s;
