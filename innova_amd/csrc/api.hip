@@ -465,8 +465,14 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
         if (rc == 1 && M > 2 && M <= 4) rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
-    if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256 && M <= 4) {
-        const int rc = launch_gemv_oil8(*w, d_x, d_y, M, (hipStream_t)stream);
+    if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256) {
+        // the register-resident kernel takes up to four activation rows per launch
+        int rc = 1;
+        for (int m0 = 0; m0 < M; m0 += 4) {
+            rc = launch_gemv_oil8(*w, d_x + (size_t)m0 * w->cols, d_y + (size_t)m0 * w->rows, M - m0 < 4 ? M - m0 : 4,
+                                  (hipStream_t)stream);
+            if (rc != 0) break;
+        }
         if (rc <= 0) return rc;
     }
     if (w->seg.nstreams) {

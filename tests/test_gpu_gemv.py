@@ -148,6 +148,13 @@ def test_oil8_fast_kernel_shapes(rows, cols, M):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("rows,cols,M", [(1000, 4096, 6), (300, 1024, 9), (37, 11008, 5), (4096, 4096, 16)])
+def test_oil8_more_than_four_activation_rows(rows, cols, M):
+    """Batches beyond four rows run as consecutive launches of four rows or fewer."""
+    err, *_ = run_case(ia.Format.OIL8, rows, cols, M, seed=5 * rows + cols + M)
+    assert err <= TOL
+
+
 def test_oil8_special_blocks():
     """Zero blocks, underflowing scales, huge outliers, zero activations, activations with a large common offset
     (the kernel forms sum(q x) - 127.5 sum(x), which must not lose the small difference)."""
