@@ -208,6 +208,7 @@ constexpr int PLD = PK;                     // LDS row pitch in bf16: 128 bytes 
                                             // row is XOR-swizzled with (row / 2) % 8 so that the tile stores (2 rows x 8
                                             // chunks per 16 lanes) and the fragment reads (16 rows x 1 chunk) touch every bank once
 constexpr int PBM = 256, PBN = 128;
+__device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> 1) & 7u; }
 
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
@@ -269,7 +270,7 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
             const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
-            *reinterpret_cast<u32x4*>(As + (buf * PBM + row) * PLD + ((kc ^ ((row >> 1) & 7u)) * 8u)) = ar[set][c];
+            *reinterpret_cast<u32x4*>(As + (buf * PBM + row) * PLD + ((kc ^ swz(row)) * 8u)) = ar[set][c];
         }
         const float scale = __half2float(__ushort_as_half((unsigned short)sr[set]));
         uint32_t packed[8];
@@ -278,10 +279,14 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
             const bf16x2 pr = bf16x2{(__bf16)(t[j].x * scale), (__bf16)(t[j].y * scale)};
             packed[j] = *reinterpret_cast<const uint32_t*>(&pr);
         }
-        const uint32_t sb = (brow >> 1) & 7u;
+        const uint32_t sb = swz(brow);
         __bf16* dst = Bs + (buf * PBN + brow) * PLD;
-        *reinterpret_cast<u32x4*>(dst + (((2u * bq) ^ sb) * 8u)) = u32x4{packed[0], packed[1], packed[2], packed[3]};
-        *reinterpret_cast<u32x4*>(dst + (((2u * bq + 1u) ^ sb) * 8u)) = u32x4{packed[4], packed[5], packed[6], packed[7]};
+        // odd rows store their second 16 bytes first: the two rows that share a swizzle value then fall into different
+        // banks within one store instruction
+        const bool odd = brow & 1u;
+        const u32x4 c0 = u32x4{packed[0], packed[1], packed[2], packed[3]}, c1 = u32x4{packed[4], packed[5], packed[6], packed[7]};
+        *reinterpret_cast<u32x4*>(dst + (((2u * bq + (odd ? 1u : 0u)) ^ sb) * 8u)) = odd ? c1 : c0;
+        *reinterpret_cast<u32x4*>(dst + (((2u * bq + (odd ? 0u : 1u)) ^ sb) * 8u)) = odd ? c0 : c1;
     };
     auto store_tiles = [&](int set, int buf) {
         f32x2 t[8];
@@ -297,7 +302,7 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
-    const uint32_t sw = ((lane & 31u) >> 1) & 7u;
+    const uint32_t sw = swz(lane & 31u);
     auto step_mfmas = [&](int buf) {
         const __bf16* ap = As + (buf * PBM + wm * 64u + (lane & 31u)) * PLD;
         const __bf16* bp = Bs + (buf * PBN + wn * 64u + (lane & 31u)) * PLD;
