@@ -1,5 +1,5 @@
 // gemv_oil4_multi.hip -- decode GEMV over uniform OIL4 tensors for a handful of activation rows
-// (2..16 tokens per pass): Qwen35Engine::gemm with small B (src/adapters/tools/qwen35_engine.cpp:47-85)
+// (up to 8, 16 or 32 tokens per pass): Qwen35Engine::gemm with small B (src/adapters/tools/qwen35_engine.cpp:47-85)
 // and the per-expert batches of moe_dispatch_batched (src/moe_variants.cpp:767-827).
 //
 // The products run on the matrix cores in FP16 with both operands split in two: a level L of the table is
@@ -18,6 +18,9 @@
 // activations are split and laid out in this operand order once per launch by pack_x_kernel (every workgroup needs
 // all of them), so the main kernel fetches its 128 operand dwords with plain 16-byte loads.  Partial sums of the
 // wavefronts are added through LDS once per tile of 64 rows.
+// Batches of more than 16 tokens run passes of 32: a wavefront then owns one block per K-pass and multiplies each
+// decoded weight operand with the activations of two token tiles (the table look-ups, which bound the main loop, are
+// shared), a row tile is 32 rows.
 #include <hip/hip_fp16.h>
 
 #include <mutex>
@@ -42,7 +45,7 @@ __device__ __forceinline__ uint32_t split_level(float L) {
     return (uint32_t)__half_as_ushort(h) | ((uint32_t)__half_as_ushort(l) << 16);
 }
 
-constexpr int kGroups = 4;                // groups of 16 rows per tile
+constexpr int kGroups = 4;                // 16 x 16 partial-sum tiles per wavefront and row tile (groups of 16 rows x token tiles)
 constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
 // partial sums of a 16 x 16 tile, accumulator lane 16 q + j, element v at float q*68 + 4 j + v of 272: for one token j the
 // 64 (group, row) pairs of a tile fall into 64 different banks
@@ -58,13 +61,18 @@ __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
               uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
               float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld) {
-    const uint32_t id = blockIdx.x * 256u + threadIdx.x;            // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
     const uint32_t bpr = cols >> 8;
     // outputs that the main kernel accumulates into (rows cut along K between workgroups) start at zero
+    const uint32_t gid = blockIdx.x * 256u + threadIdx.x, gn = gridDim.x * 256u;
     if (yc0)
-        for (uint32_t i = id; i < yc0_rows * (uint32_t)(M - m0); i += bpr * 2048u) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
+        for (uint32_t i = gid; i < yc0_rows * (uint32_t)(M - m0); i += gn) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
     if (yc1)
-        for (uint32_t i = id; i < yc1_rows * (uint32_t)(M - m0); i += bpr * 2048u) yc1[(size_t)(m0 + i / yc1_rows) * yc1_ld + i % yc1_rows] = 0.0f;
+        for (uint32_t i = gid; i < yc1_rows * (uint32_t)(M - m0); i += gn) yc1[(size_t)(m0 + i / yc1_rows) * yc1_ld + i % yc1_rows] = 0.0f;
+    // a pass of 32 tokens is two tiles of 16: blocks bpr*8 .. of the grid pack tokens m0 + 16 .. behind the first tile
+    const uint32_t tile = blockIdx.x / (bpr * 8u);
+    const uint32_t id = (blockIdx.x - tile * bpr * 8u) * 256u + threadIdx.x;   // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
+    m0 += 16 * (int)tile;
+    xp += (size_t)tile * bpr * 4096u;
     if (id >= bpr * 2048u) return;
     const uint32_t c = id & 15u, lane = (id >> 4) & 63u, h = (id >> 10) & 1u, blk = id >> 11;
     const uint32_t t = lane & 15u, kq = lane >> 4;
@@ -101,7 +109,10 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
 // HALF: passes of 8 tokens.  The activation operand then holds high parts (columns 0..7) and low parts (columns 8..15)
 // at once, so L x = (Lh + Ll)(xh + xl) takes two matrix instructions per 32 columns instead of three, the activations
 // are half as many bytes, and an output is the sum of accumulator columns j and j + 8.
-template <bool HALF>
+// NT = 2: passes of 32 tokens.  A wavefront then owns one block of the row per K-pass (8 blocks per pass) and keeps
+// the split activations of two token tiles of it, so a decoded weight operand serves two matrix instructions per
+// product term; a row tile is two groups of 16 rows.
+template <bool HALF, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, float* __restrict__ y,
                        uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
@@ -116,30 +127,34 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     // ksplit > 1: workgroup blockIdx.x takes part blockIdx.x % ksplit of every row (at most 16 blocks, so its
     // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit, and adds into y
     const uint32_t slab = ksplit > 1u ? blockIdx.x / ksplit : blockIdx.x, part = ksplit > 1u ? blockIdx.x % ksplit : 0u;
+    static_assert(NT == 1 || !HALF, "passes of 8 tokens have one token tile");
+    constexpr int BPW = NT == 2 ? 1 : 2;                                   // blocks of the row per wavefront and pass
+    constexpr uint32_t PB = 8u * BPW;                                      // blocks per pass
+    constexpr int KG = kGroups / NT;                                       // groups of 16 rows per tile
     const uint32_t blk_lo = bpr * part / ksplit, blk_hi = bpr * (part + 1u) / ksplit;
-    const uint32_t npass = (blk_hi - blk_lo + 15u) / 16u;
+    const uint32_t npass = (blk_hi - blk_lo + PB - 1u) / PB;
 
     // groups of 16 rows [g0, g1) of this workgroup
     auto group_begin = [&](uint32_t j) { return j * g_base + (j < g_rem ? j : g_rem); };
     const uint32_t g0 = group_begin(slab), g1 = group_begin(slab + 1);
-    const uint32_t ntiles = (g1 - g0 + kGroups - 1) / kGroups;
+    const uint32_t ntiles = (g1 - g0 + KG - 1) / KG;
     const uint64_t remain = (uint64_t)(rows - g0 * 16u) * row_bytes;
     const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(W + (size_t)g0 * 16u * row_bytes), 0, (int)(remain < 0x80000000ull ? remain : 0x80000000ull), 0x00020000);
-    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xp, 0, (int)(bpr * 128u * 128u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)xp, 0, (int)(bpr * 128u * 128u * NT), 0x00020000);
 
-    // activations of this wavefront's two blocks, token li, chunks kq and kq+4: FP16 pairs (positions 2c, 2c+1),
-    // high parts and low parts
+    // activations of this wavefront's two blocks (NT = 2: of its block for two token tiles), token li, chunks kq and
+    // kq+4: FP16 pairs (positions 2c, 2c+1), high parts and low parts
     uint32_t bh[2][2][16], bl[HALF ? 1 : 2][HALF ? 1 : 2][HALF ? 1 : 16];
-    v4f acc[kGroups];
+    v4f acc[kGroups];                      // [group][token tile]
     const uint32_t lanebase = (lane & 31u) * 8u;
 
-    u32x4 wv[2][2][2];                     // [buffer][block of the pair][half]
+    u32x4 wv[2][BPW][2];                   // [buffer][block of the wavefront][half]
     auto issue_group = [&](int buf, uint32_t g, uint32_t pass) {
         const uint32_t r = g * 16u + li;
 #pragma unroll
-        for (int b2 = 0; b2 < 2; ++b2) {
-            const uint32_t blk = blk_lo + pass * 16u + wave * 2u + b2;
+        for (int b2 = 0; b2 < BPW; ++b2) {
+            const uint32_t blk = blk_lo + pass * PB + wave * BPW + b2;
             const bool ok = g < g1 && r < rows && blk < blk_hi;
             const uint32_t off = (r - g0 * 16u) * row_bytes + blk * 128u + kq * 16u;
             wv[buf][b2][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off : kOobOffset, 0, 0);
@@ -151,11 +166,11 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     // loads of 16 bytes per block half
     auto load_b = [&](uint32_t pass) {
 #pragma unroll
-        for (int b2 = 0; b2 < 2; ++b2) {
-            const uint32_t blk = blk_lo + pass * 16u + wave * 2u + b2;
+        for (int b2 = 0; b2 < 2; ++b2) {   // NT = 2: b2 is the token tile, whose activations follow those of tile 0
+            const uint32_t blk = blk_lo + pass * PB + wave * BPW + (NT == 2 ? 0 : b2);
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
-                const uint32_t off = blk < blk_hi ? (blk * 2u + h) * 8192u + lane * 16u : kOobOffset;
+                const uint32_t off = blk < blk_hi ? (blk * 2u + h) * 8192u + lane * 16u + (NT == 2 ? b2 * bpr * 16384u : 0u) : kOobOffset;
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const u32x4 vh = __builtin_amdgcn_raw_buffer_load_b128(xrsrc, off == kOobOffset ? kOobOffset : off + 1024u * j, 0, 0);
@@ -184,59 +199,71 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     bool table_synced = false;
 
     for (uint32_t tile = 0; tile < ntiles; ++tile) {
-        const uint32_t tg0 = g0 + tile * kGroups;
+        const uint32_t tg0 = g0 + tile * KG;
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) acc[g] = v4f{0.f, 0.f, 0.f, 0.f};
+        for (int a = 0; a < kGroups; ++a) acc[a] = v4f{0.f, 0.f, 0.f, 0.f};
         for (uint32_t pass = 0; pass < npass; ++pass) {
             if (tile > 0 || pass > 0) issue_group(0, tg0, pass);
             if (npass > 1 || tile == 0) load_b(pass);
             if (!table_synced) { __syncthreads(); table_synced = true; }   // the level table is complete
             // ---- main loop: groups of the tile, two blocks each -------------------------------------------
 #pragma unroll
-            for (int g = 0; g < kGroups; ++g) {
-                if (g + 1 < kGroups) issue_group((g + 1) & 1, tg0 + g + 1, pass);
+            for (int g = 0; g < KG; ++g) {
+                if (g + 1 < KG) issue_group((g + 1) & 1, tg0 + g + 1, pass);
                 const bool g_on = tg0 + g < g1;                            // wave-uniform
 #pragma unroll
-                for (int b2 = 0; b2 < 2; ++b2) {
-                    const bool on = g_on && blk_lo + pass * 16u + wave * 2u + b2 < blk_hi;     // wave-uniform
+                for (int b2 = 0; b2 < BPW; ++b2) {
+                    const bool on = g_on && blk_lo + pass * PB + wave * BPW + b2 < blk_hi;     // wave-uniform
                     if (!on) continue;
                     const u32x4 w0 = wv[g & 1][b2][0], w1 = wv[g & 1][b2][1];
-                    v4f t0 = v4f{0.f, 0.f, 0.f, 0.f}, t1 = v4f{0.f, 0.f, 0.f, 0.f};   // this block: Lh xh, and Lh xl + Ll xh
+                    v4f t0[NT], t1[NT];                                    // this block: Lh xh, and Lh xl + Ll xh, per token tile
+#pragma unroll
+                    for (int t = 0; t < NT; ++t) { t0[t] = v4f{0.f, 0.f, 0.f, 0.f}; t1[t] = v4f{0.f, 0.f, 0.f, 0.f}; }
 #pragma unroll
                     for (int h = 0; h < 2; ++h) {
                         const u32x4 wh = h == 0 ? w0 : w1;
                         const uint32_t wd[4] = {wh.x, wh.y, wh.z, wh.w};
-                        uint32_t ah[16], al[16];
+                        constexpr int DS = NT == 2 ? 2 : 4;                // dwords decoded per batch of table reads
 #pragma unroll
-                        for (int d = 0; d < 4; ++d) {
+                        for (int d0 = 0; d0 < 4; d0 += DS) {
+                            uint32_t ah[4 * DS], al[4 * DS];
 #pragma unroll
-                            for (int J = 0; J < 4; ++J) {
-                                const uint32_t addr = __builtin_amdgcn_perm(wd[d], lanebase, 0x0C0C0000u | ((4u + J) << 8));
-                                const u32x2 e = *(lds_cu32x2*)(uintptr_t)addr;
-                                ah[4 * d + J] = e.x; al[4 * d + J] = e.y;
+                            for (int d = 0; d < DS; ++d) {
+#pragma unroll
+                                for (int J = 0; J < 4; ++J) {
+                                    const uint32_t addr = __builtin_amdgcn_perm(wd[d0 + d], lanebase, 0x0C0C0000u | ((4u + J) << 8));
+                                    const u32x2 e = *(lds_cu32x2*)(uintptr_t)addr;
+                                    ah[4 * d + J] = e.x; al[4 * d + J] = e.y;
+                                }
                             }
-                        }
-                        __builtin_amdgcn_sched_barrier(0);                 // all 16 table reads in flight before the first product
+                            __builtin_amdgcn_sched_barrier(0);             // the batch's table reads in flight before its first product
 #pragma unroll
-                        for (int d = 0; d < 4; ++d) {
-                            const h8 Ah = __builtin_bit_cast(h8, u32x4{ah[4 * d], ah[4 * d + 1], ah[4 * d + 2], ah[4 * d + 3]});
-                            const h8 Al = __builtin_bit_cast(h8, u32x4{al[4 * d], al[4 * d + 1], al[4 * d + 2], al[4 * d + 3]});
-                            const h8 Bh = __builtin_bit_cast(h8, u32x4{bh[b2][h][4 * d], bh[b2][h][4 * d + 1], bh[b2][h][4 * d + 2], bh[b2][h][4 * d + 3]});
-                            t0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bh, t0, 0, 0, 0);
-                            if constexpr (!HALF) {
-                                const h8 Bl = __builtin_bit_cast(h8, u32x4{bl[b2][h][4 * d], bl[b2][h][4 * d + 1], bl[b2][h][4 * d + 2], bl[b2][h][4 * d + 3]});
-                                t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bl, t1, 0, 0, 0);
+                            for (int d = 0; d < DS; ++d) {
+                                const int dd = d0 + d;
+                                const h8 Ah = __builtin_bit_cast(h8, u32x4{ah[4 * d], ah[4 * d + 1], ah[4 * d + 2], ah[4 * d + 3]});
+                                const h8 Al = __builtin_bit_cast(h8, u32x4{al[4 * d], al[4 * d + 1], al[4 * d + 2], al[4 * d + 3]});
+#pragma unroll
+                                for (int t = 0; t < NT; ++t) {
+                                    const int s2 = NT == 2 ? t : b2;       // register set of the activations
+                                    const h8 Bh = __builtin_bit_cast(h8, u32x4{bh[s2][h][4 * dd], bh[s2][h][4 * dd + 1], bh[s2][h][4 * dd + 2], bh[s2][h][4 * dd + 3]});
+                                    t0[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bh, t0[t], 0, 0, 0);
+                                    if constexpr (!HALF) {
+                                        const h8 Bl = __builtin_bit_cast(h8, u32x4{bl[s2][h][4 * dd], bl[s2][h][4 * dd + 1], bl[s2][h][4 * dd + 2], bl[s2][h][4 * dd + 3]});
+                                        t1[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Ah, Bl, t1[t], 0, 0, 0);
+                                    }
+                                    t1[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, Bh, t1[t], 0, 0, 0);
+                                }
                             }
-                            t1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(Al, Bh, t1, 0, 0, 0);
+                            __builtin_amdgcn_sched_barrier(0);
                         }
-                        __builtin_amdgcn_sched_barrier(0);
                     }
                     // the block's FP16 scale of row r sits in the low half of the first dword of lane r (kq = 0)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         const uint32_t sbits = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((4u * kq + v) * 4u), (int)w0.x) & 0xFFFFu;
                         const float scale = __half2float(__ushort_as_half((unsigned short)sbits));
-                        acc[g][v] = __fmaf_rn(t0[v] + t1[v], scale, acc[g][v]);
+#pragma unroll
+                        for (int t = 0; t < NT; ++t) acc[g * NT + t][v] = __fmaf_rn(t0[t][v] + t1[t][v], scale, acc[g * NT + t][v]);
                     }
                 }
             }
@@ -244,24 +271,26 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         // ---- tile finished: add the wavefronts' partial sums (the staging areas are idle now) ------------------
         __syncthreads();
 #pragma unroll
-        for (int g = 0; g < kGroups; ++g) {
-            const v4f d = acc[g];
-            *reinterpret_cast<float4*>(red + ((size_t)wave * kGroups + g) * kRedTile + kq * 68u + li * 4u) = make_float4(d[0], d[1], d[2], d[3]);
+        for (int a = 0; a < kGroups; ++a) {
+            const v4f d = acc[a];
+            *reinterpret_cast<float4*>(red + ((size_t)wave * kGroups + a) * kRedTile + kq * 68u + li * 4u) = make_float4(d[0], d[1], d[2], d[3]);
         }
         __syncthreads();
-        for (uint32_t o = tid; o < kGroups * 16u * 16u; o += 512u) {
-            const uint32_t rl = o & 63u, j = o >> 6;                       // row of the tile, token of the pass
-            const uint32_t g = rl >> 4, i = rl & 15u;
+        constexpr uint32_t RT = KG * 16u;                                  // rows of a tile
+        for (uint32_t o = tid; o < RT * 16u * NT; o += 512u) {
+            const uint32_t rl = o % RT, jj = o / RT;                       // row of the tile, token of the pass
+            const uint32_t g = rl >> 4, i = rl & 15u, t = jj >> 4, j = jj & 15u;
             const uint32_t r = (tg0 + g) * 16u + i;
-            if (tg0 + g < g1 && r < rows && m0 + (int)j < M && (!HALF || j < 8u)) {
+            if (tg0 + g < g1 && r < rows && m0 + (int)jj < M && (!HALF || j < 8u)) {
                 float s = 0.f;
 #pragma unroll
                 for (uint32_t w8 = 0; w8 < 8; ++w8) {
-                    s += red[((size_t)w8 * kGroups + g) * kRedTile + (i >> 2) * 68u + j * 4u + (i & 3u)];
-                    if (HALF) s += red[((size_t)w8 * kGroups + g) * kRedTile + (i >> 2) * 68u + (j + 8u) * 4u + (i & 3u)];
+                    const float* cell = red + ((size_t)w8 * kGroups + g * NT + t) * kRedTile + (i >> 2) * 68u + (i & 3u);
+                    s += cell[j * 4u];
+                    if (HALF) s += cell[(j + 8u) * 4u];
                 }
-                if (ksplit > 1u) unsafeAtomicAdd(y + (size_t)(m0 + j) * ldy + r, s);
-                else y[(size_t)(m0 + j) * ldy + r] = s;
+                if (ksplit > 1u) unsafeAtomicAdd(y + (size_t)(m0 + jj) * ldy + r, s);
+                else y[(size_t)(m0 + jj) * ldy + r] = s;
             }
         }
         if (tile + 1 < ntiles) __syncthreads();                            // red is rewritten by the next tile
@@ -280,7 +309,7 @@ int get_pack_buffer(uint32_t** out) {
     OILHIP_HIP(hipGetDevice(&dev));
     if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
     std::lock_guard<std::mutex> lk(g_xp_mu);
-    if (!g_xp[dev]) OILHIP_HIP(hipMalloc(&g_xp[dev], (size_t)(kMaxPackCols >> 8) * 128u * 128u));
+    if (!g_xp[dev]) OILHIP_HIP(hipMalloc(&g_xp[dev], (size_t)(kMaxPackCols >> 8) * 128u * 128u * 2u));   // two token tiles
     *out = g_xp[dev];
     return OILHIP_OK;
 }
@@ -299,9 +328,11 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
                w2->uniform_stride != 128 || !d_y2)) return 1;
     static bool attr_done = false;
     if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false>),
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true>),
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
+        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
         attr_done = true;
     }
@@ -309,37 +340,36 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     if (int rc = get_pack_buffer(&xp)) return rc;
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
-    // rows wider than one K-pass (16 blocks): the row is cut into parts of at most 16 blocks that go to different
-    // workgroups, so that a workgroup fetches the split activations of its part once instead of once per pass and tile
-    // (the parts' sums meet through float atomics: with three or more parts the order of the additions, and with it the
-    // last bits of y, can differ between launches)
-    auto split_of = [&](const oilhip_weights&) -> uint32_t {
-        const uint32_t np = (bpr + 15u) / 16u;
+    // rows wider than one K-pass (16 blocks, 8 for passes of 32 tokens): the row is cut into parts of at most one pass
+    // that go to different workgroups, so that a workgroup fetches the split activations of its part once instead of
+    // once per pass and tile (the parts' sums meet through float atomics: with three or more parts the order of the
+    // additions, and with it the last bits of y, can differ between launches)
+    auto split_of = [&](uint32_t pass_blocks) -> uint32_t {
+        const uint32_t np = (bpr + pass_blocks - 1u) / pass_blocks;
         return np >= 2u && np <= (uint32_t)device_cu_count() ? np : 1u;
     };
-    auto main_launch = [&](const oilhip_weights& t, float* y, uint32_t ld, bool half, int m0, int m1) {
+    auto main_launch = [&](const oilhip_weights& t, float* y, uint32_t ld, int kind, int m0, int m1) {
         const uint32_t groups = ((uint32_t)t.rows + 15u) / 16u;
-        const uint32_t ks = split_of(t);
+        const uint32_t ks = split_of(kind == 2 ? 8u : 16u);
         uint32_t slabs = (uint32_t)device_cu_count() / ks;
         if (slabs > groups) slabs = groups;
-        if (half)
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<true>, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y,
-                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
-        else
-            hipLaunchKernelGGL(gemv_oil4_multi_kernel<false>, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y,
-                               (uint32_t)t.rows, (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
+        auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
+        hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y, (uint32_t)t.rows,
+                           (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
     };
-    for (int m0 = 0; m0 < M;) {                   // passes of 16 tokens; the last 8 or fewer as a pass of 8
-        const bool half = M - m0 <= 8;
-        const int m1 = half || M - m0 < 16 ? M : m0 + 16;
-        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u), dim3(256), 0, s, d_x, d_x2, d_tok, xp, (uint32_t)w.cols, m0, m1,
-                           ldx, xrows, half ? 1 : 0, split_of(w) > 1u ? d_y : nullptr, (uint32_t)w.rows, ldy,
-                           w2 && split_of(*w2) > 1u ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
+    for (int m0 = 0; m0 < M;) {       // passes of 32 tokens while more than 16 are left, then one of 16 or of 8
+        const int left = M - m0;
+        const int kind = left <= 8 ? 0 : left <= 16 ? 1 : 2;
+        const int m1 = left <= 32 ? M : m0 + 32;
+        const bool cut = split_of(kind == 2 ? 8u : 16u) > 1u;
+        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u * (kind == 2 ? 2u : 1u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp,
+                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, cut ? d_y : nullptr, (uint32_t)w.rows, ldy,
+                           w2 && cut ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
         OILHIP_HIP(hipGetLastError());
-        main_launch(w, d_y, ldy, half, m0, m1);
+        main_launch(w, d_y, ldy, kind, m0, m1);
         OILHIP_HIP(hipGetLastError());
         if (w2) {
-            main_launch(*w2, d_y2, ldy2, half, m0, m1);
+            main_launch(*w2, d_y2, ldy2, kind, m0, m1);
             OILHIP_HIP(hipGetLastError());
         }
         m0 = m1;

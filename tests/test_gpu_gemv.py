@@ -112,10 +112,10 @@ def test_oil4_fast_kernel_shapes(rows, cols, M):
     assert rel_l2(ref32, want) <= TOL
 
 
-# the multi-token kernel: passes of 16 tokens and of 8 or fewer (alone and as the last pass of a batch), several
+# the multi-token kernel: passes of 32 tokens (two token tiles), of 16 and of 8 or fewer (alone and as the last pass of a batch), several
 # row tiles per workgroup (rows > 48 * 256), several K-slabs, an odd number of blocks per row
 @pytest.mark.parametrize("rows,cols", [(130, 4096), (61, 11008), (13000, 512), (47, 14336), (3, 256)])
-@pytest.mark.parametrize("M", [3, 5, 8, 9, 13, 17, 40])
+@pytest.mark.parametrize("M", [3, 5, 8, 9, 13, 17, 32, 33, 40, 70])
 def test_oil4_multi_token_counts(rows, cols, M):
     err, *_ = run_case(ia.Format.OIL4, rows, cols, M, seed=7 * rows + cols + M)
     assert err <= TOL
