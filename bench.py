@@ -573,7 +573,7 @@ def main():
 
     if not args.no_extra:
         extra = {}
-        for M in (4, 16):
+        for M in (4, 16, 32):
             xm = torch.randn(M, COLS, device="cuda")
             ym = torch.empty((M, ROWS), dtype=torch.float32, device="cuda")
             s_m, _ = time_ring(torch, ring, xm, ym, 400, 40)
