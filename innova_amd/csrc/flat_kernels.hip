@@ -176,6 +176,104 @@ engine_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const
     if (live) C[m * N + n] = acc;
 }
 
+// engine_kernel<8> for N a multiple of 4: the same k-ordered chain per output, fed differently.  A wavefront per 64
+// outputs leaves most of the chip idle and a single wavefront issues one instruction at a time, so the time is the
+// instruction count per k step.  The four lanes of a quad own four neighbouring columns, whose codes of one k step
+// share a dword: lane q of the quad loads the dword of step 4i + q and the quad passes the dwords round with DPP
+// (8 loads per lane and 32 steps instead of 32 byte loads, three batches of 32 steps in flight); the look-up address
+// is one v_perm_b32 (entry v of lane l at byte v*256 + l*4 of a 64 KB table); the levels of batch b+1 are looked up
+// before the chain of batch b runs.  A batch without a zero in A (the usual case) is 32 bare FMAs; one with a zero
+// keeps the reference's skip as a select behind every FMA, so the result is the reference's bit for bit either way.
+__global__ void __launch_bounds__(64)
+engine8_quad_kernel(const float* __restrict__ A, const uint8_t* __restrict__ bq, const float* __restrict__ cb,
+                    float* __restrict__ C, long long M, long long N, long long K) {
+    __shared__ float c[256 * 64];
+    {
+        const float mine[4] = {cb[threadIdx.x], cb[64 + threadIdx.x], cb[128 + threadIdx.x], cb[192 + threadIdx.x]};
+#pragma unroll
+        for (int part = 0; part < 4; ++part)
+            for (int v = 0; v < 64; ++v)
+                c[(part * 64 + v) * 64 + threadIdx.x] = __shfl(mine[part], v);
+    }
+    __syncthreads();
+    const long long n = (long long)blockIdx.x * 64 + threadIdx.x;
+    const long long m = blockIdx.y;
+    const bool live = n < N;                               // N % 4 == 0: a quad is live or idle as a whole
+    const uint32_t sub = threadIdx.x & 3u, lane = threadIdx.x;
+    const unsigned long long n4 = (unsigned long long)(live ? n - sub : N - 4);
+    const float* a_row = A + m * K;
+    constexpr int UN = 32, NB = 4;
+    const long long nb = K / UN;                           // full batches
+    const uint32_t lanebase = lane * 4u, sel = 0x0C0C0000u | ((4u + sub) << 8);
+    uint32_t dw[NB][8];
+    float av[NB];                                          // lane j < 32: A[m][32 b + j], for the zero test
+    auto clampb = [&](long long b) { return b < nb ? b : nb - 1; };
+    // a lane's byte offset inside a k step's row pair: uniform 64-bit bases, 32-bit lane offsets (N < 2^29)
+    const uint32_t lane_off = sub * (uint32_t)N + (uint32_t)n4;
+    auto fetch = [&](int slot, long long b) {              // batch b, clamped to the last one: issued unconditionally
+        const unsigned long long k0 = (unsigned long long)clampb(b) * UN;
+        const uint8_t* ub = bq + k0 * (unsigned long long)N;                 // uniform
+#pragma unroll
+        for (int i = 0; i < 8; ++i) dw[slot][i] = *reinterpret_cast<const uint32_t*>(ub + 4ull * i * (unsigned long long)N + lane_off);
+        av[slot] = a_row[k0 + (lane & 31u)];
+    };
+    float lv[2][UN];
+    auto lookup = [&](int slot, int set) {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int v = (int)dw[slot][i];
+            const uint32_t qs[4] = {(uint32_t)__builtin_amdgcn_mov_dpp(v, 0x00, 0xF, 0xF, true),     // quad_perm [0,0,0,0]
+                                    (uint32_t)__builtin_amdgcn_mov_dpp(v, 0x55, 0xF, 0xF, true),     // [1,1,1,1]
+                                    (uint32_t)__builtin_amdgcn_mov_dpp(v, 0xAA, 0xF, 0xF, true),     // [2,2,2,2]
+                                    (uint32_t)__builtin_amdgcn_mov_dpp(v, 0xFF, 0xF, 0xF, true)};    // [3,3,3,3]
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t addr = __builtin_amdgcn_perm(qs[q], lanebase, sel);
+                lv[set][4 * i + q] = *reinterpret_cast<const float*>(reinterpret_cast<const uint8_t*>(c) + addr);
+            }
+        }
+    };
+    float acc = 0.0f;
+    auto chain = [&](const float (&a)[UN], int slot, int set) {
+        const bool any_zero = __ballot(av[slot] == 0.0f) != 0ull;         // uniform
+        if (!any_zero) {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) acc = __fmaf_rn(a[j], lv[set][j], acc);
+        } else {
+#pragma unroll
+            for (int j = 0; j < UN; ++j) {
+                const float t = __fmaf_rn(a[j], lv[set][j], acc);
+                acc = a[j] != 0.0f ? t : acc;              // the reference skips the term
+            }
+        }
+    };
+    if (nb > 0) {
+#pragma unroll
+        for (int u = 0; u < NB - 1; ++u) fetch(u, u);
+        lookup(0, 0);
+        for (long long b = 0; b < nb; b += NB) {
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                if (b + u < nb) {
+                    float a[UN];                           // A[m][32 (b+u) ..], uniform: requested before the look-ups
+#pragma unroll
+                    for (int j = 0; j < UN; ++j) a[j] = a_row[(b + u) * UN + j];
+                    fetch((u + NB - 1) % NB, b + u + NB - 1);
+                    lookup((u + 1) % NB, (u + 1) & 1);     // batch b+u+1 (past the end: the clamped copy, never folded in)
+                    chain(a, u, u & 1);
+                }
+            }
+        }
+    }
+    const unsigned long long nn = n4 + sub;
+    for (long long k = nb * UN; k < K; ++k) {
+        const float a = a_row[k];
+        if (a == 0.0f) continue;
+        acc = __fmaf_rn(a, c[(uint32_t)bq[(unsigned long long)k * (unsigned long long)N + nn] * 64u + lane], acc);
+    }
+    if (live) C[m * N + n] = acc;
+}
+
 // The engines whose B operand is not a codebook index: kind 1 = Oil1Engine (one float per 32 flat positions,
 // src/oil_engines_oil1.cpp:61-82), 3 = SparkEngine (2-bit codes: 2 -> +s, 0 -> -s, else 0, with s = a * scale of
 // the flat position's block, src/oil_engines_spark.cpp:154-186), 16 = OIL16Engine (FP16 widened as
@@ -375,7 +473,9 @@ int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b, con
     if (M > 65535) return fail(OILHIP_E_ARG, "M exceeds the grid limit");
     const dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)M);
     hipStream_t s = (hipStream_t)stream;
-    if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    if (bits == 8 && (N & 3) == 0 && N < (1ll << 29) && (reinterpret_cast<uintptr_t>(d_b) & 3u) == 0)
+        hipLaunchKernelGGL(engine8_quad_kernel, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
+    else if (bits == 8) hipLaunchKernelGGL(engine_kernel<8>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     else if (bits == 4) hipLaunchKernelGGL(engine_kernel<4>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     else hipLaunchKernelGGL(engine_kernel<2>, grid, dim3(64), 0, s, d_a, d_b, d_cb, d_c, M, N, K);
     OILHIP_HIP(hipGetLastError());
