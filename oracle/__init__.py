@@ -372,3 +372,88 @@ def swiglu(g, u) -> np.ndarray:
     h = np.zeros_like(g)
     lib().orc_swiglu(C.c_void_p(g.ctypes.data), C.c_void_p(u.ctypes.data), C.c_int64(g.size), C.c_void_p(h.ctypes.data))
     return h
+
+
+# ---------------------------------------------------------------- OIL4 KV cache (src/kv_cache_oil4.cpp)
+def _vp(a):
+    return C.c_void_p(a.ctypes.data)
+
+
+def kv_half_to_float(h: np.ndarray) -> np.ndarray:
+    """CodebookOIL4::half_to_float over an array of uint16 (src/codebook.cpp:36-64)."""
+    L = lib()
+    L.orc_kv_half_to_float.restype = C.c_float
+    L.orc_kv_half_to_float.argtypes = [C.c_uint16]
+    return np.array([L.orc_kv_half_to_float(int(x)) for x in np.asarray(h).ravel()], np.float32).reshape(np.shape(h))
+
+
+def kv_float_to_half(f: np.ndarray) -> np.ndarray:
+    """CodebookOIL4::float_to_half over an array of float32 (src/codebook.cpp:16-34)."""
+    L = lib()
+    L.orc_kv_float_to_half.restype = C.c_uint16
+    L.orc_kv_float_to_half.argtypes = [C.c_float]
+    return np.array([L.orc_kv_float_to_half(float(x)) for x in np.asarray(f, np.float32).ravel()],
+                    np.uint16).reshape(np.shape(f))
+
+
+def kv_quantize_block(src: np.ndarray, fn=None):
+    """OIL4KVCache::quantize_block_oil4 (src/kv_cache_oil4.cpp:75-163): (codebook uint16[16], codes uint8[n])."""
+    src = np.ascontiguousarray(src, np.float32)
+    cb = np.zeros(16, np.uint16)
+    codes = np.zeros(max(src.size, 1), np.uint8)
+    (fn or lib().orc_kv_quantize_block)(_vp(src), C.c_int64(src.size), _vp(cb), _vp(codes))
+    return cb, codes[:src.size]
+
+
+class KVCache:
+    """OIL4KVCache (include/oil/kv_cache_oil4.h:26-83) for one layer, state in numpy arrays."""
+
+    def __init__(self, max_seq_len, num_heads, head_dim, block_size=64):
+        self.max_seq, self.per_token = int(max_seq_len), int(num_heads * head_dim)
+        self.block = block_size if block_size in (32, 64, 128) else 64
+        total = self.max_seq * self.per_token
+        self.idx_bytes = (total + 1) // 2
+        nblocks = (total + self.block - 1) // self.block
+        self.k_idx = np.zeros(self.idx_bytes, np.uint8)
+        self.v_idx = np.zeros(self.idx_bytes, np.uint8)
+        self.k_cb = np.zeros(nblocks * 16, np.uint16)
+        self.v_cb = np.zeros(nblocks * 16, np.uint16)
+        self.pos = 0
+
+    def append(self, k, v):
+        k = np.ascontiguousarray(k, np.float32).reshape(-1, self.per_token)
+        v = np.ascontiguousarray(v, np.float32).reshape(-1, self.per_token)
+        lib().orc_kv_append(_vp(self.k_idx), _vp(self.v_idx), _vp(self.k_cb), _vp(self.v_cb), C.c_int64(self.idx_bytes),
+                            C.c_int64(self.max_seq), C.c_int64(self.per_token), C.c_int64(self.block),
+                            C.c_int64(self.pos), _vp(k), _vp(v), C.c_int64(k.shape[0]))
+        self.pos += k.shape[0]
+
+    def get_range(self, start, end):
+        n = min(end, self.pos) - start
+        if end - start <= 0 or n <= 0:
+            return np.zeros((0, self.per_token), np.float32), np.zeros((0, self.per_token), np.float32)
+        out = []
+        for idx, cb in ((self.k_idx, self.k_cb), (self.v_idx, self.v_cb)):
+            o = np.zeros((n, self.per_token), np.float32)
+            lib().orc_kv_get_range(_vp(idx), _vp(cb), C.c_int64(self.idx_bytes), C.c_int64(self.per_token),
+                                   C.c_int64(self.block), C.c_int64(start), C.c_int64(n), _vp(o))
+            out.append(o)
+        return out[0], out[1]
+
+
+def ref_kv_run(max_seq, heads, dim, block, k, v, seq_lens, start, end):
+    """The compiled reference's OIL4KVCache: the appends, then get_range -> (k, v, size_bytes, context_len)."""
+    R = ref(True)
+    k = np.ascontiguousarray(k, np.float32)
+    v = np.ascontiguousarray(v, np.float32)
+    pt = heads * dim
+    tot = int(sum(seq_lens))
+    ko = np.zeros((max(tot, 1), pt), np.float32)
+    vo = np.zeros_like(ko)
+    sl = np.array(seq_lens, np.int64)
+    sb, cl = C.c_uint64(), C.c_int()
+    R.ref_kv_run.restype = C.c_int64
+    n = R.ref_kv_run(C.c_int(1), C.c_int64(max_seq), C.c_int64(heads), C.c_int64(dim), C.c_int64(block), C.c_int(0),
+                     _vp(k), _vp(v), _vp(sl), C.c_int(len(seq_lens)), C.c_int64(start), C.c_int64(end), _vp(ko), _vp(vo),
+                     C.byref(sb), C.byref(cl))
+    return ko[:n].copy(), vo[:n].copy(), sb.value, cl.value

@@ -1101,3 +1101,146 @@ void orc_swiglu(const float* g, const float* u, int64_t n, float* h) {
         h[i] = (v * (1.0f / (1.0f + expf(-v)))) * u[i];
     }
 }
+
+/* ---- OIL4 KV cache (src/kv_cache_oil4.cpp, src/codebook.cpp:16-64) ------------------------------------------ */
+uint16_t orc_kv_float_to_half(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const int32_t e = (int32_t)((u >> 23) & 0xFFu) - 127 + 15;
+    uint32_t mant = u & 0x007FFFFFu;
+    if (e <= 0) {
+        if (e < -10) return sign;
+        mant = (mant | 0x00800000u) >> (1 - e);
+        return (uint16_t)(sign | (uint16_t)(mant >> 13));
+    }
+    if (e >= 31) return (uint16_t)(sign | 0x7C00u | (mant != 0 ? 0x0200u : 0u));
+    return (uint16_t)(sign | ((uint16_t)e << 10) | (uint16_t)(mant >> 13));
+}
+
+float orc_kv_half_to_float(uint16_t h) {
+    const uint32_t sign = h & 0x8000u;
+    int32_t e = (h >> 10) & 0x1F;
+    uint16_t mant = h & 0x03FFu;
+    uint32_t f;
+    if (e == 0) {
+        if (mant == 0) {
+            f = sign << 16;
+        } else {
+            int shift = 10;
+            while ((mant & 0x0400u) == 0) { mant = (uint16_t)(mant << 1); shift--; }
+            e = 1 - shift + 127 - 15;
+            /* the reference keeps the shifted mantissa in a uint16_t: only bits 13-15 survive (codebook.cpp:52) */
+            f = (sign << 16) | ((uint32_t)e << 23) | (((uint32_t)(mant & 0x03FFu) << 13) & 0xFFFFu);
+        }
+    } else if (e == 31) {
+        f = (sign << 16) | 0x7F800000u | ((uint32_t)mant << 13);
+    } else {
+        f = (sign << 16) | ((uint32_t)(e - 15 + 127) << 23) | ((uint32_t)mant << 13);
+    }
+    float r;
+    memcpy(&r, &f, 4);
+    return r;
+}
+
+static int kv_cmp_float(const void* a, const void* b) {
+    const float x = *(const float*)a, y = *(const float*)b;
+    return x < y ? -1 : (x > y ? 1 : 0);
+}
+
+static int kv_nearest(const float* cen, float x) {
+    float best = fabsf(x - cen[0]);
+    int bi = 0;
+    for (int c = 1; c < 16; ++c) {
+        const float d = fabsf(x - cen[c]);
+        if (d < best) { best = d; bi = c; }
+    }
+    return bi;
+}
+
+void orc_kv_quantize_block(const float* src, int64_t n, uint16_t* cb16, uint8_t* codes) {
+    if (n == 0) return;
+    float lo = src[0], hi = src[0];
+    for (int64_t i = 1; i < n; ++i) {
+        if (src[i] < lo) lo = src[i];
+        if (src[i] > hi) hi = src[i];
+    }
+    if (hi - lo < 1e-10f) {
+        for (int64_t i = 0; i < n; ++i) codes[i] = 8;
+        for (int c = 0; c < 16; ++c) cb16[c] = orc_kv_float_to_half(lo);
+        return;
+    }
+    float cen[16];
+    for (int c = 0; c < 16; ++c) cen[c] = lo + (hi - lo) * ((float)c + 0.5f) / 16.0f;
+    float sorted[4096];
+    const int64_t m = n > 4096 ? 4096 : n;
+    memcpy(sorted, src, (size_t)m * 4);
+    qsort(sorted, (size_t)m, 4, kv_cmp_float);          /* values only: any correct sort gives the same array up to -0/+0 and NaN order */
+    for (int it = 0; it < 20; ++it) {
+        float sums[16] = {0};
+        int counts[16] = {0};
+        for (int64_t i = 0; i < m; ++i) {
+            const int b = kv_nearest(cen, sorted[i]);
+            sums[b] += sorted[i];
+            counts[b]++;
+        }
+        for (int c = 0; c < 16; ++c)
+            if (counts[c] > 0) cen[c] = sums[c] / (float)counts[c];
+    }
+    for (int64_t i = 0; i < n; ++i) codes[i] = (uint8_t)kv_nearest(cen, src[i]);
+    for (int c = 0; c < 16; ++c) cb16[c] = orc_kv_float_to_half(cen[c]);
+}
+
+static int64_t kv_block(int64_t block) { return block == 32 || block == 64 || block == 128 ? block : 64; }
+
+void orc_kv_append(uint8_t* k_idx, uint8_t* v_idx, uint16_t* k_cb, uint16_t* v_cb, int64_t idx_bytes,
+                   int64_t max_seq, int64_t per_token, int64_t block, int64_t pos,
+                   const float* k, const float* v, int64_t seq_len) {
+    block = kv_block(block);
+    const int64_t ibpb = (block + 1) / 2;
+    uint8_t codes[128], packed[64];
+    uint16_t cb[16];
+    for (int64_t s = 0; s < seq_len && pos + s < max_seq; ++s) {
+        int64_t left = per_token, src = s * per_token, flat = (pos + s) * per_token;
+        while (left > 0) {
+            const int64_t blk = flat / block, off = flat % block;
+            const int64_t chunk = left < block - off ? left : block - off;
+            const int64_t at = blk * ibpb + off / 2;
+            for (int pass = 0; pass < 2; ++pass) {
+                orc_kv_quantize_block((pass ? v : k) + src, chunk, cb, codes);
+                const int64_t nbytes = (chunk + 1) / 2;
+                for (int64_t i = 0; i < nbytes; ++i) {
+                    const uint8_t lo4 = codes[2 * i] & 0x0F;
+                    const uint8_t hi4 = (2 * i + 1) < chunk ? (codes[2 * i + 1] & 0x0F) : 0;
+                    packed[i] = (uint8_t)(lo4 | (hi4 << 4));
+                }
+                int64_t put = nbytes;
+                if (at + put > idx_bytes) put = idx_bytes - at;
+                if (put > 0) memcpy((pass ? v_idx : k_idx) + at, packed, (size_t)put);
+                if (pass || off == 0 || pos == 0) memcpy((pass ? v_cb : k_cb) + blk * 16, cb, 32);
+            }
+            left -= chunk; src += chunk; flat += chunk;
+        }
+    }
+}
+
+void orc_kv_get_range(const uint8_t* idx, const uint16_t* cb, int64_t idx_bytes, int64_t per_token, int64_t block,
+                      int64_t start, int64_t len, float* out) {
+    block = kv_block(block);
+    const int64_t ibpb = (block + 1) / 2;
+    for (int64_t s = 0; s < len; ++s) {
+        int64_t left = per_token, flat = (start + s) * per_token, dst = s * per_token;
+        while (left > 0) {
+            const int64_t blk = flat / block, off = flat % block;
+            const int64_t chunk = left < block - off ? left : block - off;
+            const int64_t at = blk * ibpb + off / 2;
+            for (int64_t i = 0; i < chunk; ++i) {
+                const int64_t b = at + i / 2;
+                const uint8_t byte = b < idx_bytes ? idx[b] : 0;
+                const uint8_t code = (i & 1) ? (uint8_t)(byte >> 4) : (uint8_t)(byte & 0x0F);
+                out[dst + i] = orc_kv_half_to_float(cb[blk * 16 + code]);
+            }
+            left -= chunk; flat += chunk; dst += chunk;
+        }
+    }
+}

@@ -169,6 +169,30 @@ void orc_moe_dispatch(const float* x, const float* const* gate, const float* con
                       int64_t T, int64_t K, int64_t E, int64_t D, int64_t F,
                       float* out, float* z_loss, int64_t* dropped, int as_double);
 
+/* OIL4 KV cache (src/kv_cache_oil4.cpp): flat element e = token * per_token + i of a layer lives in block
+ * e / block (block in {32, 64, 128}, anything else means 64, :25-26), 16 FP16 centroids per block, 4-bit codes two
+ * per byte, low nibble first.
+ * orc_kv_half_to_float / orc_kv_float_to_half: CodebookOIL4::half_to_float / float_to_half (src/codebook.cpp:16-64)
+ *   bit for bit: the encoder truncates the mantissa and flushes below 2^-25, the decoder's subnormal branch yields
+ *   exponent 113 - shift after normalising and keeps only the low 16 bits of the shifted mantissa (not the IEEE value; the
+ *   cache reads its centroids through it).
+ * orc_kv_quantize_block: lloyd_max_16 (:75-153): constant block -> codes 8, centroids min; else 16 uniform
+ *   centroids, 20 Lloyd iterations over the first 4096 values sorted ascending, nearest centroid by |x - c| with the
+ *   first minimum kept, centroids stored truncated to FP16.  codes: one per byte.
+ * orc_kv_append (:207-291): per token the per_token values are cut at block boundaries; each chunk is quantized on
+ *   its own, its codes packed from the chunk's first byte (block * block/2 + offset/2), K centroids written only for
+ *   chunks that start a block (or while the cache is empty), V centroids always.  pos is the number of tokens held.
+ * orc_kv_get_range (:293-362): tokens [start, start+len) -> FP32 [len][per_token], chunk by chunk with the same
+ *   byte rule; bytes past the index array read as 0. */
+float orc_kv_half_to_float(uint16_t h);
+uint16_t orc_kv_float_to_half(float f);
+void orc_kv_quantize_block(const float* src, int64_t n, uint16_t* cb16, uint8_t* codes);
+void orc_kv_append(uint8_t* k_idx, uint8_t* v_idx, uint16_t* k_cb, uint16_t* v_cb, int64_t idx_bytes,
+                   int64_t max_seq, int64_t per_token, int64_t block, int64_t pos,
+                   const float* k, const float* v, int64_t seq_len);
+void orc_kv_get_range(const uint8_t* idx, const uint16_t* cb, int64_t idx_bytes, int64_t per_token, int64_t block,
+                      int64_t start, int64_t len, float* out);
+
 #ifdef __cplusplus
 }
 #endif

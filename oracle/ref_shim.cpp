@@ -12,6 +12,8 @@
 #include "oil/kernel.h"
 #include "oil/kernel_production.h"
 #include "oil/oil_engines.h"
+#include "oil/kv_cache_oil4.h"
+#include "oil/codebook.h"
 #include "oil/types.h"
 
 #include <cstdint>
@@ -274,6 +276,45 @@ void ref_engine_dequant(int bits, const uint8_t* idx, int64_t n, const float* sc
     } else {
         oil::engines::OIL4Engine e; e.dequantize_per_block(idx, scales, n, block, out);
     }
+}
+
+// CodebookOIL4::half_to_float / float_to_half (include/oil/codebook.h:79-80)
+float ref_kv_half_to_float(uint16_t h) { return oil::CodebookOIL4::half_to_float(h); }
+uint16_t ref_kv_float_to_half(float f) { return oil::CodebookOIL4::float_to_half(f); }
+
+// OIL4KVCache::quantize_block_oil4 / dequantize_block_oil4 (include/oil/kv_cache_oil4.h:52-57): one code per byte
+void ref_kv_quantize_block(const float* src, int64_t n, uint16_t* cb16, uint8_t* codes) {
+    oil::OIL4KVCache::quantize_block_oil4(src, codes, cb16, n);
+}
+void ref_kv_dequantize_block(const uint8_t* codes, const uint16_t* cb16, float* dst, int64_t n) {
+    oil::OIL4KVCache::dequantize_block_oil4(codes, cb16, dst, n);
+}
+
+// One OIL4KVCache: n_appends calls of append(layer, k, v) with seq_lens[i] tokens each (k and v hold the tokens of
+// all calls back to back, [token][heads * dim]), then get_range(layer, start, end).  Returns the number of tokens
+// get_range gave back; size_bytes / context_len as the cache reports them.
+int64_t ref_kv_run(int layers, int64_t max_seq, int64_t heads, int64_t dim, int64_t block, int layer,
+                   const float* k, const float* v, const int64_t* seq_lens, int n_appends,
+                   int64_t start, int64_t end, float* k_out, float* v_out, uint64_t* size_bytes, int* context_len) {
+    oil::OIL4KVCache cache(layers, max_seq, heads, dim, block);
+    const int64_t per_token = heads * dim;
+    int64_t at = 0;
+    for (int a = 0; a < n_appends; ++a) {
+        const int64_t s = seq_lens[a];
+        oil::Tensor kt(oil::Shape{1, heads, s, dim}), vt(oil::Shape{1, heads, s, dim});
+        std::memcpy(kt.data<float>(), k + at * per_token, (size_t)(s * per_token) * 4);
+        std::memcpy(vt.data<float>(), v + at * per_token, (size_t)(s * per_token) * 4);
+        cache.append(layer, kt, vt);
+        at += s;
+    }
+    if (size_bytes) *size_bytes = cache.size_bytes();
+    if (context_len) *context_len = cache.context_len();
+    auto kv = cache.get_range(layer, start, end);
+    if (kv.first.numel() == 0) return 0;
+    const int64_t len = kv.first.shape().dims[2];
+    std::memcpy(k_out, kv.first.data<float>(), (size_t)(len * per_token) * 4);
+    std::memcpy(v_out, kv.second.data<float>(), (size_t)(len * per_token) * 4);
+    return len;
 }
 
 }  // extern "C"

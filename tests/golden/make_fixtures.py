@@ -482,8 +482,75 @@ def make_engines():
     print("engines.npz written")
 
 
+
+KV_CASES = [  # max_seq, heads, dim, block, appends (tokens per call); even and odd tokens, tokens shorter than a block
+    (64, 2, 32, 64, [5, 1, 1, 3]), (24, 8, 128, 64, [7, 1, 1]), (32, 1, 48, 64, [3, 2, 1, 1]), (32, 1, 16, 32, [1, 1, 1, 4]),
+    (40, 3, 11, 64, [4, 1, 2]), (16, 2, 64, 128, [16]), (16, 1, 24, 77, [2, 2, 2]), (20, 5, 7, 32, [3, 1, 1, 1, 5]),
+    (8, 1, 64, 64, [1] * 8), (8, 2, 64, 32, [4, 4])]
+KV_BLOCK_SIZES = [1, 2, 3, 7, 16, 31, 32, 33, 64, 100, 127, 128, 200, 5000]
+
+
+def kv_inputs(i):
+    ms, h, d, block, lens = KV_CASES[i]
+    rng = np.random.default_rng(900 + i)
+    tot = sum(lens)
+    k = rng.standard_normal((tot, h * d)).astype(np.float32)
+    v = (rng.standard_normal((tot, h * d)) * 3).astype(np.float32)
+    if i % 3 == 1:
+        k[:, : h * d // 2] = 0.25          # constant chunks
+    return k, v
+
+
+def kv_block_inputs(j):
+    n = KV_BLOCK_SIZES[j % len(KV_BLOCK_SIZES)]
+    rng = np.random.default_rng(950 + j)
+    x = rng.standard_normal(n).astype(np.float32)
+    kind = j % 6
+    if kind == 1: x *= 1e-6
+    if kind == 2: x = (np.round(x * 2) / 2).astype(np.float32)
+    if kind == 3: x[:] = x[0]
+    if kind == 4: x *= 1e4
+    if kind == 5: x = (x * 1e-3).astype(np.float32); x[::3] = 0
+    return x
+
+
+def make_kv():
+    R = O.ref(True)
+    assert R is not None, "build oracle/_ref first (make -C oracle ref)"
+    R.ref_kv_half_to_float.restype = C.c_float
+    R.ref_kv_half_to_float.argtypes = [C.c_uint16]
+    R.ref_kv_float_to_half.restype = C.c_uint16
+    R.ref_kv_float_to_half.argtypes = [C.c_float]
+    out = {"h2f": np.array([R.ref_kv_half_to_float(h) for h in range(65536)], np.float32).view(np.uint32)}
+    fbits = kv_f2h_inputs()
+    out["f2h"] = np.array([R.ref_kv_float_to_half(float(f)) for f in fbits.view(np.float32)], np.uint16)
+    for j in range(84):
+        cb, codes = O.kv_quantize_block(kv_block_inputs(j), fn=R.ref_kv_quantize_block)
+        out[f"qcb{j}"], out[f"qcodes{j}"] = cb, codes
+    for i, (ms, h, d, block, lens) in enumerate(KV_CASES):
+        k, v = kv_inputs(i)
+        tot = sum(lens)
+        for r, (st, en) in enumerate([(0, tot), (1, tot - 1), (0, tot + 5)]):
+            ko, vo, sb, cl = O.ref_kv_run(ms, h, d, block, k, v, lens, st, en)
+            out[f"k{i}_{r}"], out[f"v{i}_{r}"] = ko.view(np.uint32), vo.view(np.uint32)
+            out[f"meta{i}_{r}"] = np.array([sb, cl], np.int64)
+    np.savez_compressed(os.path.join(HERE, "kv.npz"), **out)
+    print("kv.npz written")
+
+
+def kv_f2h_inputs():
+    rng = np.random.default_rng(970)
+    bits = np.concatenate([rng.integers(0, 2 ** 32, 20000, dtype=np.uint64).astype(np.uint32),
+                           np.arange(0x33000000, 0x33000000 + 1000, dtype=np.uint32),
+                           np.arange(0x38000000, 0x38000000 + 20000, 7, dtype=np.uint32),
+                           np.array([0, 0x80000000, 0x7f800000, 0xff800000, 0x477fe000, 0x477ff000, 0x47800000, 0x38800000,
+                                     0x387fffff, 0x33800000, 0x337fffff], dtype=np.uint32)])
+    f = bits.view(np.float32)
+    return bits[~np.isnan(f)]
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe", "engines"]
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe", "engines", "kv"]
     for name in which:
         {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner,
-         "container": make_container, "moe": make_moe, "engines": make_engines}[name]()
+         "container": make_container, "moe": make_moe, "engines": make_engines, "kv": make_kv}[name]()
