@@ -270,6 +270,43 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                        const float* weights, int64_t T, int64_t K, float* d_out, void* d_workspace,
                        size_t workspace_bytes, float* z_loss, int64_t* dropped, void* stream);
 
+/* ------------------------------------------------------------ OIL4 KV cache
+ * The device-resident oil::OIL4KVCache (include/oil/kv_cache_oil4.h:26-83, src/kv_cache_oil4.cpp): per layer the K and
+ * V streams [token][heads * dim] as 4-bit codes (two per byte, low nibble first) with 16 FP16 centroids per block of
+ * 32 / 64 / 128 consecutive values (any other block_size means 64, :25-26).  heads * dim must be even.  Codes and
+ * centroids are the reference's bit for bit (inputs must be finite).
+ * oilhip_kv_create            : OIL4KVCache(num_layers, max_seq_len, num_heads, head_dim, block_size) / init (:13-43)
+ * oilhip_kv_append            : append(layer, k, v) (:207-291); d_k, d_v: [seq_len][heads * dim] FP32 on the device.
+ *                               Tokens beyond max_seq_len are dropped but still counted, layer >= num_layers is ignored,
+ *                               as in the reference.  Chunks are quantized by the 16-level Lloyd-Max of :75-153.
+ * oilhip_kv_get_range         : get_range(layer, start, end) (:293-362) -> d_k, d_v [len][heads * dim] FP32, *len = tokens
+ *                               written (end is clipped to the tokens held; 0 where the reference returns empty tensors).
+ *                               get_all is get_range(layer, 0, context).  Tokens that were dropped are never returned
+ *                               (the reference reads past its arrays there).
+ * oilhip_kv_info              : context_len() (layer 0), block_size(), size_bytes(), size_bytes_fp32_equivalent() (:364-392)
+ * oilhip_kv_clear / _resize   : clear() (:394-402), resize(new_max_seq_len) (:404-416, every layer empty afterwards;
+ *                               synchronises the device and reallocates)
+ * oilhip_kv_state             : host copies of a layer's code and centroid arrays ((max_seq*heads*dim+1)/2 bytes and
+ *                               16 uint16 per block each) for checks and checkpoints; any pointer may be NULL
+ * oilhip_kv_quantize_blocks   : OIL4KVCache::quantize_block_oil4 (:165-168) over nblocks runs of n <= 128 values:
+ *                               d_codes one code per byte [nblocks][n], d_cb16 [nblocks][16]
+ * oilhip_kv_dequantize_blocks : OIL4KVCache::dequantize_block_oil4 (:170-174), any n, through
+ *                               CodebookOIL4::half_to_float (src/codebook.cpp:36-64) */
+typedef struct oilhip_kv oilhip_kv;
+int oilhip_kv_create(int num_layers, int64_t max_seq_len, int64_t num_heads, int64_t head_dim, int64_t block_size,
+                     oilhip_kv** out);
+int oilhip_kv_destroy(oilhip_kv* c);
+int oilhip_kv_append(oilhip_kv* c, int layer, const float* d_k, const float* d_v, int64_t seq_len, void* stream);
+int oilhip_kv_get_range(const oilhip_kv* c, int layer, int64_t start, int64_t end, float* d_k, float* d_v, int64_t* len_out,
+                        void* stream);
+int oilhip_kv_info(const oilhip_kv* c, int* context_len, int64_t* block_size, uint64_t* size_bytes, uint64_t* fp32_bytes);
+int oilhip_kv_clear(oilhip_kv* c, void* stream);
+int oilhip_kv_resize(oilhip_kv* c, int64_t new_max_seq_len);
+int oilhip_kv_state(const oilhip_kv* c, int layer, uint8_t* k_idx, uint8_t* v_idx, uint16_t* k_cb, uint16_t* v_cb);
+int oilhip_kv_quantize_blocks(const float* d_src, int64_t n, int64_t nblocks, uint8_t* d_codes, uint16_t* d_cb16, void* stream);
+int oilhip_kv_dequantize_blocks(const uint8_t* d_codes, const uint16_t* d_cb16, float* d_dst, int64_t n, int64_t nblocks,
+                                void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -79,6 +79,16 @@ _SIGNATURES = {
     "oilhip_prod_gemv_oil4": (C.c_int, [vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_prod_gemv_oil8": (C.c_int, [vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_engine_quant_gemm": (C.c_int, [C.c_int, vp, vp, vp, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
+    "oilhip_kv_create": (C.c_int, [C.c_int, C.c_int64, C.c_int64, C.c_int64, C.c_int64, C.POINTER(vp)]),
+    "oilhip_kv_destroy": (C.c_int, [vp]),
+    "oilhip_kv_append": (C.c_int, [vp, C.c_int, vp, vp, C.c_int64, vp]),
+    "oilhip_kv_get_range": (C.c_int, [vp, C.c_int, C.c_int64, C.c_int64, vp, vp, C.POINTER(C.c_int64), vp]),
+    "oilhip_kv_info": (C.c_int, [vp, C.POINTER(C.c_int), C.POINTER(C.c_int64), C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]),
+    "oilhip_kv_clear": (C.c_int, [vp, vp]),
+    "oilhip_kv_resize": (C.c_int, [vp, C.c_int64]),
+    "oilhip_kv_state": (C.c_int, [vp, C.c_int, vp, vp, vp, vp]),
+    "oilhip_kv_quantize_blocks": (C.c_int, [vp, C.c_int64, C.c_int64, vp, vp, vp]),
+    "oilhip_kv_dequantize_blocks": (C.c_int, [vp, vp, vp, C.c_int64, C.c_int64, vp]),
 }
 
 

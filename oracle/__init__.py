@@ -380,11 +380,18 @@ def _vp(a):
 
 
 def kv_half_to_float(h: np.ndarray) -> np.ndarray:
-    """CodebookOIL4::half_to_float over an array of uint16 (src/codebook.cpp:36-64)."""
-    L = lib()
-    L.orc_kv_half_to_float.restype = C.c_float
-    L.orc_kv_half_to_float.argtypes = [C.c_uint16]
-    return np.array([L.orc_kv_half_to_float(int(x)) for x in np.asarray(h).ravel()], np.float32).reshape(np.shape(h))
+    """CodebookOIL4::half_to_float over an array of uint16 (src/codebook.cpp:36-64).  Runs through orc_kv_get_range so
+    that the floats come back through memory (a ctypes float return would quiet signalling NaNs)."""
+    hh = np.asarray(h, np.uint16).ravel()
+    nb = (hh.size + 15) // 16
+    cb = np.zeros(nb * 16, np.uint16)
+    cb[:hh.size] = hh
+    idx = np.tile(np.array([0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE] * 2, np.uint8), nb)   # codes 0..15 twice per block of 32
+    out = np.zeros((nb, 32), np.float32)
+    if nb:
+        lib().orc_kv_get_range(_vp(idx), _vp(cb), C.c_int64(idx.size), C.c_int64(32), C.c_int64(32), C.c_int64(0),
+                               C.c_int64(nb), _vp(out))
+    return out[:, :16].ravel()[:hh.size].reshape(np.shape(h)).copy()
 
 
 def kv_float_to_half(f: np.ndarray) -> np.ndarray:

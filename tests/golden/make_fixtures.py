@@ -517,11 +517,15 @@ def kv_block_inputs(j):
 def make_kv():
     R = O.ref(True)
     assert R is not None, "build oracle/_ref first (make -C oracle ref)"
-    R.ref_kv_half_to_float.restype = C.c_float
-    R.ref_kv_half_to_float.argtypes = [C.c_uint16]
     R.ref_kv_float_to_half.restype = C.c_uint16
     R.ref_kv_float_to_half.argtypes = [C.c_float]
-    out = {"h2f": np.array([R.ref_kv_half_to_float(h) for h in range(65536)], np.float32).view(np.uint32)}
+    # through dequantize_block_oil4 so that the floats come back through memory, signalling NaNs intact
+    h2f = np.zeros((4096, 16), np.float32)
+    codes = np.arange(16, dtype=np.uint8)
+    for b in range(4096):
+        cb = np.arange(b * 16, b * 16 + 16, dtype=np.uint16)
+        R.ref_kv_dequantize_block(C.c_void_p(codes.ctypes.data), C.c_void_p(cb.ctypes.data), C.c_void_p(h2f[b].ctypes.data), C.c_int64(16))
+    out = {"h2f": h2f.ravel().view(np.uint32)}
     fbits = kv_f2h_inputs()
     out["f2h"] = np.array([R.ref_kv_float_to_half(float(f)) for f in fbits.view(np.float32)], np.uint16)
     for j in range(84):
