@@ -467,6 +467,59 @@ def bench_dequant_and_engine(torch, ia, payload, blocks):
     return out
 
 
+def bench_kv_cache(torch, ia):
+    """The OIL4 KV cache of one Llama-7B-shaped layer (32 heads x 128, block 64): get_range over a 4096-token context
+    (per value 0.5 B of codes + 0.5 B of centroids read, 4 B of FP32 written, K and V in one launch), a 2048-token
+    prefill append and a one-token decode append (Lloyd-Max on the device, one wavefront per 64-value chunk)."""
+    heads, dim, ctx = 32, 128, 4096
+    pt = heads * dim
+    c = ia.OIL4KVCache(1, ctx + 64, heads, dim, 64)
+    k = torch.randn((1, heads, 2048, dim), device="cuda")
+    v = torch.randn((1, heads, 2048, dim), device="cuda")
+    k1, v1 = k.reshape(-1)[:pt].reshape(1, heads, 1, dim).contiguous(), v.reshape(-1)[:pt].reshape(1, heads, 1, dim).contiguous()
+
+    def timed(fn, reps, before=None):
+        tot = 0.0
+        for r in range(reps + 1):
+            if before:
+                before()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn()
+            e1.record()
+            torch.cuda.synchronize()
+            if r:
+                tot += e0.elapsed_time(e1) * 1e-3
+        return tot / reps
+
+    out = {}
+    t = timed(lambda: c.append(0, k, v), 5, before=c.clear)
+    out["kv_append_prefill_2048tok_us"] = round(t * 1e6, 1)
+    out["kv_append_prefill_Mtok_per_s"] = round(2048 / t / 1e6, 3)
+    c.clear()
+    c.append(0, k, v)
+    c.append(0, k, v)
+    t = timed(lambda: c.append(0, k1, v1), 20)
+    out["kv_append_decode_1tok_us"] = round(t * 1e6, 1)
+    L = ia._lib.lib()
+    import ctypes as C
+    outs = [(torch.empty((ctx, pt), dtype=torch.float32, device="cuda"), torch.empty((ctx, pt), dtype=torch.float32, device="cuda"))
+            for _ in range(4)]                         # 4 x 134 MB of outputs in turn: more than the 256 MB Infinity Cache
+    got = C.c_int64()
+
+    def ring():
+        for r in range(12):
+            ko, vo = outs[r % 4]
+            ia._lib.check(L.oilhip_kv_get_range(c._h, 0, 0, ctx, ko.data_ptr(), vo.data_ptr(), C.byref(got), ia._lib.current_stream()))
+
+    t = timed(ring, 3) / 12
+    assert got.value == ctx
+    nbytes = 2 * ctx * pt * (0.5 + 32 / 64 + 4)
+    out["kv_get_range_4096tok_us"] = round(t * 1e6, 1)
+    out["kv_get_range_4096tok_GBps"] = round(nbytes / t / 1e9, 1)
+    return out
+
+
 def bench_moe(torch, ia):
     """MoE step: 8 OIL4 experts (gate/up 14336x4096, down 4096x14336: 704.6 MB of payload), 64 tokens, top-2.
     One expert is quantized on the host and uploaded 8 times (distinct device copies, same bytes)."""
@@ -612,6 +665,7 @@ def main():
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))
         extra.update(bench_moe(torch, ia))
+        extra.update(bench_kv_cache(torch, ia))
         # the secondary legs against the same published peaks as the headline's roofline (HBM 8 TB/s, bf16 MFMA 2.5 PFLOP/s):
         # payload GB/s for the memory-bound ones, TFLOP/s for the prefill GEMM
         sec_roof = {}
@@ -625,7 +679,8 @@ def main():
                                 ("config4_prefill_M2048_N11008", "prefill_M2048_N11008_TFLOPs", "mfma"),
                                 ("config4_prefill_M512_N4096", "prefill_M512_N4096_TFLOPs", "mfma"),
                                 ("config5_moe_step", "moe_GBps", "hbm"),
-                                ("dequant_oil4_written", "dequant_oil4_11008x4096_written_GBps", "hbm")):
+                                ("dequant_oil4_written", "dequant_oil4_11008x4096_written_GBps", "hbm"),
+                                ("kv_cache_get_range_4096tok", "kv_get_range_4096tok_GBps", "hbm")):
             if key in extra:
                 peak = HBM_PEAK_GBS if bound == "hbm" else 2500.0
                 sec_roof[leg] = {"bound": bound, "achieved": extra[key], "peak": peak,

@@ -84,7 +84,6 @@ __device__ __forceinline__ uint32_t kv_nearest(const float (&cen)[16], float x) 
 struct KvLds {
     float srt[128];
     float cen[16];
-    uint8_t bucket[128];
     uint8_t code[128];
 };
 
@@ -138,19 +137,51 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
 #pragma unroll
     for (int c = 0; c < 16; ++c) cen[c] = L.cen[c];
     for (int it = 0; it < 20; ++it) {
-        if (lane < n) L.bucket[lane] = (uint8_t)kv_nearest(cen, s0);
-        if (lane + 64 < n) L.bucket[lane + 64] = (uint8_t)kv_nearest(cen, s1);
-        __syncthreads();
-        if (lane < 16) {                 // lane c sums its cluster in ascending order, as the reference's loop does
-            float sum = 0.f;
-            int cnt = 0;
-            for (uint32_t i = 0; i < n; ++i)
-                if (L.bucket[i] == lane) { sum = __fadd_rn(sum, L.srt[i]); ++cnt; }
-            if (cnt > 0) L.cen[lane] = __fdiv_rn(sum, (float)cnt);      // an empty cluster keeps its centroid
+        // lane c < 16 collects the members of cluster c as bit masks over the sorted order and adds them up in that
+        // order, as the reference's loop over the sorted values does (four LDS reads in flight per round)
+        const uint32_t b0 = lane < n ? kv_nearest(cen, s0) : 16u;
+        const uint32_t b1 = lane + 64 < n ? kv_nearest(cen, s1) : 16u;
+        uint64_t m0 = 0, m1 = 0;
+#pragma unroll
+        for (uint32_t c = 0; c < 16; ++c) {
+            const uint64_t w0 = __ballot(b0 == c);
+            const uint64_t w1 = n > 64 ? __ballot(b1 == c) : 0ull;
+            if (lane == c) { m0 = w0; m1 = w1; }
         }
+        float sum = 0.f;
+        const int cnt = __popcll(m0) + __popcll(m1);
+        for (int half = 0; half < 2; ++half) {
+            uint64_t m = half ? m1 : m0;
+            const float* base = L.srt + 64 * half;
+            while (m) {
+                uint32_t i[4];
+                bool h[4];
+                float val[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    h[u] = m != 0;
+                    i[u] = h[u] ? (uint32_t)__builtin_ctzll(m) : 0u;
+                    m &= m - 1;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) val[u] = base[i[u]];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    if (h[u]) sum = __fadd_rn(sum, val[u]);
+            }
+        }
+        bool moved = false;
+        if (lane < 16 && cnt > 0) {                                              // an empty cluster keeps its centroid
+            const float nv = __fdiv_rn(sum, (float)cnt);
+            moved = __float_as_uint(nv) != __float_as_uint(L.cen[lane]);
+            L.cen[lane] = nv;
+        }
+        const bool any_moved = __ballot(moved) != 0;
         __syncthreads();
+        if (!any_moved) break;           // a fixed point: the remaining iterations would reproduce these centroids bit for bit
 #pragma unroll
         for (int c = 0; c < 16; ++c) cen[c] = L.cen[c];
+        __syncthreads();
     }
     if (lane < n) L.code[lane] = (uint8_t)kv_nearest(cen, x0);
     if (lane + 64 < n) L.code[lane + 64] = (uint8_t)kv_nearest(cen, x1);
