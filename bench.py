@@ -561,6 +561,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
+    ap.add_argument("--kv-only", action="store_true", help="only run the KV-cache leg (for profiling its kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain 1 GiB device copies (reference for the FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -577,6 +578,9 @@ def main():
         sys.exit("bench.py: no GPU visible")
     info = ia.probe()
     log(f"device: {info['name']} gfx{info['gfx']} {info['compute_units']} CUs")
+    if args.kv_only:
+        print(json.dumps({"kv_cache_leg": bench_kv_cache(torch, ia)}), flush=True)
+        return
     if args.calibrate_copy:
         a = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()     # 1 GiB
         b = torch.empty_like(a)

@@ -12,6 +12,7 @@
 #include <cstdint>
 #include <stdexcept>
 #include <string>
+#include <utility>
 #include <vector>
 
 #if __has_include("oil/types.h")
@@ -91,6 +92,40 @@ public:
 private:
     void* handle_ = nullptr;
     uint64_t rows_ = 0, cols_ = 0;
+};
+
+// oil::OIL4KVCache (include/oil/kv_cache_oil4.h:26-83) with its state in HBM.  Same methods and meaning; where the
+// reference passes oil::Tensor, host pointers over the same memory: k / v of append are [seq_len][heads * dim] floats
+// (what the reference reads from its [1, heads, seq, dim] tensors, src/kv_cache_oil4.cpp:213-229), get_range returns
+// the two [len][heads * dim] arrays.  heads * dim must be even; errors throw oil::Error.
+class OIL4KVCache {
+public:
+    OIL4KVCache(int num_layers, int64_t max_seq_len, int64_t num_heads, int64_t head_dim, int64_t block_size = 64);
+    ~OIL4KVCache();
+    OIL4KVCache(const OIL4KVCache&) = delete;
+    OIL4KVCache& operator=(const OIL4KVCache&) = delete;
+    void append(int layer, const float* k, const float* v, int64_t seq_len);
+    std::pair<std::vector<float>, std::vector<float>> get_range(int layer, int64_t start, int64_t end) const;
+    std::pair<std::vector<float>, std::vector<float>> get_all(int layer) const;
+    int context_len() const;
+    int64_t max_seq_len() const { return max_seq_len_; }
+    int64_t block_size() const;
+    int num_layers() const { return num_layers_; }
+    int64_t num_heads() const { return num_heads_; }
+    int64_t head_dim() const { return head_dim_; }
+    size_t size_bytes() const;
+    size_t size_bytes_fp32_equivalent() const;
+    double compression_ratio() const;
+    void clear();
+    void resize(int64_t new_max_seq_len);
+    // n <= 128 values; indices one code per byte
+    static void quantize_block_oil4(const float* src, uint8_t* indices, uint16_t* codebook_fp16, int64_t n);
+    static void dequantize_block_oil4(const uint8_t* indices, const uint16_t* codebook_fp16, float* dst, int64_t n);
+    static constexpr int OIL4_CODEBOOK_SIZE = 16;
+private:
+    void* handle_ = nullptr;
+    int num_layers_ = 0;
+    int64_t max_seq_len_ = 0, num_heads_ = 0, head_dim_ = 0;
 };
 
 // backend::probe_hardware / select_optimal_backend hook (include/oil/backend.h:98-139):

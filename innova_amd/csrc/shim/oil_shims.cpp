@@ -5,6 +5,8 @@
 
 #include <cstring>
 
+#include <algorithm>
+
 #include "../../../include/oilhip.h"
 
 namespace {
@@ -187,6 +189,90 @@ uint64_t DeviceTensor::payload_bytes() const {
     uint64_t v = 0;
     ok(oilhip_weights_info(static_cast<oilhip_weights*>(handle_), nullptr, nullptr, nullptr, &v, nullptr), "info");
     return v;
+}
+
+// ---- OIL4KVCache (include/oil/kv_cache_oil4.h:26-83)
+OIL4KVCache::OIL4KVCache(int num_layers, int64_t max_seq_len, int64_t num_heads, int64_t head_dim, int64_t block_size)
+    : num_layers_(num_layers), max_seq_len_(max_seq_len), num_heads_(num_heads), head_dim_(head_dim) {
+    oilhip_kv* h = nullptr;
+    ok(oilhip_kv_create(num_layers, max_seq_len, num_heads, head_dim, block_size, &h), "OIL4KVCache");
+    handle_ = h;
+}
+OIL4KVCache::~OIL4KVCache() { oilhip_kv_destroy(static_cast<oilhip_kv*>(handle_)); }
+
+void OIL4KVCache::append(int layer, const float* k, const float* v, int64_t seq_len) {
+    const size_t n = sz(seq_len) * sz(num_heads_ * head_dim_);
+    Dev<float> dk(k, n), dv(v, n);
+    ok(oilhip_kv_append(static_cast<oilhip_kv*>(handle_), layer, dk.get(), dv.get(), seq_len, nullptr), "OIL4KVCache::append");
+    hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+}
+
+std::pair<std::vector<float>, std::vector<float>> OIL4KVCache::get_range(int layer, int64_t start, int64_t end) const {
+    const int64_t want = std::max<int64_t>(0, std::min(end, max_seq_len_) - start);
+    const size_t per_token = sz(num_heads_ * head_dim_);
+    Dev<float> dk(nullptr, sz(want) * per_token), dv(nullptr, sz(want) * per_token);
+    int64_t len = 0;
+    ok(oilhip_kv_get_range(static_cast<const oilhip_kv*>(handle_), layer, start, end, dk.get(), dv.get(), &len, nullptr),
+       "OIL4KVCache::get_range");
+    std::pair<std::vector<float>, std::vector<float>> out;
+    out.first.resize(sz(len) * per_token);
+    out.second.resize(sz(len) * per_token);
+    if (len > 0) {
+        hip_ok(hipMemcpy(out.first.data(), dk.get(), out.first.size() * 4, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+        hip_ok(hipMemcpy(out.second.data(), dv.get(), out.second.size() * 4, hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    }
+    return out;
+}
+std::pair<std::vector<float>, std::vector<float>> OIL4KVCache::get_all(int layer) const { return get_range(layer, 0, max_seq_len_); }
+
+int OIL4KVCache::context_len() const {
+    int v = 0;
+    ok(oilhip_kv_info(static_cast<const oilhip_kv*>(handle_), &v, nullptr, nullptr, nullptr), "kv_info");
+    return v;
+}
+int64_t OIL4KVCache::block_size() const {
+    int64_t v = 0;
+    ok(oilhip_kv_info(static_cast<const oilhip_kv*>(handle_), nullptr, &v, nullptr, nullptr), "kv_info");
+    return v;
+}
+size_t OIL4KVCache::size_bytes() const {
+    uint64_t v = 0;
+    ok(oilhip_kv_info(static_cast<const oilhip_kv*>(handle_), nullptr, nullptr, &v, nullptr), "kv_info");
+    return (size_t)v;
+}
+size_t OIL4KVCache::size_bytes_fp32_equivalent() const {
+    uint64_t v = 0;
+    ok(oilhip_kv_info(static_cast<const oilhip_kv*>(handle_), nullptr, nullptr, nullptr, &v), "kv_info");
+    return (size_t)v;
+}
+double OIL4KVCache::compression_ratio() const {
+    const size_t q = size_bytes();
+    return q == 0 ? 0.0 : (double)size_bytes_fp32_equivalent() / (double)q;
+}
+void OIL4KVCache::clear() {
+    ok(oilhip_kv_clear(static_cast<oilhip_kv*>(handle_), nullptr), "OIL4KVCache::clear");
+    hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+}
+void OIL4KVCache::resize(int64_t new_max_seq_len) {
+    ok(oilhip_kv_resize(static_cast<oilhip_kv*>(handle_), new_max_seq_len), "OIL4KVCache::resize");
+    max_seq_len_ = new_max_seq_len;
+}
+void OIL4KVCache::quantize_block_oil4(const float* src, uint8_t* indices, uint16_t* codebook_fp16, int64_t n) {
+    if (n <= 0) return;
+    Dev<float> ds(src, sz(n));
+    Dev<uint8_t> dc(nullptr, sz(n));
+    Dev<uint16_t> db(nullptr, 16);
+    ok(oilhip_kv_quantize_blocks(ds.get(), n, 1, dc.get(), db.get(), nullptr), "OIL4KVCache::quantize_block_oil4");
+    dc.to_host(indices);
+    db.to_host(codebook_fp16);
+}
+void OIL4KVCache::dequantize_block_oil4(const uint8_t* indices, const uint16_t* codebook_fp16, float* dst, int64_t n) {
+    if (n <= 0) return;
+    Dev<uint8_t> dc(indices, sz(n));
+    Dev<uint16_t> db(codebook_fp16, 16);
+    Dev<float> dd(nullptr, sz(n));
+    ok(oilhip_kv_dequantize_blocks(dc.get(), db.get(), dd.get(), n, 1, nullptr), "OIL4KVCache::dequantize_block_oil4");
+    dd.to_host(dst);
 }
 
 bool probe(std::string* name, uint64_t* hbm_bytes, int* compute_units) {

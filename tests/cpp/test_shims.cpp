@@ -1,6 +1,7 @@
 // test_shims.cpp -- the C++ drop-in layer called the way the reference's own tests call
 // its kernels (tests/test_kernel.cpp:82-103, tests/test_quant_engines.cpp:229-263,
 // tests/test_block_codec.cpp), with results checked against brute-force double loops.
+#include <algorithm>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -137,6 +138,39 @@ int main() {
         bool threw = false;
         try { gfx950::DeviceTensor bad(refs, rows + 1, cols); } catch (const oil::Error&) { threw = true; }
         CHECK(threw, "shape mismatch must throw oil::Error");
+    }
+    {   // OIL4KVCache: prefill + two decode appends; ranges are slices of the whole, the static pair round-trips
+        // through the cache's own centroids, appends past max_seq_len are dropped but counted
+        const int heads = 4, dim = 64, pt = heads * dim, n = 9;
+        gfx950::OIL4KVCache cache(2, 10, heads, dim, 64);
+        std::vector<float> k((size_t)n * pt), v((size_t)n * pt);
+        for (auto& x : k) x = frand();
+        for (auto& x : v) x = frand() * 3.0f;
+        cache.append(0, k.data(), v.data(), 7);
+        cache.append(0, k.data() + 7 * pt, v.data() + 7 * pt, 1);
+        cache.append(0, k.data() + 8 * pt, v.data() + 8 * pt, 1);
+        CHECK(cache.context_len() == 9 && cache.block_size() == 64 && cache.num_layers() == 2, "kv accessors");
+        auto all = cache.get_all(0);
+        CHECK(all.first.size() == (size_t)n * pt && all.second.size() == (size_t)n * pt, "get_all size %zu", all.first.size());
+        auto part = cache.get_range(0, 2, 5);
+        CHECK(part.first.size() == (size_t)3 * pt && std::memcmp(part.first.data(), all.first.data() + 2 * pt, (size_t)3 * pt * 4) == 0, "get_range slice");
+        float worst = 0.f;
+        for (size_t i = 0; i < all.first.size(); ++i) worst = std::max(worst, std::fabs(all.first[i] - k[i]));
+        CHECK(worst < 0.25f, "kv quantization error %.3g", worst);
+        CHECK(cache.get_all(1).first.empty() && cache.get_range(5, 0, 3).first.empty(), "empty layer / no such layer");
+        std::vector<uint8_t> codes(64);
+        std::vector<uint16_t> cb(16);
+        std::vector<float> back(64);
+        gfx950::OIL4KVCache::quantize_block_oil4(k.data(), codes.data(), cb.data(), 64);
+        gfx950::OIL4KVCache::dequantize_block_oil4(codes.data(), cb.data(), back.data(), 64);
+        CHECK(std::memcmp(back.data(), all.first.data(), 64 * 4) == 0, "static pair equals the cache's first block");
+        cache.append(0, k.data(), v.data(), 3);
+        CHECK(cache.context_len() == 12 && cache.get_all(0).first.size() == (size_t)10 * pt, "overflow: dropped, counted");
+        cache.clear();
+        CHECK(cache.context_len() == 0 && cache.get_all(0).first.empty(), "clear");
+        bool threw = false;
+        try { gfx950::OIL4KVCache odd(1, 4, 3, 5); } catch (const oil::Error&) { threw = true; }
+        CHECK(threw, "odd token size must throw oil::Error");
     }
     std::printf("test_shims: %d checks, %d failures\n", g_checks, g_fail);
     return g_fail ? 1 : 0;
