@@ -467,7 +467,7 @@ def bench_dequant_and_engine(torch, ia, payload, blocks):
     return out
 
 
-def bench_kv_cache(torch, ia):
+def bench_kv_cache(torch, ia, with_cpu=False):
     """The OIL4 KV cache of one Llama-7B-shaped layer (32 heads x 128, block 64): get_range over a 4096-token context
     (per value 0.5 B of codes + 0.5 B of centroids read, 4 B of FP32 written, K and V in one launch), a 2048-token
     prefill append and a one-token decode append (Lloyd-Max on the device, one wavefront per 64-value chunk)."""
@@ -517,6 +517,22 @@ def bench_kv_cache(torch, ia):
     nbytes = 2 * ctx * pt * (0.5 + 32 / 64 + 4)
     out["kv_get_range_4096tok_us"] = round(t * 1e6, 1)
     out["kv_get_range_4096tok_GBps"] = round(nbytes / t / 1e9, 1)
+    if with_cpu:
+        # the same cache on one host core through the oracle's restatement of OIL4KVCache (a bounded sample: 32 tokens
+        # appended, then read back 8 times)
+        import numpy as np
+        import oracle as O
+        oc = O.KVCache(64, heads, dim, 64)
+        kh, vh = k.reshape(-1, pt)[:32].cpu().numpy(), v.reshape(-1, pt)[:32].cpu().numpy()
+        t0 = time.perf_counter()
+        oc.append(kh, vh)
+        t_app = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        for _ in range(8):
+            oc.get_range(0, 32)
+        t_get = (time.perf_counter() - t0) / 8
+        out["kv_cpu_port_1core_append_us_per_token"] = round(t_app / 32 * 1e6, 1)
+        out["kv_cpu_port_1core_get_range_GBps"] = round(2 * 32 * pt * (0.5 + 32 / 64 + 4) / t_get / 1e9, 3)
     return out
 
 
@@ -579,7 +595,7 @@ def main():
     info = ia.probe()
     log(f"device: {info['name']} gfx{info['gfx']} {info['compute_units']} CUs")
     if args.kv_only:
-        print(json.dumps({"kv_cache_leg": bench_kv_cache(torch, ia)}), flush=True)
+        print(json.dumps({"kv_cache_leg": bench_kv_cache(torch, ia, with_cpu=not args.no_cpu)}), flush=True)
         return
     if args.calibrate_copy:
         a = torch.empty(1 << 28, dtype=torch.float32, device="cuda").normal_()     # 1 GiB
@@ -669,7 +685,7 @@ def main():
         extra.update(bench_mixed_stack(torch, ia))
         extra.update(bench_prefill(torch, ia, payload, blocks))
         extra.update(bench_moe(torch, ia))
-        extra.update(bench_kv_cache(torch, ia))
+        extra.update(bench_kv_cache(torch, ia, with_cpu=not args.no_cpu))
         # the secondary legs against the same published peaks as the headline's roofline (HBM 8 TB/s, bf16 MFMA 2.5 PFLOP/s):
         # payload GB/s for the memory-bound ones, TFLOP/s for the prefill GEMM
         sec_roof = {}
