@@ -137,44 +137,68 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
 #pragma unroll
     for (int c = 0; c < 16; ++c) cen[c] = L.cen[c];
     for (int it = 0; it < 20; ++it) {
-        // lane c < 16 collects the members of cluster c as bit masks over the sorted order and adds them up in that
-        // order, as the reference's loop over the sorted values does (four LDS reads in flight per round)
         const uint32_t b0 = lane < n ? kv_nearest(cen, s0) : 16u;
-        const uint32_t b1 = lane + 64 < n ? kv_nearest(cen, s1) : 16u;
-        uint64_t m0 = 0, m1 = 0;
-#pragma unroll
-        for (uint32_t c = 0; c < 16; ++c) {
-            const uint64_t w0 = __ballot(b0 == c);
-            const uint64_t w1 = n > 64 ? __ballot(b1 == c) : 0ull;
-            if (lane == c) { m0 = w0; m1 = w1; }
-        }
-        float sum = 0.f;
-        const int cnt = __popcll(m0) + __popcll(m1);
-        for (int half = 0; half < 2; ++half) {
-            uint64_t m = half ? m1 : m0;
-            const float* base = L.srt + 64 * half;
-            while (m) {
-                uint32_t i[4];
-                bool h[4];
-                float val[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    h[u] = m != 0;
-                    i[u] = h[u] ? (uint32_t)__builtin_ctzll(m) : 0u;
-                    m &= m - 1;
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) val[u] = base[i[u]];
-#pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    if (h[u]) sum = __fadd_rn(sum, val[u]);
-            }
-        }
         bool moved = false;
-        if (lane < 16 && cnt > 0) {                                              // an empty cluster keeps its centroid
-            const float nv = __fdiv_rn(sum, (float)cnt);
-            moved = __float_as_uint(nv) != __float_as_uint(L.cen[lane]);
-            L.cen[lane] = nv;
+        // the cluster of the value to the left (wave_shr:1; lane 0 reads 0)
+        const uint32_t prev = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)b0, 0x138, 0xF, 0xF, true);
+        if (n <= 64 && __ballot(lane > 0 && b0 < prev) == 0) {
+            // Cluster numbers do not fall along the sorted values (the usual case), so every cluster is one run of
+            // lanes.  Each lane folds its run from the left, one neighbour step at a time: after step t the lanes at
+            // depth <= t of their run hold 0 + x_first + ... + x_self in exactly the reference's order.  The last lane
+            // of a run owns the cluster's sum and count.
+            const uint64_t heads = __ballot(lane == 0 || b0 != prev);
+            const uint32_t first = 63u - (uint32_t)__builtin_clzll(heads & (~0ull >> (63u - lane)));
+            const uint32_t depth = lane - first;
+            float fold = __fadd_rn(0.f, s0);
+            for (uint32_t t = 1; __ballot(depth >= t) != 0; ++t) {
+                const float left = __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(fold), 0x138, 0xF, 0xF, true));
+                const float next = __fadd_rn(left, s0);
+                fold = depth >= t ? next : fold;
+            }
+            const bool tail = lane == 63 || ((heads >> ((lane + 1) & 63u)) & 1ull) != 0;
+            if (tail && b0 < 16) {
+                const float nv = __fdiv_rn(fold, (float)(depth + 1));
+                moved = __float_as_uint(nv) != __float_as_uint(L.cen[b0]);
+                L.cen[b0] = nv;
+            }
+        } else {
+            // lane c < 16 collects the members of cluster c as bit masks over the sorted order and adds them up in that
+            // order, as the reference's loop over the sorted values does (four LDS reads in flight per round)
+            const uint32_t b1 = lane + 64 < n ? kv_nearest(cen, s1) : 16u;
+            uint64_t m0 = 0, m1 = 0;
+#pragma unroll
+            for (uint32_t c = 0; c < 16; ++c) {
+                const uint64_t w0 = __ballot(b0 == c);
+                const uint64_t w1 = n > 64 ? __ballot(b1 == c) : 0ull;
+                if (lane == c) { m0 = w0; m1 = w1; }
+            }
+            float sum = 0.f;
+            const int cnt = __popcll(m0) + __popcll(m1);
+            for (int half = 0; half < 2; ++half) {
+                uint64_t m = half ? m1 : m0;
+                const float* base = L.srt + 64 * half;
+                while (m) {
+                    uint32_t i[4];
+                    bool h[4];
+                    float val[4];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) {
+                        h[u] = m != 0;
+                        i[u] = h[u] ? (uint32_t)__builtin_ctzll(m) : 0u;
+                        m &= m - 1;
+                    }
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) val[u] = base[i[u]];
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+                        if (h[u]) sum = __fadd_rn(sum, val[u]);
+                }
+            }
+            if (lane < 16 && cnt > 0) {                                              // an empty cluster keeps its centroid
+                const float nv = __fdiv_rn(sum, (float)cnt);
+                moved = __float_as_uint(nv) != __float_as_uint(L.cen[lane]);
+                L.cen[lane] = nv;
+            }
         }
         const bool any_moved = __ballot(moved) != 0;
         __syncthreads();
