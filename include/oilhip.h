@@ -273,8 +273,8 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
 /* ------------------------------------------------------------ OIL4 KV cache
  * The device-resident oil::OIL4KVCache (include/oil/kv_cache_oil4.h:26-83, src/kv_cache_oil4.cpp): per layer the K and
  * V streams [token][heads * dim] as 4-bit codes (two per byte, low nibble first) with 16 FP16 centroids per block of
- * 32 / 64 / 128 consecutive values (any other block_size means 64, :25-26).  heads * dim must be even.  Codes and
- * centroids are the reference's bit for bit (inputs must be finite).
+ * 32 / 64 / 128 consecutive values (any other block_size means 64, :25-26).  Codes and centroids are the
+ * reference's bit for bit (inputs must be finite), also where heads * dim is odd and the reference's chunks share bytes.
  * oilhip_kv_create            : OIL4KVCache(num_layers, max_seq_len, num_heads, head_dim, block_size) / init (:13-43)
  * oilhip_kv_append            : append(layer, k, v) (:207-291); d_k, d_v: [seq_len][heads * dim] FP32 on the device.
  *                               Tokens beyond max_seq_len are dropped but still counted, layer >= num_layers is ignored,

@@ -97,7 +97,7 @@ private:
 // oil::OIL4KVCache (include/oil/kv_cache_oil4.h:26-83) with its state in HBM.  Same methods and meaning; where the
 // reference passes oil::Tensor, host pointers over the same memory: k / v of append are [seq_len][heads * dim] floats
 // (what the reference reads from its [1, heads, seq, dim] tensors, src/kv_cache_oil4.cpp:213-229), get_range returns
-// the two [len][heads * dim] arrays.  heads * dim must be even; errors throw oil::Error.
+// the two [len][heads * dim] arrays.  Errors throw oil::Error.
 class OIL4KVCache {
 public:
     OIL4KVCache(int num_layers, int64_t max_seq_len, int64_t num_heads, int64_t head_dim, int64_t block_size = 64);

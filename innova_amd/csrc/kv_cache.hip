@@ -8,9 +8,11 @@
 //   get_range : codes -> centroids -> FP32 [len][heads * dim] through the cache's own half decode
 //               (CodebookOIL4::half_to_float, src/codebook.cpp:36-64, which is not IEEE for subnormals).
 //
-// The device path needs an even number of values per token: every chunk then starts on a byte and element e of a
-// layer is nibble e & 1 of byte e / 2 (with an odd count the reference's chunks overlap in a byte and the result
-// depends on the order of the writes).
+// A chunk's codes are packed from its own first byte, block * (block / 2) + offset / 2 (:246).  With an even number
+// of values per token that makes element e of a layer nibble e & 1 of byte e / 2.  With an odd number a chunk that
+// starts at an even offset and holds an odd count shares its last byte with the chunk behind it, and the later write
+// wins (the earlier chunk's last code is lost, as in the reference); the kernels reproduce that by leaving the shared
+// byte to the later chunk.
 #include <algorithm>
 #include <new>
 #include <vector>
@@ -218,7 +220,7 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
 __global__ void __launch_bounds__(64)
 kv_append_kernel(uint8_t* __restrict__ k_idx, uint8_t* __restrict__ v_idx, uint16_t* __restrict__ k_cb,
                  uint16_t* __restrict__ v_cb, const float* __restrict__ k, const float* __restrict__ v, int64_t pos,
-                 int64_t ntok, int64_t per_token, uint32_t block, uint32_t chunks_per_token) {
+                 int64_t ntok, int64_t per_token, uint32_t block, uint32_t chunks_per_token, int64_t idx_bytes) {
     __shared__ KvLds L;
     const uint32_t lane = threadIdx.x;
     const int64_t s = blockIdx.x / chunks_per_token;
@@ -232,9 +234,14 @@ kv_append_kernel(uint8_t* __restrict__ k_idx, uint8_t* __restrict__ v_idx, uint1
     const uint32_t n = (uint32_t)(b - a);
     const float* src = (is_v ? v : k) + (a - pos * per_token);
     kv_quantize_chunk(src, n, lane, L);
-    uint8_t* idx = (is_v ? v_idx : k_idx) + (a >> 1);
-    if (lane < (n >> 1)) idx[lane] = (uint8_t)(L.code[2 * lane] | (L.code[2 * lane + 1] << 4));
     const bool last_on_block = (b % block) == 0 || b == (pos + ntok) * per_token;
+    const uint32_t off = (uint32_t)(a % block);
+    const int64_t at = blk * (int64_t)(block >> 1) + (off >> 1);
+    uint32_t nbytes = (n + 1) >> 1;
+    if (!(off & 1u) && (n & 1u) && !last_on_block) --nbytes;        // that byte belongs to the next chunk of this call
+    if (at + nbytes > idx_bytes) nbytes = at < idx_bytes ? (uint32_t)(idx_bytes - at) : 0u;   // :248-249
+    uint8_t* idx = (is_v ? v_idx : k_idx) + at;
+    if (lane < nbytes) idx[lane] = (uint8_t)(L.code[2 * lane] | (2 * lane + 1 < n ? L.code[2 * lane + 1] << 4 : 0));
     const bool store_cb = (is_v || pos == 0) ? last_on_block : (a % block) == 0;
     if (store_cb && lane < 16) (is_v ? v_cb : k_cb)[blk * 16 + lane] = (uint16_t)kv_float_to_half(L.cen[lane]);
 }
@@ -260,7 +267,7 @@ kv_dequantize_blocks_kernel(const uint8_t* __restrict__ codes, const uint16_t* _
     dst[i] = kv_half_to_float(cb[(i / n) * 16 + (codes[i] & 15u)]);
 }
 
-// get_range for tokens whose value count is a multiple of 4.  A workgroup decodes kTile consecutive elements of K
+// get_range for tokens whose value count is a multiple of 4 (value e is then nibble e & 1 of byte e / 2).  A workgroup decodes kTile consecutive elements of K
 // (blockIdx.y = 0) or V (1): the centroids of the blocks under the tile go to LDS as FP32 once, then each thread
 // turns 2 bytes of codes into one 16-byte store, four times.
 constexpr uint32_t kTile = 4096;
@@ -294,18 +301,25 @@ kv_get_range_kernel(const uint8_t* __restrict__ k_idx, const uint8_t* __restrict
     }
 }
 
-// get_range, one element per thread (even value counts that are not multiples of 4)
+// get_range, one value per thread, with the reference's chunk arithmetic (:318-334): the chunk of a value starts at
+// the later of its token's first value and its block's first value, and its codes count from the chunk's own byte.
 __global__ void __launch_bounds__(256)
 kv_get_range_scalar_kernel(const uint8_t* __restrict__ k_idx, const uint8_t* __restrict__ v_idx,
                            const uint16_t* __restrict__ k_cb, const uint16_t* __restrict__ v_cb, float* __restrict__ k_out,
-                           float* __restrict__ v_out, uint64_t first, uint64_t count, uint32_t block_shift) {
+                           float* __restrict__ v_out, uint64_t first, uint64_t count, uint32_t block_shift, uint64_t per_token,
+                           uint64_t idx_bytes) {
     const uint64_t j = (uint64_t)blockIdx.x * 256 + threadIdx.x;
     if (j >= count) return;
     const uint64_t e = first + j;
+    const uint64_t blk = e >> block_shift;
+    const uint64_t tok_lo = e / per_token * per_token, blk_lo = blk << block_shift;
+    const uint64_t a = tok_lo > blk_lo ? tok_lo : blk_lo;
+    const uint64_t at = (blk << (block_shift - 1)) + ((a - blk_lo) >> 1) + ((e - a) >> 1);
     const uint8_t* idx = blockIdx.y ? v_idx : k_idx;
     const uint16_t* cb = blockIdx.y ? v_cb : k_cb;
-    const uint32_t code = (idx[e >> 1] >> (4 * (uint32_t)(e & 1))) & 15u;
-    (blockIdx.y ? v_out : k_out)[j] = kv_half_to_float(cb[(e >> block_shift) * 16 + code]);
+    const uint32_t byte = at < idx_bytes ? idx[at] : 0u;                              // :322-325
+    const uint32_t code = (byte >> (4 * (uint32_t)((e - a) & 1))) & 15u;
+    (blockIdx.y ? v_out : k_out)[j] = kv_half_to_float(cb[blk * 16 + code]);
 }
 
 __global__ void __launch_bounds__(256) kv_zero_kernel(uint4* p, uint64_t n16) {
@@ -350,7 +364,6 @@ int oilhip_kv_create(int num_layers, int64_t max_seq_len, int64_t num_heads, int
     *out = nullptr;
     if (num_layers < 0 || max_seq_len < 0 || num_heads < 0 || head_dim < 0) return fail(OILHIP_E_ARG, "kv_create: negative size");
     const int64_t per_token = num_heads * head_dim;
-    if (per_token & 1) return fail(OILHIP_E_ARG, "kv_create: heads * dim must be even on the device path (odd token sizes make chunks share a byte)");
     if (per_token > 0 && max_seq_len > ((int64_t)1 << 40) / per_token) return fail(OILHIP_E_ARG, "kv_create: cache too large");
     oilhip_kv* c = new (std::nothrow) oilhip_kv;
     if (!c) return fail(OILHIP_E_NOMEM, "kv_create: out of host memory");
@@ -389,7 +402,7 @@ int oilhip_kv_append(oilhip_kv* c, int layer, const float* d_k, const float* d_v
         if (ntok * (int64_t)cpt > 0x7FFFFFFF) return fail(OILHIP_E_ARG, "kv_append: too many tokens for one call");
         hipLaunchKernelGGL(kv_append_kernel, dim3((uint32_t)(ntok * cpt), 2), dim3(64), 0, (hipStream_t)stream,
                            kv_idx(c, layer, 0), kv_idx(c, layer, 1), kv_cb(c, layer, 0), kv_cb(c, layer, 1), d_k, d_v, pos, ntok,
-                           c->per_token, (uint32_t)c->block, cpt);
+                           c->per_token, (uint32_t)c->block, cpt, c->idx_bytes);
         OILHIP_HIP(hipGetLastError());
     }
     c->pos[(size_t)layer] = pos + seq_len;                                          // :290, dropped tokens counted as well
@@ -422,7 +435,7 @@ int oilhip_kv_get_range(const oilhip_kv* c, int layer, int64_t start, int64_t en
         if (groups > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "kv_get_range: range too long for one call");
         hipLaunchKernelGGL(kv_get_range_scalar_kernel, dim3((uint32_t)groups, 2), dim3(256), 0, (hipStream_t)stream,
                            kv_idx(c, layer, 0), kv_idx(c, layer, 1), kv_cb(c, layer, 0), kv_cb(c, layer, 1), d_k, d_v, first, count,
-                           shift);
+                           shift, (uint64_t)c->per_token, (uint64_t)c->idx_bytes);
     }
     OILHIP_HIP(hipGetLastError());
     if (len_out) *len_out = len;

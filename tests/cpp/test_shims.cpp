@@ -168,9 +168,12 @@ int main() {
         CHECK(cache.context_len() == 12 && cache.get_all(0).first.size() == (size_t)10 * pt, "overflow: dropped, counted");
         cache.clear();
         CHECK(cache.context_len() == 0 && cache.get_all(0).first.empty(), "clear");
+        gfx950::OIL4KVCache odd(1, 4, 3, 5);            // an odd value count per token: chunks share bytes, as in the reference
+        odd.append(0, k.data(), v.data(), 3);
+        CHECK(odd.get_all(0).first.size() == 45, "odd token size");
         bool threw = false;
-        try { gfx950::OIL4KVCache odd(1, 4, 3, 5); } catch (const oil::Error&) { threw = true; }
-        CHECK(threw, "odd token size must throw oil::Error");
+        try { gfx950::OIL4KVCache bad(1, -4, 3, 5); } catch (const oil::Error&) { threw = true; }
+        CHECK(threw, "negative size must throw oil::Error");
     }
     std::printf("test_shims: %d checks, %d failures\n", g_checks, g_fail);
     return g_fail ? 1 : 0;

@@ -65,10 +65,6 @@ def test_quantize_blocks_fixture_and_oracle():
 @pytest.mark.parametrize("i", range(len(MF.KV_CASES)))
 def test_cache_fixture(i):
     ms, h, d, block, lens = MF.KV_CASES[i]
-    if (h * d) % 2:
-        with pytest.raises(ia.OilHipError):        # odd token sizes are refused (chunks would share a byte)
-            ia.OIL4KVCache(1, ms, h, d, block)
-        return
     k, v = MF.kv_inputs(i)
     c = ia.OIL4KVCache(2, ms, h, d, block)
     o = O.KVCache(ms, h, d, block)
@@ -95,7 +91,8 @@ def test_cache_fixture(i):
 
 
 @pytest.mark.parametrize("heads,dim,block,prefill,steps", [(8, 128, 64, 96, 5), (2, 64, 128, 33, 3), (4, 80, 32, 40, 4),
-                                                          (1, 6, 64, 50, 7), (3, 50, 64, 21, 6)])
+                                                          (1, 6, 64, 50, 7), (3, 50, 64, 21, 6),
+                                                          (3, 11, 64, 19, 5), (5, 7, 32, 30, 4), (1, 129, 128, 9, 3)])   # odd token sizes: chunks share bytes
 def test_prefill_then_decode_against_oracle(heads, dim, block, prefill, steps):
     rng = np.random.default_rng(heads * 1000 + dim)
     ms = prefill + steps + 2
@@ -166,7 +163,7 @@ def test_full_size_layer():
 
 def test_argument_errors():
     with pytest.raises(ia.OilHipError):
-        ia.OIL4KVCache(1, 8, 3, 5, 64)
+        ia.OIL4KVCache(1, -8, 3, 5, 64)
     c = ia.OIL4KVCache(1, 8, 2, 8, 64)
     with pytest.raises(ia.OilHipError):
         c.get_range(0, -1, 3)
