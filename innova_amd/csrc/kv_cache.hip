@@ -117,24 +117,42 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
     }
     if (lane < 16) L.cen[lane] = __fadd_rn(lo, __fdiv_rn(__fmul_rn(range, (float)lane + 0.5f), 16.0f));
 
-    // ascending sort of the n values (bitonic network over 64 or 128 slots, padded with +inf)
-    const uint32_t slots = n <= 64 ? 64u : 128u;
-    L.srt[lane] = lane < n ? x0 : __builtin_inff();
-    L.srt[lane + 64] = lane + 64 < n ? x1 : __builtin_inff();
-    __syncthreads();
-    for (uint32_t k = 2; k <= slots; k <<= 1) {
-        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
-            if (lane < (slots >> 1)) {
+    // ascending sort of the n values, padded with +inf: a bitonic network, in registers with one value per lane for
+    // chunks of up to 64 values (both lanes of a pair evaluate the same comparison, so equal values are never
+    // duplicated), over 128 LDS slots otherwise
+    float s0, s1;
+    if (n <= 64) {
+        s0 = lane < n ? x0 : __builtin_inff();
+        s1 = __builtin_inff();
+#pragma unroll
+        for (uint32_t k = 2; k <= 64; k <<= 1) {
+#pragma unroll
+            for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+                const float other = __shfl_xor(s0, (int)j, 64);
+                const bool keep_small = ((lane & j) == 0) == ((lane & k) == 0);
+                const bool take = keep_small ? other < s0 : other > s0;
+                s0 = take ? other : s0;
+            }
+        }
+        L.srt[lane] = s0;
+        __syncthreads();
+    } else {
+        L.srt[lane] = x0;
+        L.srt[lane + 64] = lane + 64 < n ? x1 : __builtin_inff();
+        __syncthreads();
+        for (uint32_t k = 2; k <= 128; k <<= 1) {
+            for (uint32_t j = k >> 1; j > 0; j >>= 1) {
                 const uint32_t i = ((lane & ~(j - 1)) << 1) | (lane & (j - 1));
                 const uint32_t p = i | j;
                 const bool up = (i & k) == 0;
                 const float a = L.srt[i], b = L.srt[p];
                 if ((a > b) == up) { L.srt[i] = b; L.srt[p] = a; }
+                __syncthreads();
             }
-            __syncthreads();
         }
+        s0 = L.srt[lane];
+        s1 = L.srt[lane + 64];
     }
-    const float s0 = L.srt[lane], s1 = L.srt[lane + 64];
     float cen[16];
 #pragma unroll
     for (int c = 0; c < 16; ++c) cen[c] = L.cen[c];
