@@ -89,16 +89,13 @@ struct KvLds {
     uint8_t code[128];
 };
 
-// lloyd_max_16 (src/kv_cache_oil4.cpp:75-153) for n <= 128 values by one wavefront.  Leaves the n codes in L.code and
-// the 16 centroids (FP32) in L.cen.
-__device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uint32_t lane, KvLds& L) {
-    const float x0 = lane < n ? src[lane] : 0.f;
-    const float x1 = lane + 64 < n ? src[lane + 64] : 0.f;
-    // minimum with the first of equal values kept (the sign of a zero minimum reaches the constant chunk's centroids)
-    float lo = lane < n ? x0 : __builtin_inff();
+// Minimum (the first of equal values: the sign of a zero minimum reaches a constant chunk's centroids) and maximum of
+// the chunk, in every lane.
+__device__ __forceinline__ void kv_min_max(float x0, float x1, uint32_t n, uint32_t lane, float& lo, float& hi) {
+    lo = lane < n ? x0 : __builtin_inff();
     uint32_t lo_i = lane;
     if (lane + 64 < n && x1 < lo) { lo = x1; lo_i = lane + 64; }
-    float hi = lane < n ? x0 : -__builtin_inff();
+    hi = lane < n ? x0 : -__builtin_inff();
     if (lane + 64 < n && x1 > hi) hi = x1;
     for (int o = 32; o > 0; o >>= 1) {
         const float ol = __shfl_xor(lo, o, 64);
@@ -107,20 +104,17 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
         const float oh = __shfl_xor(hi, o, 64);
         if (oh > hi) hi = oh;
     }
-    const float range = __fsub_rn(hi, lo);
-    if (range < 1e-10f) {
-        if (lane < n) L.code[lane] = 8;
-        if (lane + 64 < n) L.code[lane + 64] = 8;
-        if (lane < 16) L.cen[lane] = lo;
-        __syncthreads();
-        return;
-    }
-    if (lane < 16) L.cen[lane] = __fadd_rn(lo, __fdiv_rn(__fmul_rn(range, (float)lane + 0.5f), 16.0f));
+}
 
-    // ascending sort of the n values, padded with +inf: a bitonic network, in registers with one value per lane for
+// lloyd_max_16 (src/kv_cache_oil4.cpp:75-153) for n <= 128 values by one wavefront.  Leaves the n codes in L.code and
+// the 16 centroids (FP32) in L.cen.
+__device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uint32_t lane, KvLds& L) {
+    const float x0 = lane < n ? src[lane] : 0.f;
+    const float x1 = lane + 64 < n ? src[lane + 64] : 0.f;
+    // Ascending sort of the n values, padded with +inf: a bitonic network, in registers with one value per lane for
     // chunks of up to 64 values (both lanes of a pair evaluate the same comparison, so equal values are never
-    // duplicated), over 128 LDS slots otherwise
-    float s0, s1;
+    // duplicated), over 128 LDS slots otherwise.  The sorted ends are the minimum and the maximum.
+    float s0, s1, lo, hi;
     if (n <= 64) {
         s0 = lane < n ? x0 : __builtin_inff();
         s1 = __builtin_inff();
@@ -134,6 +128,22 @@ __device__ void kv_quantize_chunk(const float* __restrict__ src, uint32_t n, uin
                 s0 = take ? other : s0;
             }
         }
+        lo = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s0), 0));
+        hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(s0), (int)n - 1));
+    } else {
+        kv_min_max(x0, x1, n, lane, lo, hi);
+    }
+    const float range = __fsub_rn(hi, lo);
+    if (range < 1e-10f) {
+        if (n <= 64) kv_min_max(x0, x1, n, lane, lo, hi);       // which of several equal zeros comes first
+        if (lane < n) L.code[lane] = 8;
+        if (lane + 64 < n) L.code[lane + 64] = 8;
+        if (lane < 16) L.cen[lane] = lo;
+        __syncthreads();
+        return;
+    }
+    if (lane < 16) L.cen[lane] = __fadd_rn(lo, __fdiv_rn(__fmul_rn(range, (float)lane + 0.5f), 16.0f));
+    if (n <= 64) {
         L.srt[lane] = s0;
         __syncthreads();
     } else {
