@@ -50,8 +50,9 @@ class Ring:
             d.close()
 
 
-def time_ring(torch, ring, x, y, steps, warmup):
-    """Average seconds per GEMV launch over `steps` launches (graph replay of the ring)."""
+def time_ring(torch, ring, x, y, steps, warmup, settle_s=0.0):
+    """Average seconds per GEMV launch over `steps` launches (graph replay of the ring).  settle_s: untimed replays for
+    that long in front of the timed region, so that a device that comes out of idle has reached its steady clocks."""
     n = len(ring.items)
     for i in range(max(warmup, n)):                    # untimed warm-up (also first-call setup)
         ring.items[i % n].gemv(x, out=y)
@@ -67,6 +68,11 @@ def time_ring(torch, ring, x, y, steps, warmup):
     with torch.cuda.stream(stream):
         graph.replay()
         torch.cuda.synchronize()
+        t_end = time.perf_counter() + settle_s
+        while time.perf_counter() < t_end:
+            for _ in range(8):
+                graph.replay()
+            torch.cuda.synchronize()
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
@@ -614,7 +620,7 @@ def main():
     x = torch.from_numpy(xh).cuda()
     y = torch.empty((1, ROWS), dtype=torch.float32, device="cuda")
 
-    sec, wall = time_ring(torch, ring, x, y, args.steps, args.warmup)
+    sec, wall = time_ring(torch, ring, x, y, args.steps, args.warmup, settle_s=0.3)
     algo_bytes = ring.payload_bytes + 4 * COLS + 4 * ROWS          # weights + x + y, each once
     value = ring.payload_bytes / sec / 1e9
     achieved = algo_bytes / sec / 1e9
