@@ -2,11 +2,13 @@
 """Headline benchmark: OIL4 decode GEMV at the Llama-7B up/gate projection shape
 (K = 4096 -> N = 11008, M = 1, FP32 activations), one MI355X.
 
-A "step" is one GEMV launch over one resident OIL4 weight matrix.  Because one
-matrix (22.5 MB) fits the 256 MB Infinity Cache, steps walk a ring of distinct
-device copies (> 800 MB in total) so every launch streams its weights from
-HBM; the ring is replayed through a HIP graph so the host launch path is not
-what is being timed.  `value` is payload bytes / time (effective weight GB/s).
+A "step" is one pass of the GEMV over a ring of 40 resident copies of the OIL4
+weight matrix (40 launches, 902 MB streamed): one matrix (22.5 MB) fits the
+256 MB Infinity Cache, so every launch of a step reads a copy that the cache
+no longer holds.  A step is one replay of a HIP graph, so nothing but graph
+replays sits inside the timed region; K steps make a round and rounds repeat
+until the region is at least 50 ms long.  `ms_per_step` is per step (40
+launches); `value` and `roofline` are per launch: payload bytes / time.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
 """
@@ -23,9 +25,9 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E, published
 ROWS, COLS = 11008, 4096       # W is [N rows][K cols]: y = W x
 RING = 40                      # distinct weight copies: 40 x 22.5 MB = 902 MB > 256 MB cache
-# HBM bytes per GEMV launch from rocprofv3 counters (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB, factors
-# from a plain 1 GiB copy); measured once per kernel version, see profiles/oil4_gemv_4096x11008_m1.md
-HBM_TRAFFIC_BYTES_PER_LAUNCH = 22908314
+# HBM bytes per GEMV launch, cited from the rocprofv3 counter runs summarised in profiles/oil4_gemv_4096x11008_m1.md
+# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from a plain 1 GiB copy); not measured in this run
+HBM_TRAFFIC_BYTES_PER_LAUNCH = 22881894
 
 
 def log(*a):
@@ -50,21 +52,26 @@ class Ring:
             d.close()
 
 
-def time_ring(torch, ring, x, y, steps, warmup, settle_s=0.0):
-    """Average seconds per GEMV launch over `steps` launches (graph replay of the ring).  settle_s: untimed replays for
-    that long in front of the timed region, so that a device that comes out of idle has reached its steady clocks."""
+def time_ring(torch, ring, x, y, steps, warmup, settle_s=0.0, min_region_s=0.05):
+    """One step = one replay of a HIP graph that holds one GEMV launch per ring copy (`len(ring.items)` launches).
+    Nothing but graph replays sits between the two events: `steps` replays make one round, and rounds are repeated
+    until the timed region is at least `min_region_s` long.  Returns (seconds per launch, host seconds per launch,
+    rounds, seconds of the timed region).  settle_s: untimed replays for that long in front of the timed region, so
+    that a device that comes out of idle has reached its steady clocks."""
     n = len(ring.items)
-    for i in range(max(warmup, n)):                    # untimed warm-up (also first-call setup)
-        ring.items[i % n].gemv(x, out=y)
-    torch.cuda.synchronize()
     stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):                    # untimed warm-up passes, on the stream that is captured below:
+        for i in range(max(warmup, 1)):                # first-call set-up, and scratch that belongs to the stream
+            for d in ring.items:
+                d.gemv(x, out=y)
+    torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(stream):
         with torch.cuda.graph(graph, stream=stream):
             for d in ring.items:
                 d.gemv(x, out=y)
     torch.cuda.synchronize()
-    reps, tail = divmod(steps, n)
     with torch.cuda.stream(stream):
         graph.replay()
         torch.cuda.synchronize()
@@ -73,20 +80,28 @@ def time_ring(torch, ring, x, y, steps, warmup, settle_s=0.0):
             for _ in range(8):
                 graph.replay()
             torch.cuda.synchronize()
+        # a short untimed probe sizes the number of rounds
+        p0, p1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        p0.record(stream)
+        for _ in range(4):
+            graph.replay()
+        p1.record(stream)
+        torch.cuda.synchronize()
+        est = max(p0.elapsed_time(p1) * 1e-3 / 4, 1e-7)                 # seconds per replay
+        rounds = max(1, int(-(-min_region_s // (est * steps))))
         e0 = torch.cuda.Event(enable_timing=True)
         e1 = torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record(stream)
-        for _ in range(reps):
+        for _ in range(rounds * steps):
             graph.replay()
-        for i in range(tail):
-            ring.items[i].gemv(x, out=y)
         e1.record(stream)
         torch.cuda.synchronize()
         wall = time.perf_counter() - t0
     dev = e0.elapsed_time(e1) * 1e-3
-    return dev / steps, wall / steps
+    launches = rounds * steps * n
+    return dev / launches, wall / launches, rounds, dev
 
 
 def cpu_baseline(payload, blocks, rows, cols, x):
@@ -219,7 +234,7 @@ def bench_tall(torch, ia):
         ring = Ring(ia, payload, blocks, rows, COLS, copies)
         x = torch.randn(1, COLS, device="cuda")
         y = torch.empty((1, rows), dtype=torch.float32, device="cuda")
-        s_t, _ = time_ring(torch, ring, x, y, 40 * copies, copies)
+        s_t = time_ring(torch, ring, x, y, 4, 1)[0]
         out[f"{label}_M1_us"] = round(s_t * 1e6, 2)
         out[f"{label}_M1_GBps"] = round(ring.payload_bytes / s_t / 1e9, 1)
         ring.close()
@@ -238,7 +253,7 @@ def bench_oil8(torch, ia):
     ring = Ring(ia, p8, b8, 4096, 4096, 56)
     x = torch.randn(1, 4096, device="cuda")
     y = torch.empty((1, 4096), dtype=torch.float32, device="cuda")
-    t, _ = time_ring(torch, ring, x, y, 1120, 56)
+    t = time_ring(torch, ring, x, y, 4, 1)[0]
     ring.close()
     out = {"oil8_block_4096x4096_M1_GBps": round(p8.size / t / 1e9, 1), "oil8_block_4096x4096_M1_us": round(t * 1e6, 2)}
     idx = [torch.randint(0, 256, (4096 * 4096,), dtype=torch.uint8, device="cuda") for _ in range(56)]
@@ -579,8 +594,8 @@ def bench_moe(torch, ia):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=4000)
-    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=100, help="timed steps per round (a step = one replay of the 40-launch ring)")
+    ap.add_argument("--warmup", type=int, default=5, help="untimed warm-up steps")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--kv-only", action="store_true", help="only run the KV-cache leg (for profiling its kernels)")
@@ -620,7 +635,7 @@ def main():
     x = torch.from_numpy(xh).cuda()
     y = torch.empty((1, ROWS), dtype=torch.float32, device="cuda")
 
-    sec, wall = time_ring(torch, ring, x, y, args.steps, args.warmup, settle_s=0.3)
+    sec, wall, rounds, region_s = time_ring(torch, ring, x, y, args.steps, args.warmup, settle_s=0.3)
     algo_bytes = ring.payload_bytes + 4 * COLS + 4 * ROWS          # weights + x + y, each once
     value = ring.payload_bytes / sec / 1e9
     achieved = algo_bytes / sec / 1e9
@@ -634,7 +649,7 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
-        "ms_per_step": round(sec * 1e3, 6),
+        "ms_per_step": round(sec * RING * 1e3, 6),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -642,12 +657,15 @@ def main():
         "data": "synthetic",
         "config": {"workload": "OIL4 decode GEMV, Llama-7B up/gate projection K=4096 -> N=11008, M=1, "
                                "FP32 activations ~N(0,1), weights ~N(0,0.02) quantized to OIL4 wire blocks",
-                   "rows": ROWS, "cols": COLS, "M": 1, "ring_copies": RING,
-                   "payload_bytes": ring.payload_bytes},
+                   "rows": ROWS, "cols": COLS, "M": 1, "ring_copies": RING, "launches_per_step": RING,
+                   "payload_bytes": ring.payload_bytes, "timed_rounds": rounds, "timed_launches": rounds * args.steps * RING,
+                   "timed_region_ms": round(region_s * 1e3, 3)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic},
+                     "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                     "traffic_source": "cited from profiles/oil4_gemv_4096x11008_m1.md (rocprofv3 --pmc), not measured in this run",
+                     "us_per_launch": round(sec * 1e6, 3)},
         "pct_of_hbm_peak": round(100.0 * value / HBM_PEAK_GBS, 2),
-        "host_wall_ms_per_step": round(wall * 1e3, 6),
+        "host_wall_ms_per_step": round(wall * RING * 1e3, 6),
     }
 
     if not args.no_extra:
@@ -655,7 +673,7 @@ def main():
         for M in (4, 16, 32):
             xm = torch.randn(M, COLS, device="cuda")
             ym = torch.empty((M, ROWS), dtype=torch.float32, device="cuda")
-            s_m, _ = time_ring(torch, ring, xm, ym, 400, 40)
+            s_m = time_ring(torch, ring, xm, ym, 4, 1)[0]
             extra[f"up_gate_M{M}_GBps"] = round(ring.payload_bytes / s_m / 1e9, 1)
         ring.close()
         # down projection K = 11008 -> N = 4096
@@ -664,12 +682,12 @@ def main():
         ring_d = Ring(ia, pd, bd, COLS, ROWS, RING)
         xd = torch.randn(1, ROWS, device="cuda")
         yd = torch.empty((1, COLS), dtype=torch.float32, device="cuda")
-        s_d, _ = time_ring(torch, ring_d, xd, yd, 2000, 100)
+        s_d = time_ring(torch, ring_d, xd, yd, 4, 1)[0]
         extra["down_M1_GBps"] = round(ring_d.payload_bytes / s_d / 1e9, 1)
         for M in (4, 16):
             xm = torch.randn(M, ROWS, device="cuda")
             ym = torch.empty((M, COLS), dtype=torch.float32, device="cuda")
-            s_m, _ = time_ring(torch, ring_d, xm, ym, 400, 40)
+            s_m = time_ring(torch, ring_d, xm, ym, 4, 1)[0]
             extra[f"down_M{M}_GBps"] = round(ring_d.payload_bytes / s_m / 1e9, 1)
         ring_d.close()
         # weights-only decode rate of a Llama-7B-shaped stack: per layer 4 x (4096x4096), 2 x up/gate, 1 x down
@@ -679,7 +697,7 @@ def main():
         ring_q = Ring(ia, pq, bq, 4096, 4096, 64)
         xq = torch.randn(1, 4096, device="cuda")
         yq = torch.empty((1, 4096), dtype=torch.float32, device="cuda")
-        t_qkvo, _ = time_ring(torch, ring_q, xq, yq, 2048, 128)
+        t_qkvo = time_ring(torch, ring_q, xq, yq, 4, 1)[0]
         ring_q.close()
         per_layer = 4 * t_qkvo + 2 * sec + s_d
         extra["qkvo_4096x4096_M1_GBps"] = round(pq.size / t_qkvo / 1e9, 1)

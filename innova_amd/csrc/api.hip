@@ -4,6 +4,8 @@
 #include <mutex>
 #include <new>
 #include <algorithm>
+#include <map>
+#include <tuple>
 #include <vector>
 
 #include "common.h"
@@ -62,7 +64,44 @@ int device_cu_count() {
     return g_cus[dev];
 }
 
-static int check_matmul_shape(const oilhip_weights* w, const void* x, const void* y, int M) {
+int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    const uint64_t bit = 1ull << (dev & 63);
+    if (done.load(std::memory_order_acquire) & bit) return OILHIP_OK;
+    OILHIP_HIP(hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes));
+    done.fetch_or(bit, std::memory_order_release);
+    return OILHIP_OK;
+}
+
+static std::mutex g_scratch_mu;
+static std::map<std::tuple<int, void*, int>, std::pair<void*, size_t>> g_scratch;
+
+int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    auto& e = g_scratch[std::make_tuple(dev, (void*)s, slot)];
+    if (e.second < bytes) {
+        hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return fail(OILHIP_E_ARG, "this call needs " + std::to_string(bytes) + " bytes of device scratch on its stream and cannot "
+                        "allocate them during stream capture: make the same call once on this stream outside capture first");
+        }
+        const size_t want = bytes > 2 * e.second ? bytes : 2 * e.second;
+        void* p = nullptr;
+        if (hipMalloc(&p, want) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(OILHIP_E_NOMEM, "hipMalloc of " + std::to_string(want) + " bytes of scratch failed");
+        }
+        e = {p, want};                       // the smaller buffer stays allocated (see common.h)
+    }
+    *out = e.first;
+    return OILHIP_OK;
+}
+
+int check_matmul_shape(const oilhip_weights* w, const void* x, const void* y, int M) {
     if (!w || !x || !y) return fail(OILHIP_E_ARG, "null argument");
     if (M < 1) return fail(OILHIP_E_ARG, "M must be >= 1");
     if (!w->all_full || (w->cols % 256) != 0 || w->cols == 0 || w->rows == 0)
@@ -125,6 +164,9 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
         const int s = slot_of[d.fmt];
         if (!seen[s]) {
             seen[s] = true;
+            // the stream kernel decodes blocks of the size the quantizer writes; other channel sizes stay with the
+            // kernels that follow the descriptors weight by weight
+            if (d.cb_bytes != full_block_cb_bytes(d.fmt) || d.cb_bytes + d.idx_bytes != full_block_bytes(d.fmt)) return;
             g.cb_bytes[s] = d.cb_bytes;
             g.idx_bytes[s] = d.idx_bytes;
             g.stride[s] = ((uint32_t)d.cb_bytes + d.idx_bytes + 15u) & ~15u;
@@ -235,11 +277,12 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
 static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vector<uint64_t>& out_off,
                   uint64_t algo_bytes, uint64_t rows, uint64_t cols, oilhip_weights** out) {
     const uint32_t nblocks = (uint32_t)db.size();
-    bool all_full = true, uniform = true, regular = nblocks > 0;
+    bool all_full = true, uniform = true, regular = nblocks > 0, nominal = true;
     uint64_t total_nw = 0;
     for (uint32_t b = 0; b < nblocks; ++b) {
         total_nw += db[b].nw;
         all_full &= db[b].nw == 256;
+        nominal &= db[b].cb_bytes == full_block_cb_bytes(db[b].fmt) && (uint32_t)db[b].cb_bytes + db[b].idx_bytes == full_block_bytes(db[b].fmt);
         uniform &= db[b].fmt == db[0].fmt;
         if (b > 0) regular &= (db[b].off16 - db[b - 1].off16) == (db[1].off16 - db[0].off16) &&
                               db[b].idx_bytes == db[0].idx_bytes && db[b].cb_bytes == db[0].cb_bytes;
@@ -255,7 +298,9 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
     if ((e = hipGetDevice(&w->device)) != hipSuccess) return bail(e, "hipGetDevice");
     // window streams for every tensor of full blocks but the uniform OIL4 and OIL8 ones, which have kernels of their own
     // that read the blocks back to back
-    const bool own_kernel = uniform && regular && nblocks && (db[0].fmt == OILHIP_OIL4 || db[0].fmt == OILHIP_OIL8);
+    const bool own_kernel = uniform && regular && nblocks && db[0].cb_bytes == 0 && db[0].off16 == 0 &&
+                            ((db[0].fmt == OILHIP_OIL4 && db[0].idx_bytes == 128) || (db[0].fmt == OILHIP_OIL8 && db[0].idx_bytes == 256)) &&
+                            (nblocks == 1 || (db[1].off16 - db[0].off16) * 16u == db[0].idx_bytes);
     if (all_full && nblocks && !own_kernel) pack_window_streams(pay, db, rows, cols, w->seg);
     if (w->seg.nstreams) regular = false;
     // 64 spare bytes so vector loads that straddle the end of the last block stay in bounds
@@ -280,6 +325,7 @@ static int upload(std::vector<uint8_t>& pay, std::vector<DevBlock>& db, std::vec
     w->nblocks = nblocks;
     w->uniform_fmt = (uniform && nblocks) ? db[0].fmt : -1;
     w->all_full = all_full && nblocks > 0;
+    w->nominal = w->all_full && nominal;
     if (regular && uniform && nblocks)
         w->uniform_stride = nblocks > 1 ? (db[1].off16 - db[0].off16) * 16u
                                         : (uint32_t)((db[0].cb_bytes + db[0].idx_bytes + 15u) & ~15u);
@@ -424,7 +470,7 @@ int oilhip_weights_stack_rows(const oilhip_weights* const* parts, int n, oilhip_
         return bail(e, "hipMemcpy(blocks)");
     w->payload_bytes = algo;
     w->rows = rows; w->cols = p0->cols; w->nblocks = (uint32_t)nblocks;
-    w->uniform_fmt = p0->uniform_fmt; w->all_full = true;
+    w->uniform_fmt = p0->uniform_fmt; w->all_full = true; w->nominal = p0->nominal;
     w->uniform_stride = p0->uniform_stride; w->uniform_cb = p0->uniform_cb; w->uniform_idx = p0->uniform_idx; w->uniform_base = 0;
     *out = w;
     return OILHIP_OK;
@@ -455,7 +501,7 @@ int oilhip_dequant_f32(const oilhip_weights* w, float* d_out, void* stream) {
 
 int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
     if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
-    if (w->uniform_fmt == OILHIP_OIL4 && w->uniform_stride == 128) {
+    if (plain_oil4(*w)) {
         // one or two rows: the register-resident kernel; from three on the matrix-core kernel (16 rows per pass) is faster
         int rc = 1;                                                                          // 1: shape not covered
         if (M <= 2) rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
@@ -465,7 +511,7 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
         if (rc == 1 && M > 2 && M <= 4) rc = launch_gemv_oil4(*w, d_x, d_y, M, (hipStream_t)stream);
         if (rc <= 0) return rc;
     }
-    if (w->uniform_fmt == OILHIP_OIL8 && w->uniform_stride == 256) {
+    if (plain_oil8(*w)) {
         // the register-resident kernel takes up to four activation rows per launch
         int rc = 1;
         for (int m0 = 0; m0 < M; m0 += 4) {
@@ -493,7 +539,7 @@ int oilhip_gemv_f32_general(const oilhip_weights* w, const float* d_x, float* d_
 
 int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x, float* d_y, int M, void* stream) {
     if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
-    if (w->uniform_fmt != OILHIP_OIL4 || w->uniform_stride != 128)
+    if (!plain_oil4(*w))
         return fail(OILHIP_E_ARG, "bf16 prefill GEMM is implemented for uniform OIL4 tensors");
     return launch_gemm_oil4_bf16(*w, d_x, d_y, M, (hipStream_t)stream);
 }

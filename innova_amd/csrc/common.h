@@ -3,12 +3,21 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
 #include <string>
 
 #include "../../include/oilhip.h"
 #include "block_decode.h"
 
 namespace oilhip {
+
+// bytes of a full 256-weight block of each format (codebook channel + index channel) and of its codebook channel,
+// as quantize_block_all writes them (src/block_codec.cpp:368-574)
+__host__ __device__ constexpr uint32_t full_block_bytes(int f) {
+    constexpr uint32_t n[15] = {16, 48, 64, 128, 256, 512, 1024, 32, 48, 80, 144, 272, 512, 64, 64};
+    return f >= 0 && f < 15 ? n[f] : 0u;
+}
+__host__ __device__ constexpr uint32_t full_block_cb_bytes(int f) { return f == 0 ? 16u : 0u; }
 
 // Thread-local text behind oilhip_last_error().
 void set_error(const std::string& msg);
@@ -24,6 +33,20 @@ int fail(int code, const std::string& msg);
 // Per-device decode tables (device pointer), created on first use.
 int get_tables(const DecodeTables** out);
 int device_cu_count();
+// shape rules shared by every matmul entry point: non-null pointers, M >= 1, full blocks, cols a multiple of 256
+int check_matmul_shape(const oilhip_weights* w, const void* x, const void* y, int M);
+
+// Raises a kernel's dynamic LDS limit once per device.  `done` is the call site's own flag word (one bit per device);
+// concurrent first calls may both set the attribute, which is harmless.
+int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes);
+
+// Device scratch of at least `bytes` that belongs to (current device, stream, slot): kernels queued on one stream run
+// in order, so calls on different streams never share a buffer.  A buffer is never freed or moved while the process
+// lives (a captured graph or a queued kernel may still point at it): a request that outgrows it gets a new, larger
+// one and the old one stays allocated.  No allocation can happen while the stream is being captured, so the first
+// call of a given size on a stream has to be made outside capture; otherwise the call fails with OILHIP_E_ARG.
+enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1 };
+int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
 // Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream
 // (gemv_seg.hip).  The first window of stream s sits at byte s * stream_bytes of the payload buffer, the later ones
@@ -61,9 +84,20 @@ struct oilhip_weights {
     uint32_t uniform_cb = 0, uniform_idx = 0;   // channel sizes of every block when regular
     uint32_t uniform_base = 0;              // byte offset of block 0 when regular
     bool all_full = false;                  // every block holds exactly 256 weights
+    bool nominal = false;                   // ... and has the channel sizes the quantizer writes for its format
 };
 
 namespace oilhip {
+// Uniform OIL4 / OIL8 tensors in the plain layout the specialised kernels read: every block's bytes in the index
+// channel, blocks back to back from byte 0.  Anything else (a non-empty codebook channel, padding between blocks)
+// goes through the kernels that follow the descriptors.
+inline bool plain_oil4(const oilhip_weights& w) {
+    return w.uniform_fmt == OILHIP_OIL4 && w.uniform_stride == 128 && w.uniform_cb == 0 && w.uniform_idx == 128 && w.uniform_base == 0;
+}
+inline bool plain_oil8(const oilhip_weights& w) {
+    return w.uniform_fmt == OILHIP_OIL8 && w.uniform_stride == 256 && w.uniform_cb == 0 && w.uniform_idx == 256 && w.uniform_base == 0;
+}
+
 // kernels (each returns an OILHIP_* code and sets the error text)
 int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
 int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
@@ -79,7 +113,10 @@ int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_ac
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2 = nullptr,
-                           float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr);
+                           float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr, uint32_t* d_pack = nullptr);
+// widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
+constexpr uint32_t kGemvPackMaxCols = 32768;
+constexpr size_t kGemvPackBytes = (size_t)(kGemvPackMaxCols >> 8) * 128u * 128u * 2u;
 // rows that mix formats, stored tile by tile and format by format
 int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // every format, a lane per run of 32 weights

@@ -20,8 +20,6 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
-#include <cstdlib>
-#include <mutex>
 
 #include "common.h"
 
@@ -372,40 +370,14 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
         }
 }
 
-// grow-only device scratch for X' (one per process and device; calls that overlap on one device race on it)
-std::mutex g_scratch_mu;
-uint16_t* g_scratch[64] = {};
-size_t g_scratch_bytes[64] = {};
-
-int get_scratch(size_t bytes, uint16_t** out) {
-    int dev = 0;
-    OILHIP_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
-    std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (g_scratch_bytes[dev] < bytes) {
-        if (g_scratch[dev]) {
-            OILHIP_HIP(hipDeviceSynchronize());
-            OILHIP_HIP(hipFree(g_scratch[dev]));
-            g_scratch[dev] = nullptr;
-            g_scratch_bytes[dev] = 0;
-        }
-        OILHIP_HIP(hipMalloc(&g_scratch[dev], bytes));
-        g_scratch_bytes[dev] = bytes;
-    }
-    *out = g_scratch[dev];
-    return OILHIP_OK;
-}
 
 template <int WBM, int WBN>
 int launch(const oilhip_weights& w, const uint16_t* xp, float* d_y, uint32_t M, uint32_t Mpad, hipStream_t s) {
     constexpr int BM = 64 * WBM, BN = 64 * WBN;
     const size_t lds_bytes = (size_t)kTabBytes + (size_t)(BM + BN) * LDK * 2;
-    static bool attr_done = false;
+    static std::atomic<uint64_t> attr_done{0};
     auto kern = gemm_oil4_bf16_kernel<WBM, WBN>;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done = true;
-    }
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
     const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols;
     hipLaunchKernelGGL(kern, dim3((N + BN - 1) / BN, Mpad / BM), dim3(256), lds_bytes, s, w.d_payload, xp, d_y, M, N, K, Mpad);
     OILHIP_HIP(hipGetLastError());
@@ -417,24 +389,18 @@ int launch(const oilhip_weights& w, const uint16_t* xp, float* d_y, uint32_t M, 
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
     const uint32_t K = (uint32_t)w.cols;
-    static const int tile = [] { const char* e = getenv("OILHIP_GEMM_TILE"); return e ? atoi(e) : 0; }();
-    const bool big = tile ? tile == 256 : M > 256;
+    const bool big = M > 256;
     const uint32_t BM = big ? 256 : 128;
     const uint32_t Mpad = ((uint32_t)M + BM - 1) / BM * BM;
     uint16_t* xp = nullptr;
-    if (int rc = get_scratch((size_t)Mpad * K * 2, &xp)) return rc;
+    if (int rc = stream_scratch(s, kScratchGemmX, (size_t)Mpad * K * 2, reinterpret_cast<void**>(&xp))) return rc;
     uint32_t gx = (K + 255) / 256;
     if (gx > 64) gx = 64;
     hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
     OILHIP_HIP(hipGetLastError());
-    static const int pipe = [] { const char* e = getenv("OILHIP_GEMM_PIPE"); return e ? atoi(e) : 1; }();
-    if (big && pipe) {
-        static bool attr_done = false;
-        if (!attr_done) {
-            OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-            attr_done = true;
-        }
+    if (big) {
+        static std::atomic<uint64_t> attr_done{0};
+        if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel), 160 * 1024)) return rc;
         const uint32_t N = (uint32_t)w.rows;
         const size_t lds_bytes = (size_t)kTabBytes + 2ull * (PBM + PBN) * PLD * 2;
         // a grid that leaves half of the compute units idle is cut in two along K (two partial sums into a zeroed Y)
@@ -449,7 +415,7 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
         OILHIP_HIP(hipGetLastError());
         return OILHIP_OK;
     }
-    return big ? launch<4, 4>(w, xp, d_y, (uint32_t)M, Mpad, s) : launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
+    return launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
 }
 
 }  // namespace oilhip

@@ -23,7 +23,6 @@
 // instructions per row.
 #include <hip/hip_fp16.h>
 
-#include <cstdlib>
 
 #include "common.h"
 #include "oil4_lds.h"
@@ -32,6 +31,12 @@
 #define OILHIP_PFA 3
 #define OILHIP_PFB 6
 #define OILHIP_PFC 6
+#endif
+#ifndef OILHIP_OIL4_WGT
+#define OILHIP_OIL4_WGT 512      // threads per workgroup of the decode kernel (512 or 1024)
+#endif
+#ifndef OILHIP_OIL4_AUX
+#define OILHIP_OIL4_AUX 0        // cache policy of the weight loads: 2 = nt (streamed once, not kept in L2 / the Infinity Cache)
 #endif
 
 namespace oilhip {
@@ -51,11 +56,12 @@ constexpr int kXsBlock = 288;  // floats per block in the LDS copy of x: 256 + 3
 // XF = 3: not a block tensor but rows of cols/2 bytes of packed codes (low nibble first) with a 16-entry FP16 codebook
 // passed through xw and one scale for the whole matrix (gemv_oil4 of src/kernel_production.cpp): x stays in natural
 // order, the pair table is built from the codebook, there is no block scale and y is multiplied by out_scale.
-template <int CS, int RPW, int MB, int MAXT, int XF = 0, bool ROLL = false>
-__global__ void __launch_bounds__(MAXT) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <int CS, int RPW, int MB, int WGT, int XF = 0, bool ROLL = false>
+__global__ void __launch_bounds__(WGT) __attribute__((amdgpu_waves_per_eu(WGT / 256, WGT / 256)))
 gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, const float* __restrict__ xw, float* __restrict__ y,
                  uint32_t rows, uint32_t cols, uint32_t S, uint32_t G, uint32_t nchunks, int m0, int M,
-                 uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups, float out_scale) {
+                 uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups_lo, uint32_t wave_groups_hi, float out_scale) {
+    constexpr uint32_t NW = WGT / 64;   // wavefronts per workgroup
     constexpr int NL = CS * RPW;      // wave-loads per chunk
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
@@ -66,7 +72,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));      // uniform: scalar registers
-    const uint32_t grp = (wave_groups >> (4u * wave)) & 15u, slab = wave - grp * S;         // wave / S, wave % S
+    const uint32_t grp = ((wave < 8u ? wave_groups_lo : wave_groups_hi) >> (4u * (wave & 7u))) & 15u, slab = wave - grp * S;   // wave / S, wave % S
     const uint32_t bpr = cols >> 8;
     const uint32_t lp = lane & 7u;
 
@@ -84,7 +90,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     // ---- x first (needed soonest), then every weight load of the first chunk ----------
     // Nothing that waits on vector memory may follow the weight loads before their use:
     // loads return in order, so it would wait for every weight byte.
-    constexpr int XPT = 4;            // float4 pieces of x fetched up front per thread
+    constexpr int XPT = 2048 / WGT;   // float4 pieces of x fetched up front per thread
     constexpr uint32_t XW = XF == 1 ? 2u : 1u;                                // input floats per activation
     const __amdgpu_buffer_rsrc_t nrsrc = __builtin_amdgcn_make_buffer_rsrc((void*)(XF == 2 ? xw : x), 0, (int)(cols * 4u), 0x00020000);
     const __amdgpu_buffer_rsrc_t xrsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -92,7 +98,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     u32x4 xpre[MB][XPT], xup[XF ? MB : 1][XF ? XPT : 1];
 #pragma unroll
     for (int u = 0; u < XPT; ++u) {
-        const uint32_t d4 = tid + u * 512u;                             // float4 index into the padded row
+        const uint32_t d4 = tid + u * (uint32_t)WGT;                    // float4 index into the padded row
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             const uint32_t off = (d4 * 4u < cols && m0 + m < M) ? d4 * 16u + m * cols * XW * 4u : kOobOffset;
@@ -151,12 +157,12 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     u32x4 wv[NL];
     auto issue_load = [&](int n, uint32_t rel) {           // rel: first row of the chunk, counted from r0
         const int it = n / CS, cs = n % CS;
-        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, 0);
+        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, OILHIP_OIL4_AUX);
     };
     // The 64 KB pair table is written while the weight loads queue up: float4 number e of the
-    // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + 512*k,
-    // k = 0..7, so its low nibble (tid >> 4) & 15 is fixed and its high nibble is (tid >> 8) + 2k,
-    // uniform across the wavefront.  Levels come from literals: no memory access, no barrier.
+    // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + WGT*k,
+    // k = 0 .. 4096/WGT - 1, so its low nibble (tid >> 4) & 15 is fixed and its high nibble is
+    // (tid >> 8) + (WGT/256) k, uniform across the wavefront.  Levels come from literals: no memory access, no barrier.
     // A wave-load takes the address unit of the CU a good dozen cycles and eight wavefronts queue there, so the
     // table writes are slotted in between the loads instead of after them.
     issue_load(0, 0u);
@@ -173,15 +179,16 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         lv_lane = level_literal(lane & 15u);
         lo_fix = level_literal((tid >> 4) & 15u);
     }
+    constexpr int TK = 4096 / WGT;                                            // table writes per thread
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
+    for (int k = 0; k < TK; ++k) {
         if (k + 1 < PFA) issue_load(k + 1, 0u);
-        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((wave >> 2) + 2u * k)));
-        reinterpret_cast<float4*>(tab)[tid + 512u * k] = make_float4(lo_fix, hi, lo_fix, hi);
+        const float hi = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(lv_lane), (int)((wave >> 2) + (uint32_t)(WGT / 256) * k)));
+        reinterpret_cast<float4*>(tab)[tid + (uint32_t)WGT * k] = make_float4(lo_fix, hi, lo_fix, hi);
         __builtin_amdgcn_sched_barrier(0);
     }
 #pragma unroll
-    for (int n = (PFA < 9 ? PFA : 9); n < PFB; ++n) issue_load(n, 0u);
+    for (int n = (PFA < TK + 1 ? PFA : TK + 1); n < PFB; ++n) issue_load(n, 0u);
     __builtin_amdgcn_sched_barrier(0);
 
     // ---- x into LDS in nibble order -------------------------------------------------------------
@@ -209,24 +216,24 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         dst[xoff[2]] = __uint_as_float(v.z);
         if (xlast_ok) dst[xoff[3]] = __uint_as_float(v.w);
     };
-    for (uint32_t bz = tid; XF != 3 && bz < nblk * MB; bz += 512u) {          // scale nibbles of every block
+    for (uint32_t bz = tid; XF != 3 && bz < nblk * MB; bz += (uint32_t)WGT) { // scale nibbles of every block
         const uint32_t m = bz / nblk, b = bz % nblk;
         *reinterpret_cast<float4*>(xs + (size_t)m * xstride + b * kXsBlock) = make_float4(0.f, 0.f, 0.f, 0.f);
     }
-    for (uint32_t z = bpr * 64u + tid; z < nblk * 64u; z += 512u) {           // blocks past the end of the row
+    for (uint32_t z = bpr * 64u + tid; z < nblk * 64u; z += (uint32_t)WGT) {  // blocks past the end of the row
 #pragma unroll
         for (int m = 0; m < MB; ++m)
             reinterpret_cast<float4*>(xs + (size_t)m * xstride + (z >> 6) * kXsBlock)[z & 63u] = make_float4(0.f, 0.f, 0.f, 0.f);
     }
 #pragma unroll
     for (int u = 0; u < XPT; ++u) {
-        const uint32_t d4 = tid + u * 512u;
+        const uint32_t d4 = tid + u * (uint32_t)WGT;
         if (d4 * 4u < cols) {
 #pragma unroll
             for (int m = 0; m < MB; ++m) scatter4(d4, transform4(xpre[m][u], xup[XF ? m : 0][XF ? u : 0]), m);
         }
     }
-    for (uint32_t d4 = tid + XPT * 512u; d4 * 4u < cols; d4 += 512u) {    // rows wider than XPT*4*workgroup
+    for (uint32_t d4 = tid + XPT * (uint32_t)WGT; d4 * 4u < cols; d4 += (uint32_t)WGT) {    // rows wider than XPT*4*workgroup
 #pragma unroll
         for (int m = 0; m < MB; ++m) {
             const uint32_t off = (m0 + m < M) ? d4 * 16u + m * cols * XW * 4u : kOobOffset;
@@ -238,7 +245,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     }
 #pragma unroll
     for (int n = PFB; n < PFC; ++n) issue_load(n, 0u);
-    float* ssq_part = red + (size_t)G * RPW * MB * S;                         // 8 floats past the slab partials
+    float* ssq_part = red + (size_t)G * RPW * MB * S;                         // one float per wavefront past the slab partials
     if (XF == 2) {
         float v = ssq;
         v += dpp_quad_xor1(v);
@@ -252,7 +259,9 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     __syncthreads();
     float yscale = XF == 3 ? out_scale : 1.0f;
     if (XF == 2) {
-        const float tot = ((ssq_part[0] + ssq_part[1]) + (ssq_part[2] + ssq_part[3])) + ((ssq_part[4] + ssq_part[5]) + (ssq_part[6] + ssq_part[7]));
+        float tot = 0.0f;
+#pragma unroll
+        for (uint32_t q = 0; q < NW; q += 4) tot += (ssq_part[q] + ssq_part[q + 1]) + (ssq_part[q + 2] + ssq_part[q + 3]);
         yscale = 1.0f / sqrtf(tot / (float)cols + 1e-6f);
     }
 
@@ -355,7 +364,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         }
         __syncthreads();
         // ---- slab partials -> y -------------------------------------------------
-        for (uint32_t o = tid; o < G * RPW * MB; o += 512u) {
+        for (uint32_t o = tid; o < G * RPW * MB; o += (uint32_t)WGT) {
             const uint32_t g2 = o / (RPW * MB), rem = o % (RPW * MB), slot = rem / MB, m = rem % MB;
             const uint32_t jg2 = blockIdx.x * G + g2;
             const uint32_t q0 = group_begin(jg2), q1 = group_begin(jg2 + 1);
@@ -371,6 +380,8 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     }
 }
 
+constexpr int kWgt = OILHIP_OIL4_WGT;
+
 // One launch configuration of the kernel above.
 struct Oil4Plan {
     int cs, rpw, maxt;     // template choice
@@ -378,23 +389,19 @@ struct Oil4Plan {
     size_t lds_bytes;
 };
 
-template <int CS, int RPW, int MB, int MAXT, int XF, bool ROLL>
+template <int CS, int RPW, int MB, int WGT, int XF, bool ROLL>
 int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, int M, hipStream_t s, const Oil4Plan& p,
            float out_scale = 1.0f) {
-    static bool attr_done = false;
-    auto kern = gemv_oil4_kernel<CS, RPW, MB, MAXT, XF, ROLL>;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        attr_done = true;
-    }
+    static std::atomic<uint64_t> attr_done{0};
+    auto kern = gemv_oil4_kernel<CS, RPW, MB, WGT, XF, ROLL>;
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), kMaxLds)) return rc;
     const uint32_t J = p.grid * p.G;
-    uint32_t wave_groups = 0;                                   // wave / S for each of the 8 wavefronts, 4 bits each
-    for (uint32_t wv = 0; wv < 8; ++wv) wave_groups |= (wv / p.S) << (4u * wv);
+    uint64_t wave_groups = 0;                                   // wave / S for each of the wavefronts, 4 bits each
+    for (uint32_t wv = 0; wv < (uint32_t)WGT / 64u; ++wv) wave_groups |= (uint64_t)(wv / p.S) << (4u * wv);
     for (int m0 = 0; m0 < M; m0 += MB) {
-        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(512), p.lds_bytes, s, w.d_payload, d_x, d_xw, d_y,
+        hipLaunchKernelGGL(kern, dim3(p.grid), dim3(WGT), p.lds_bytes, s, w.d_payload, d_x, d_xw, d_y,
                            (uint32_t)w.rows, (uint32_t)w.cols, p.S, p.G, p.nchunks, m0, M,
-                           (uint32_t)w.rows / J, (uint32_t)w.rows % J, wave_groups, out_scale);
+                           (uint32_t)w.rows / J, (uint32_t)w.rows % J, (uint32_t)wave_groups, (uint32_t)(wave_groups >> 32), out_scale);
         OILHIP_HIP(hipGetLastError());
     }
     return OILHIP_OK;
@@ -403,7 +410,8 @@ int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* 
 // Chooses column sets per wave, slabs, waves per workgroup and chunking for a shape.
 bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan* p) {
     const uint32_t sets = ((cols >> 8) + 7) / 8;                  // column sets (1 KB wave-loads) per row
-    const int cs_max = MB == 1 ? 3 : 1;                           // register budget: 32*CS*MB activations per lane
+    // register budget: 32*CS*MB activations per lane, out of 256 registers (two wavefronts per SIMD) or 128 (four)
+    const int cs_max = MB == 1 ? (kWgt == 1024 ? 2 : 3) : 1;
     // fewest slabs first (less cross-wave reduction), then least padding
     int best_cs = 1; uint32_t best_S = sets; double best_cost = 1e30;
     for (int cs = 1; cs <= cs_max; ++cs) {
@@ -422,7 +430,7 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     if (grid == 0) grid = 1;
     const uint32_t Jn = grid * G;
     const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
-    const int budget = 12 / best_cs;                               // wave-loads in flight per wave (register budget)
+    const int budget = (kWgt == 1024 ? 6 : 12) / best_cs;          // wave-loads in flight per wave (register budget)
     int rpw = 1;
     if (max_rows <= (uint32_t)budget) {                            // one chunk: the smallest that holds every row
         for (int cand : {1, 2, 3, 4, 6, 12}) if ((uint32_t)cand >= max_rows) { rpw = cand; break; }
@@ -436,13 +444,13 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
             if (slots < best_slots) { best_slots = slots; rpw = cand; }
         }
     }
-    p->cs = best_cs; p->rpw = rpw; p->maxt = 512;
+    p->cs = best_cs; p->rpw = rpw; p->maxt = kWgt;
     p->S = S; p->G = G; p->grid = grid;
     p->nchunks = (max_rows + rpw - 1) / rpw;
     if (p->nchunks == 0) p->nchunks = 1;
     p->lds_bytes = (size_t)kTabBytes + 4ull * MB * (S * best_cs * 8 * kXsBlock) + 4ull * G * rpw * MB * S + 64;
     if ((uint64_t)(max_rows + 2u * (uint32_t)rpw) * ((uint64_t)(cols >> 8) * 128u) >= 0x80000000ull) return false;   // per-wave buffer range
-    return p->lds_bytes <= (size_t)kMaxLds && S * G <= 8;
+    return p->lds_bytes <= (size_t)kMaxLds && S * G <= (uint32_t)kWgt / 64u;
 }
 
 template <int MB, int XF = 0>
@@ -450,12 +458,16 @@ int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float
              float out_scale = 1.0f) {
 #define OIL4_CASE(CS_, RPW_) \
     if (p.cs == CS_ && p.rpw == RPW_) \
-        return p.nchunks > 1 ? launch<CS_, RPW_, MB, 512, XF, true>(w, d_x, d_xw, d_y, M, s, p, out_scale) \
-                             : launch<CS_, RPW_, MB, 512, XF, false>(w, d_x, d_xw, d_y, M, s, p, out_scale);
-    OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
+        return p.nchunks > 1 ? launch<CS_, RPW_, MB, kWgt, XF, true>(w, d_x, d_xw, d_y, M, s, p, out_scale) \
+                             : launch<CS_, RPW_, MB, kWgt, XF, false>(w, d_x, d_xw, d_y, M, s, p, out_scale);
+    OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6)
+    if constexpr (kWgt == 512) { OIL4_CASE(1, 12) }
     if constexpr (MB == 1) {
-        OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)
-        OIL4_CASE(3, 1) OIL4_CASE(3, 2) OIL4_CASE(3, 3) OIL4_CASE(3, 4)
+        OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3)
+        if constexpr (kWgt == 512) {
+            OIL4_CASE(2, 4) OIL4_CASE(2, 6)
+            OIL4_CASE(3, 1) OIL4_CASE(3, 2) OIL4_CASE(3, 3) OIL4_CASE(3, 4)
+        }
     }
 #undef OIL4_CASE
     return 1;
@@ -467,7 +479,7 @@ int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int 
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || M > 16) return 1;
     Oil4Plan p;                                   // rows beyond two go in passes of two (the matrix-core kernel is the
     const int MB = M == 1 ? 1 : 2;                // better choice there and the caller tries it first)
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, 8, &p)) return 1;
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, MB, kWgt / 64, &p)) return 1;
     return MB == 1 ? dispatch<1>(w, d_x, nullptr, d_y, M, s, p) : dispatch<2>(w, d_x, nullptr, d_y, M, s, p);
 }
 
@@ -475,7 +487,7 @@ int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int 
 int launch_gemv_oil4_swiglu(const oilhip_weights& w, const float* d_h, float* d_y, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x3FFFFFFFull) return 1;
     Oil4Plan p;
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, 8, &p)) return 1;
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, kWgt / 64, &p)) return 1;
     return dispatch<1, 1>(w, d_h, nullptr, d_y, 1, s, p);
 }
 
@@ -483,7 +495,7 @@ int launch_gemv_oil4_swiglu(const oilhip_weights& w, const float* d_h, float* d_
 int launch_gemv_oil4_rmsnorm(const oilhip_weights& w, const float* d_x, const float* d_xw, float* d_y, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x3FFFFFFFull) return 1;
     Oil4Plan p;
-    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, 8, &p)) return 1;
+    if (!make_plan((uint32_t)w.rows, (uint32_t)w.cols, 1, kWgt / 64, &p)) return 1;
     return dispatch<1, 2>(w, d_x, d_xw, d_y, 1, s, p);
 }
 
@@ -496,7 +508,7 @@ int launch_gemv_flat4(const uint8_t* d_w, const uint16_t* d_cb16, float scale, c
     w.d_payload = const_cast<uint8_t*>(d_w);
     w.rows = (uint64_t)rows; w.cols = (uint64_t)K;
     Oil4Plan p;
-    if (!make_plan((uint32_t)rows, (uint32_t)K, 1, 8, &p)) return 1;
+    if (!make_plan((uint32_t)rows, (uint32_t)K, 1, kWgt / 64, &p)) return 1;
     return dispatch<1, 3>(w, d_x, reinterpret_cast<const float*>(d_cb16), d_y, 1, s, p, scale);
 }
 

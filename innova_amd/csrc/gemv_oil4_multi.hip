@@ -23,8 +23,6 @@
 // shared), a row tile is 32 rows.
 #include <hip/hip_fp16.h>
 
-#include <mutex>
-
 #include "common.h"
 #include "oil4_lds.h"
 
@@ -298,21 +296,10 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 }
 
 
-// device scratch for the packed activations of one pass (one per process and device; calls that overlap on one
-// device race on it, like the prefill GEMM's)
-std::mutex g_xp_mu;
-uint32_t* g_xp[64] = {};
-constexpr uint32_t kMaxPackCols = 32768;
-
-int get_pack_buffer(uint32_t** out) {
-    int dev = 0;
-    OILHIP_HIP(hipGetDevice(&dev));
-    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
-    std::lock_guard<std::mutex> lk(g_xp_mu);
-    if (!g_xp[dev]) OILHIP_HIP(hipMalloc(&g_xp[dev], (size_t)(kMaxPackCols >> 8) * 128u * 128u * 2u));   // two token tiles
-    *out = g_xp[dev];
-    return OILHIP_OK;
-}
+// the packed activations of one pass (two token tiles) live in a scratch buffer of the stream the call runs on, or in
+// the buffer the caller hands in
+constexpr uint32_t kMaxPackCols = kGemvPackMaxCols;
+constexpr size_t kPackBytes = kGemvPackBytes;
 
 }  // namespace
 
@@ -322,22 +309,16 @@ int get_pack_buffer(uint32_t** out) {
 // Returns 1 when the shape is outside what this kernel covers.
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2, float* d_y2,
-                           uint32_t ldy2, const float* d_x2) {
+                           uint32_t ldy2, const float* d_x2, uint32_t* d_pack) {
     if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
-    if (w2 && (w2->cols != w.cols || w2->rows == 0 || w2->rows > 0x7FFFFFFFull || w2->uniform_fmt != OILHIP_OIL4 ||
-               w2->uniform_stride != 128 || !d_y2)) return 1;
-    static bool attr_done = false;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        attr_done = true;
-    }
-    uint32_t* xp = nullptr;
-    if (int rc = get_pack_buffer(&xp)) return rc;
+    if (w2 && (w2->cols != w.cols || w2->rows == 0 || w2->rows > 0x7FFFFFFFull || !plain_oil4(*w2) || !d_y2)) return 1;
+    static std::atomic<uint64_t> attr_done[3];
+    if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>), kMaxLds)) return rc;
+    if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>), kMaxLds)) return rc;
+    if (int rc = ensure_max_lds(attr_done[2], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>), kMaxLds)) return rc;
+    uint32_t* xp = d_pack;
+    if (!xp)
+        if (int rc = stream_scratch(s, kScratchGemvPack, kPackBytes, reinterpret_cast<void**>(&xp))) return rc;
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
     // rows wider than one K-pass (16 blocks, 8 for passes of 32 tokens): the row is cut into parts of at most one pass

@@ -292,12 +292,9 @@ struct Oil8Plan {
 
 template <int CS, int RPW, int MB, bool ROLL, bool FLAT>
 int launch(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s, const Oil8Plan& p, const float* d_cb, float out_scale) {
-    static bool attr_done = false;
+    static std::atomic<uint64_t> attr_done{0};
     auto kern = gemv_oil8_kernel<CS, RPW, MB, ROLL, FLAT>;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLds));
-        attr_done = true;
-    }
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), kMaxLds)) return rc;
     const uint32_t J = p.grid * p.G;
     uint32_t wave_groups = 0;                                   // wave / S for each of the 8 wavefronts, 4 bits each
     for (uint32_t wv = 0; wv < 8; ++wv) wave_groups |= (wv / p.S) << (4u * wv);

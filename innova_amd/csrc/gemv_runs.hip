@@ -150,14 +150,11 @@ gemv_runs_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict
 
 template <int MB>
 int launch_runs(const oilhip_weights& w, const DecodeTables* T, const float* d_x, float* d_y, int m0, int M, hipStream_t s) {
-    static bool attr_done = false;
+    static std::atomic<uint64_t> attr_done{0};
     auto kern = gemv_runs_kernel<MB>;
     const size_t lds = (size_t)MB * ((w.cols >> 5) * kRunPad + (w.cols >> 5)) * 4 + 532 * 4;
     if (lds > 160 * 1024) return 1;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done = true;
-    }
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
     uint32_t per_cu = (uint32_t)((160 * 1024) / lds);                 // workgroups a CU can hold: small loads need many waves in flight
     if (per_cu > 3) per_cu = 3;                                       // register budget: 3 wavefronts per SIMD
     uint32_t grid = (uint32_t)device_cu_count() * per_cu;
@@ -174,7 +171,7 @@ int launch_runs(const oilhip_weights& w, const DecodeTables* T, const float* d_x
 
 // Returns 1 when the shape is outside what this kernel covers (the caller falls back).
 int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s) {
-    if (!w.all_full || (w.cols & 255u) || w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || w.rows == 0) return 1;
+    if (!w.nominal || (w.cols & 255u) || w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull || w.rows == 0) return 1;
     const DecodeTables* T = nullptr;
     if (int rc = get_tables(&T)) return rc;
     if ((size_t)((w.cols >> 5) * (kRunPad + 1)) * 4 + 532 * 4 > 160 * 1024) return 1;

@@ -337,15 +337,12 @@ size_t seg_lds_bytes(const oilhip_weights& w) {
 template <int MB, int XF = 0>
 int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x, float* d_y, int m0, int M, hipStream_t s,
                const float* d_xw = nullptr) {
-    static bool attr_done = false;
+    static std::atomic<uint64_t> attr_done{0};
     auto kern = gemv_seg_kernel<MB, XF>;
     const SegLayout& g = w.seg;
     const size_t lds = seg_lds_bytes<MB>(w);
     if (lds > 160 * 1024) return 1;
-    if (!attr_done) {
-        OILHIP_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        attr_done = true;
-    }
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
     SegArgs A{};
     A.nstreams = g.nstreams; A.blind16 = g.blind16; A.stream_bytes = g.stream_bytes;
     for (uint32_t i = 0; i < g.nf; ++i) { A.cb_bytes[i] = g.cb_bytes[i]; A.idx_bytes[i] = g.idx_bytes[i]; A.stride[i] = g.stride[i]; }

@@ -33,12 +33,6 @@ dequant_kernel(const uint8_t* __restrict__ payload, const DevBlock* __restrict__
 // null) or wherever their descriptors say (tensors stored as window streams).
 struct FullTables { const float* lv8; const float* t255; const float* q127; const float* lv4; const float* lv2; };   // LDS copies
 
-// bytes of a full block of each format (codebook channel + index channel) and of its codebook channel
-__host__ __device__ constexpr uint32_t full_block_bytes(int f) {
-    constexpr uint32_t n[15] = {16, 48, 64, 128, 256, 512, 1024, 32, 48, 80, 144, 272, 512, 64, 64};
-    return f >= 0 && f < 15 ? n[f] : 0u;
-}
-__host__ __device__ constexpr uint32_t full_block_cb_bytes(int f) { return f == 0 ? 16u : 0u; }
 
 template <int FMT>
 __device__ __forceinline__ float4 decode_full4(const uint8_t* __restrict__ p, uint32_t lane, const FullTables& L) {

@@ -100,7 +100,8 @@ int oilhip_rmsnorm_f32(const float* d_x, const float* d_w, int n, int rows, floa
 int oilhip_gemv_rmsnorm_f32(const oilhip_weights* w, const float* d_x, const float* d_normw, float* d_y, int M, float* d_xn,
                             void* stream) {
     if (!w || !d_x || !d_normw || !d_y || M <= 0) return fail(OILHIP_E_ARG, "gemv_rmsnorm: bad arguments");
-    if (M == 1 && w->uniform_fmt == OILHIP_OIL4 && w->uniform_stride == 128) {
+    if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
+    if (M == 1 && plain_oil4(*w)) {
         const int rc = launch_gemv_oil4_rmsnorm(*w, d_x, d_normw, d_y, (hipStream_t)stream);   // the norm rides on the staging of x
         if (rc <= 0) return rc;
     }
@@ -119,13 +120,15 @@ int oilhip_mlp_step_f32(const oilhip_weights* gate_up, const oilhip_weights* dow
     const uint64_t F = down->cols;
     if (gate_up->rows != 2 * F || gate_up->cols != down->rows)
         return fail(OILHIP_E_ARG, "mlp_step: gate_up must be 2F x D (gate rows first) and down D x F");
+    if (int rc = check_matmul_shape(gate_up, d_x, d_y, M)) return rc;
+    if (int rc = check_matmul_shape(down, d_x, d_y, M)) return rc;
     hipStream_t s = (hipStream_t)stream;
     float* h2 = d_scratch;                                   // [M][2F]
     float* h = d_scratch + (size_t)M * 2 * F;                // [M][F]
     float* xn = h + (size_t)M * F;                           // [M][D], only with d_normw
     if (int rc = d_normw ? oilhip_gemv_rmsnorm_f32(gate_up, d_x, d_normw, h2, M, xn, stream)
                          : oilhip_gemv_f32(gate_up, d_x, h2, M, stream)) return rc;
-    if (M == 1 && down->uniform_fmt == OILHIP_OIL4 && down->uniform_stride == 128) {
+    if (M == 1 && plain_oil4(*down)) {
         const int rc = launch_gemv_oil4_swiglu(*down, h2, d_y, s);      // SwiGLU formed while the activations are staged
         if (rc <= 0) return rc;
     }

@@ -102,7 +102,7 @@ Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
 // one projection of an expert batch: Y[nt][rows] from rows tok[] of X (or X itself when tok is null)
 int expert_gemv(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int nt, uint32_t xrows,
                 float* d_gather, hipStream_t s) {
-    if (w.uniform_fmt == OILHIP_OIL4 && w.uniform_stride == 128) {
+    if (plain_oil4(w)) {
         const int rc = launch_gemv_oil4_multi(w, d_x, d_tok, d_y, nt, (uint32_t)w.cols, (uint32_t)w.rows, xrows, s);
         if (rc <= 0) return rc;
     }
@@ -155,9 +155,10 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                        size_t workspace_bytes, float* z_loss, int64_t* dropped, void* stream) {
     if (!gate || !up || !down || E <= 0 || !d_x || !indices || !weights || T <= 0 || K <= 0 || !d_out || !d_workspace)
         return fail(OILHIP_E_ARG, "moe_forward: bad arguments");
+    for (int e = 0; e < E; ++e)
+        if (!gate[e] || !up[e] || !down[e]) return fail(OILHIP_E_ARG, "moe_forward: null expert tensor");
     const int64_t D = (int64_t)gate[0]->cols, F = (int64_t)gate[0]->rows;
     for (int e = 0; e < E; ++e) {
-        if (!gate[e] || !up[e] || !down[e]) return fail(OILHIP_E_ARG, "moe_forward: null expert tensor");
         if ((int64_t)gate[e]->cols != D || (int64_t)gate[e]->rows != F || (int64_t)up[e]->cols != D || (int64_t)up[e]->rows != F ||
             (int64_t)down[e]->cols != F || (int64_t)down[e]->rows != D)
             return fail(OILHIP_E_ARG, "moe_forward: expert " + std::to_string(e) + " has mismatched shapes");
@@ -205,7 +206,7 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         if (nt == 0) continue;
         // gate and up read the same gathered activations: uniform OIL4 experts split them once per pass for both
         int both = 1;
-        if (gate[e]->uniform_fmt == OILHIP_OIL4 && gate[e]->uniform_stride == 128)
+        if (plain_oil4(*gate[e]))
             both = launch_gemv_oil4_multi(*gate[e], d_x, ws.tok + b, ws.g, nt, (uint32_t)D, (uint32_t)F, (uint32_t)T, s, up[e], ws.u,
                                           (uint32_t)F);
         if (both < 0) return both;
@@ -215,7 +216,7 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         }
         // silu(gate) * up: formed while the down projection's activations are split (uniform OIL4), or by a kernel of its own
         int fused = 1;
-        if (down[e]->uniform_fmt == OILHIP_OIL4 && down[e]->uniform_stride == 128)
+        if (plain_oil4(*down[e]))
             fused = launch_gemv_oil4_multi(*down[e], ws.g, nullptr, ws.o, nt, (uint32_t)F, (uint32_t)D, (uint32_t)nt, s, nullptr, nullptr, 0,
                                            ws.u);
         if (fused < 0) return fused;
