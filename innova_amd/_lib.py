@@ -72,6 +72,7 @@ _SIGNATURES = {
     "oilhip_dequant_f32": (C.c_int, [vp, vp, vp]),
     "oilhip_gemv_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_gemv_f32_general": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_gemv_oil4_f32_noalloc": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_gemm_bf16": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_flat_oil8_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_flat_oil4_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),

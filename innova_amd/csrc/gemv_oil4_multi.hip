@@ -23,6 +23,8 @@
 // shared), a row tile is 32 rows.
 #include <hip/hip_fp16.h>
 
+#include <mutex>
+
 #include "common.h"
 #include "oil4_lds.h"
 
@@ -301,6 +303,29 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 constexpr uint32_t kMaxPackCols = kGemvPackMaxCols;
 constexpr size_t kPackBytes = kGemvPackBytes;
 
+// The same scratch for the entry point that allocates nothing: a fixed array in the code object (4 MB, held by every
+// GPU the library runs on until the process ends).  In host code the array's name is only a stand-in: the device
+// address comes from hipGetSymbolAddress, once per device with that device current, and only that pointer is ever
+// handed to a kernel.
+static __device__ __align__(256) uint8_t scratch[kPackBytes];
+std::mutex g_static_mu;
+uint32_t* g_static_ptr[64] = {};
+
+int static_pack_buffer(uint32_t** out) {
+    int dev = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= 64) return fail(OILHIP_E_ARG, "device index out of range");
+    std::lock_guard<std::mutex> lk(g_static_mu);
+    if (!g_static_ptr[dev]) {
+        void* p = nullptr;
+        OILHIP_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(OILHIP_E_DEVICE, "hipGetSymbolAddress returned a null address for the static scratch");
+        g_static_ptr[dev] = static_cast<uint32_t*>(p);
+    }
+    *out = g_static_ptr[dev];
+    return OILHIP_OK;
+}
+
 }  // namespace
 
 // Y[m][r] for m < M: x row tok[m] (or m when tok is null) of an [xrows][ldx] activation matrix; with w2 the same
@@ -359,3 +384,25 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
 }
 
 }  // namespace oilhip
+
+extern "C" int oilhip_gemv_oil4_f32_noalloc(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
+    using namespace oilhip;
+    if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
+    if (!plain_oil4(*w)) return fail(OILHIP_E_ARG, "gemv_oil4_f32_noalloc: the tensor must be uniform OIL4 in the plain 128-byte block layout");
+    if (w->cols > kGemvPackMaxCols)
+        return fail(OILHIP_E_ARG, "gemv_oil4_f32_noalloc: rows of " + std::to_string(w->cols) + " weights exceed the static scratch (at most " +
+                                      std::to_string(kGemvPackMaxCols) + " columns)");
+    hipStream_t s = (hipStream_t)stream;
+    int rc = 1;                                                             // 1: shape not covered by that kernel
+    if (M <= 2) rc = launch_gemv_oil4(*w, d_x, d_y, M, s);                  // the register-resident kernel uses no scratch
+    if (rc == 1 && M >= 2) {
+        uint32_t* pack = nullptr;
+        if (int e = static_pack_buffer(&pack)) return e;
+        rc = launch_gemv_oil4_multi(*w, d_x, nullptr, d_y, M, (uint32_t)w->cols, (uint32_t)w->rows, (uint32_t)M, s, nullptr, nullptr, 0,
+                                    nullptr, pack);
+    }
+    if (rc == 1 && M > 2 && M <= 4) rc = launch_gemv_oil4(*w, d_x, d_y, M, s);
+    if (rc == 1) return fail(OILHIP_E_ARG, "gemv_oil4_f32_noalloc: this shape needs a kernel that allocates; use oilhip_gemv_f32");
+    return rc;
+}
+

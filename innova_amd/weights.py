@@ -108,12 +108,14 @@ class DeviceWeights:
         assert out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and out.numel() == M * self.rows
         return x2, M, out
 
-    def gemv(self, x, out=None, general: bool = False):
+    def gemv(self, x, out=None, general: bool = False, noalloc: bool = False):
         """Y[M][rows] = X[M][cols] . W^T, FP32 (decode path).  general=True forces the
-        all-format kernel (used by tests to cross-check the specialised kernels)."""
+        all-format kernel (used by tests to cross-check the specialised kernels); noalloc=True takes the entry
+        point that allocates no device memory (uniform OIL4 only, scratch in a fixed device array)."""
         import torch
         x2, M, out = self._xy(x, torch.float32, out)
-        fn = _lib.lib().oilhip_gemv_f32_general if general else _lib.lib().oilhip_gemv_f32
+        L = _lib.lib()
+        fn = L.oilhip_gemv_f32_general if general else L.oilhip_gemv_oil4_f32_noalloc if noalloc else L.oilhip_gemv_f32
         _lib.check(fn(self.handle, x2.data_ptr(), out.data_ptr(), M, _lib.current_stream()))
         return out
 
