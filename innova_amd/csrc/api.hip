@@ -95,6 +95,11 @@ int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out) {
             (void)hipGetLastError();
             return fail(OILHIP_E_NOMEM, "hipMalloc of " + std::to_string(want) + " bytes of scratch failed");
         }
+        if (hipMemset(p, 0, want) != hipSuccess) {
+            (void)hipGetLastError();
+            (void)hipFree(p);
+            return fail(OILHIP_E_DEVICE, "hipMemset of the new scratch failed");
+        }
         e = {p, want};                       // the smaller buffer stays allocated (see common.h)
     }
     *out = e.first;

@@ -45,6 +45,7 @@ int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes);
 // lives (a captured graph or a queued kernel may still point at it): a request that outgrows it gets a new, larger
 // one and the old one stays allocated.  No allocation can happen while the stream is being captured, so the first
 // call of a given size on a stream has to be made outside capture; otherwise the call fails with OILHIP_E_ARG.
+// New buffers are zero-filled.
 enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1 };
 int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
@@ -116,7 +117,8 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
                            float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr, uint32_t* d_pack = nullptr);
 // widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
 constexpr uint32_t kGemvPackMaxCols = 32768;
-constexpr size_t kGemvPackBytes = (size_t)(kGemvPackMaxCols >> 8) * 128u * 128u * 2u;
+constexpr size_t kGemvPackExpBytes = (size_t)(kGemvPackMaxCols >> 8) * 2u * 16u * 4u;    // one scale exponent per (token tile, block, column)
+constexpr size_t kGemvPackBytes = (size_t)(kGemvPackMaxCols >> 8) * 128u * 128u * 2u + kGemvPackExpBytes;   // two token tiles, then the exponents
 // rows that mix formats, stored tile by tile and format by format
 int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // every format, a lane per run of 32 weights

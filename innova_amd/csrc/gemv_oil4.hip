@@ -35,8 +35,14 @@
 #ifndef OILHIP_OIL4_WGT
 #define OILHIP_OIL4_WGT 512      // threads per workgroup of the decode kernel (512 or 1024)
 #endif
+#ifndef OILHIP_OIL4_LA
+#define OILHIP_OIL4_LA 0         // 0: chosen by the workgroup size
+#endif
+#ifndef OILHIP_OIL4_SKIP
+#define OILHIP_OIL4_SKIP 0       // 1: single-chunk launches skip the products of row slots past the group's rows
+#endif
 #ifndef OILHIP_OIL4_AUX
-#define OILHIP_OIL4_AUX 0        // cache policy of the weight loads: 2 = nt (streamed once, not kept in L2 / the Infinity Cache)
+#define OILHIP_OIL4_AUX 2        // cache policy of the weight loads: 2 = nt (streamed once, not kept in L2 / the Infinity Cache)
 #endif
 
 namespace oilhip {
@@ -63,6 +69,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
                  uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups_lo, uint32_t wave_groups_hi, float out_scale) {
     constexpr uint32_t NW = WGT / 64;   // wavefronts per workgroup
     constexpr int NL = CS * RPW;      // wave-loads per chunk
+    constexpr int LA = OILHIP_OIL4_LA ? OILHIP_OIL4_LA : (WGT == 1024 ? 1 : 4);   // dwords of a wave-load decoded per pipeline step
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
     const uint32_t nblk = S * CS * 8;                                         // blocks covered by all slabs (>= cols/256)
@@ -290,12 +297,38 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
             for (int n = 0; n < NL; ++n) issue_load(n, ch * RPW);
         }
         float part[MB][RPW];                              // per-lane partial of each row, block scales applied
-        LevelPair cur[16];
-        lookup_load(wv[0], lanebase, cur);
+        // A wave-load is consumed in units of LA dwords (4 LA packed bytes): the table reads of the next unit are in
+        // flight while the products of the current one are formed.  Four wavefronts per SIMD hide the table latency
+        // between them, so their units are one dword and the two staging arrays 16 registers; two wavefronts per SIMD
+        // stage a whole wave-load.
+        constexpr int UPL = 4 / LA, UB = 4 * LA;          // units per wave-load, packed bytes per unit
+        // rows of this chunk that exist (single-chunk launches skip the products of the row slots past them; with
+        // rolling loads the count of outstanding loads must not depend on it, so there every slot is worked)
+        constexpr bool SKIP = OILHIP_OIL4_SKIP && !ROLL;
+        const uint32_t nvalid = !SKIP ? (uint32_t)RPW : (r1 > cbase ? r1 - cbase : 0u);
+        LevelPair cur[UB];
+        auto lookup_unit = [&](int u, LevelPair (&t)[UB]) {
+            const u32x4 w4 = wv[u / UPL];
+            const uint32_t wd[4] = {w4.x, w4.y, w4.z, w4.w};
+#pragma unroll
+            for (int d = 0; d < LA; ++d) {
+                const uint32_t word = wd[(u % UPL) * LA + d];
+                t[4 * d + 0] = lookup<0>(word, lanebase);
+                t[4 * d + 1] = lookup<1>(word, lanebase);
+                t[4 * d + 2] = lookup<2>(word, lanebase);
+                t[4 * d + 3] = lookup<3>(word, lanebase);
+            }
+        };
+        lookup_unit(0, cur);
 #pragma unroll
         for (int n = 0; n < NL; ++n) {
             const int it = n / CS, cs = n % CS;
-            // The two wavefronts of a SIMD are served oldest first; left alone the older one runs ahead and the
+            if (SKIP && (uint32_t)it >= nvalid) {                             // wave-uniform: this row slot is past the group's rows
+#pragma unroll
+                for (int m = 0; m < MB; ++m) if (cs == 0) part[m][it] = 0.0f;
+                continue;
+            }
+            // The wavefronts of a SIMD are served oldest first; left alone the older one runs ahead and the
             // younger finishes its rows on its own.  Priority falls with progress, so whichever is behind goes first.
             if (!ROLL && (n == 0 || (n * 4) / NL != ((n - 1) * 4) / NL)) {
                 const int pr = 3 - (n * 4) / NL;
@@ -304,32 +337,44 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
                 else if (pr == 1) __builtin_amdgcn_s_setprio(1);
                 else __builtin_amdgcn_s_setprio(0);
             }
-            LevelPair nxt[16];
-            if (n + 1 < NL) lookup_load(wv[n + 1], lanebase, nxt);    // next load's table reads fly during these FMAs
-            __builtin_amdgcn_sched_barrier(0);                        // keep them above the FMAs
-            // the block's FP16 scale sits in the low half of its first lane's first dword
-            const float scale = XF == 3 ? 1.0f : __half2float(__ushort_as_half((unsigned short)(dpp_bcast8(wv[n].x) & 0xFFFFu)));
+            float a0[MB], a1[MB];
 #pragma unroll
-            for (int m = 0; m < MB; ++m) {
-                float a0 = 0.0f, a1 = 0.0f;
+            for (int m = 0; m < MB; ++m) { a0[m] = 0.0f; a1[m] = 0.0f; }
 #pragma unroll
-                for (int k = 0; k < 16; k += 2) {
-                    a0 = __fmaf_rn(cur[k].lo, xr[m][cs][2 * k], a0);
-                    a0 = __fmaf_rn(cur[k].hi, xr[m][cs][2 * k + 1], a0);
-                    a1 = __fmaf_rn(cur[k + 1].lo, xr[m][cs][2 * k + 2], a1);
-                    a1 = __fmaf_rn(cur[k + 1].hi, xr[m][cs][2 * k + 3], a1);
+            for (int q = 0; q < UPL; ++q) {
+                const int u = n * UPL + q;
+                LevelPair nxt[UB];
+                const bool more = u + 1 < NL * UPL && (!SKIP || q + 1 < UPL || (uint32_t)((n + 1) / CS) < nvalid);
+                if (more) lookup_unit(u + 1, nxt);                    // next unit's table reads fly during these FMAs
+                __builtin_amdgcn_sched_barrier(0);                    // keep them above the FMAs
+#pragma unroll
+                for (int m = 0; m < MB; ++m) {
+#pragma unroll
+                    for (int k = 0; k < UB; k += 2) {
+                        const int kb = q * UB + k;                    // packed byte of the wave-load
+                        a0[m] = __fmaf_rn(cur[k].lo, xr[m][cs][2 * kb], a0[m]);
+                        a0[m] = __fmaf_rn(cur[k].hi, xr[m][cs][2 * kb + 1], a0[m]);
+                        a1[m] = __fmaf_rn(cur[k + 1].lo, xr[m][cs][2 * kb + 2], a1[m]);
+                        a1[m] = __fmaf_rn(cur[k + 1].hi, xr[m][cs][2 * kb + 3], a1[m]);
+                    }
                 }
-                part[m][it] = cs == 0 ? (a0 + a1) * scale : __fmaf_rn(a0 + a1, scale, part[m][it]);
-            }
-            if (n + 1 < NL) {
+                if (q == UPL - 1) {
+                    // the block's FP16 scale sits in the low half of its first lane's first dword
+                    const float scale = XF == 3 ? 1.0f : __half2float(__ushort_as_half((unsigned short)(dpp_bcast8(wv[n].x) & 0xFFFFu)));
 #pragma unroll
-                for (int k = 0; k < 16; ++k) cur[k] = nxt[k];
+                    for (int m = 0; m < MB; ++m)
+                        part[m][it] = cs == 0 ? (a0[m] + a1[m]) * scale : __fmaf_rn(a0[m] + a1[m], scale, part[m][it]);
+                    // ROLL (shapes with more than one chunk): wv[n] is free, the same wave-load of the next chunk takes its
+                    // place, so NL loads stay in flight across chunks.  Issued unconditionally (past the last row the offset is
+                    // out of range: zeros, no fetch), which keeps the count of outstanding loads at every wait a constant.
+                    if (ROLL) issue_load(n, (ch + 1u) * RPW);
+                }
+                if (more) {
+#pragma unroll
+                    for (int k = 0; k < UB; ++k) cur[k] = nxt[k];
+                }
+                __builtin_amdgcn_sched_barrier(0);                    // one scheduling region per unit
             }
-            // ROLL (shapes with more than one chunk): wv[n] is free, the same wave-load of the next chunk takes its
-            // place, so NL loads stay in flight across chunks.  Issued unconditionally (past the last row the offset is
-            // out of range: zeros, no fetch), which keeps the count of outstanding loads at every wait a constant.
-            if (ROLL) issue_load(n, (ch + 1u) * RPW);
-            __builtin_amdgcn_sched_barrier(0);                        // one scheduling region per wave-load
         }
         // ---- all rows of the chunk reduced over the 64 lanes together (independent chains) ----
 #pragma unroll

@@ -57,52 +57,77 @@ constexpr int kRedBytes = 8 * kGroups * kRedTile * 4;
 // low parts.  Piece j (dwords 4j .. 4j+3 of the 32) of all 64 lanes is one contiguous KB at
 // ((blk*2 + h)*8 + j)*1024 + l*16 bytes, so that a wavefront fetches it with one coalesced 16-byte load per lane.  Nibble p = 32*(kq + 4h) + s of a block holds weight
 // i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
+// A wavefront packs one block of one token column (256 activations): it finds their largest magnitude, scales them by
+// the power of two that brings it to [2^14, 2^15) (so the FP16 split keeps 22 bits whatever the magnitude of the
+// activations; blocks that are zero or hold a non-finite value stay unscaled) and leaves the exponent at
+// xp_exp[(tile * bpr + blk) * 16 + column] for the main kernel, which undoes it on the block's partial sums.
+__device__ __forceinline__ float pack_value(const float* __restrict__ x, const float* __restrict__ x2, size_t at) {
+    float v = x[at];
+    // x2: the activations are silu(x) * x2, the SwiGLU product in front of an expert's down projection
+    // (ExpertFFN::forward, src/moe_variants.cpp:77-91), formed here instead of in a kernel of its own
+    if (x2) v = (v / (1.0f + expf(-v))) * x2[at];
+    return v;
+}
+
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
-              uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
+              int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
               float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld) {
-    const uint32_t bpr = cols >> 8;
+    const uint32_t bpr = cols >> 8, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     // outputs that the main kernel accumulates into (rows cut along K between workgroups) start at zero
-    const uint32_t gid = blockIdx.x * 256u + threadIdx.x, gn = gridDim.x * 256u;
+    const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
     if (yc0)
         for (uint32_t i = gid; i < yc0_rows * (uint32_t)(M - m0); i += gn) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
     if (yc1)
         for (uint32_t i = gid; i < yc1_rows * (uint32_t)(M - m0); i += gn) yc1[(size_t)(m0 + i / yc1_rows) * yc1_ld + i % yc1_rows] = 0.0f;
-    // a pass of 32 tokens is two tiles of 16: blocks bpr*8 .. of the grid pack tokens m0 + 16 .. behind the first tile
-    const uint32_t tile = blockIdx.x / (bpr * 8u);
-    const uint32_t id = (blockIdx.x - tile * bpr * 8u) * 256u + threadIdx.x;   // ((blk*2 + h)*64 + lane)*16 + c: one FP16 pair per thread
-    m0 += 16 * (int)tile;
+    // workgroup = 4 blocks of token column t of a tile (a pass of 32 tokens is two tiles of 16, the second one's data
+    // behind the first's); passes of 8 tokens have 8 token columns: columns 0..7 of the operand carry their high
+    // parts and columns 8..15 their low parts, in the pieces that otherwise hold the high parts of 16 tokens
+    const uint32_t ncol = half ? 8u : 16u, nbg = (bpr + 3u) / 4u;
+    const uint32_t blk = (blockIdx.x % nbg) * 4u + wave, t = (blockIdx.x / nbg) % ncol, tile = blockIdx.x / (nbg * ncol);
+    if (blk >= bpr) return;
+    const int m = m0 + 16 * (int)tile + (int)t;
     xp += (size_t)tile * bpr * 4096u;
-    if (id >= bpr * 2048u) return;
-    const uint32_t c = id & 15u, lane = (id >> 4) & 63u, h = (id >> 10) & 1u, blk = id >> 11;
-    const uint32_t t = lane & 15u, kq = lane >> 4;
-    // passes of 8 tokens: columns 0..7 carry the high parts of tokens 0..7, columns 8..15 their low parts, in the
-    // pieces that otherwise hold the high parts of 16 tokens; the low-part pieces are not used
-    const int m = m0 + (int)(half ? (t & 7u) : t);
     const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
-    float v[2] = {0.0f, 0.0f};
-    if (src < xrows) {
-        const size_t at = (size_t)src * ldx + (size_t)blk * 256u;
+    const bool live = src < xrows;
+    const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u : 0;
+    // this lane's two pairs: pair id = lane + 64 k holds positions 2c, 2c+1 of chunk kq + 4h
+    float v[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+    uint32_t mx = 0u;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
             const uint32_t pn = 32u * (kq + 4u * h) + 2u * c + e;
-            if (pn >= 4u) {
+            if (live && pn >= 4u) {
                 const uint32_t q = pn - 4u;
-                v[e] = x[at + q + q / 63u];
-                // x2: the activations are silu(x) * x2, the SwiGLU product in front of an expert's down projection
-                // (ExpertFFN::forward, src/moe_variants.cpp:77-91), formed here instead of in a kernel of its own
-                if (x2) v[e] = (v[e] / (1.0f + expf(-v[e]))) * x2[at + q + q / 63u];
+                v[k][e] = pack_value(x, x2, at + q + q / 63u);
             }
+            mx = max(mx, __float_as_uint(v[k][e]) & 0x7FFFFFFFu);
         }
     }
-    const auto ph = __builtin_amdgcn_cvt_pkrtz(v[0], v[1]);           // x = xh + xl, both FP16 (round toward zero)
-    const auto pl = __builtin_amdgcn_cvt_pkrtz(v[0] - (float)ph[0], v[1] - (float)ph[1]);
-    uint32_t* o = xp + ((size_t)(id >> 10) * 8u * 64u + lane) * 4u + (c & 3u);     // piece 0 of this lane, element c & 3
-    if (half) {
-        o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, t < 8u ? ph : pl);
-    } else {
-        o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
-        o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
+    const int ex = (int)(mx >> 23);
+    const int e2 = (mx == 0u || ex == 255) ? 0 : 14 - (ex - 127);
+    if (lane == 0) {
+        xp_exp[(tile * bpr + blk) * 16u + t] = e2;
+        if (half) xp_exp[(tile * bpr + blk) * 16u + t + 8u] = e2;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
+        const float s0 = ldexpf(v[k][0], e2), s1 = ldexpf(v[k][1], e2);
+        const auto ph = __builtin_amdgcn_cvt_pkrtz(s0, s1);           // x = xh + xl, both FP16 (round toward zero)
+        const auto pl = __builtin_amdgcn_cvt_pkrtz(s0 - (float)ph[0], s1 - (float)ph[1]);
+        uint32_t* o = xp + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (c & 3u);     // piece 0 of lane 16 kq + t, element c & 3
+        if (half) {
+            o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
+            o[(size_t)(c >> 2) * 256u + 32u] = __builtin_bit_cast(uint32_t, pl);                   // lane 16 kq + t + 8
+        } else {
+            o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
+            o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+        }
     }
 }
 
@@ -114,12 +139,13 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
 // product term; a row tile is two groups of 16 rows.
 template <bool HALF, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, float* __restrict__ y,
+gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
                        uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
                        uint32_t ksplit) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
+    float* undo = reinterpret_cast<float*>(lds + kRedBase + kRedBytes);    // [NT][blocks of this part][16 columns]: 2^-e of the packed activations
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t li = lane & 15u, kq = lane >> 4;
@@ -157,8 +183,8 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
             const uint32_t blk = blk_lo + pass * PB + wave * BPW + b2;
             const bool ok = g < g1 && r < rows && blk < blk_hi;
             const uint32_t off = (r - g0 * 16u) * row_bytes + blk * 128u + kq * 16u;
-            wv[buf][b2][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off : kOobOffset, 0, 0);
-            wv[buf][b2][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off + 64u : kOobOffset, 0, 0);
+            wv[buf][b2][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off : kOobOffset, 0, 2);
+            wv[buf][b2][1] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off + 64u : kOobOffset, 0, 2);
         }
     };
 
@@ -196,6 +222,10 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
             reinterpret_cast<uint4*>(tab)[tid + 512u * k] = make_uint4(e_hi, e_lo, e_hi, e_lo);
         }
     }
+    for (uint32_t i = tid; i < (uint32_t)NT * (blk_hi - blk_lo) * 16u; i += 512u) {
+        const uint32_t t = i / ((blk_hi - blk_lo) * 16u), rem = i % ((blk_hi - blk_lo) * 16u);
+        undo[i] = ldexpf(1.0f, -xp_exp[(t * bpr + blk_lo) * 16u + rem]);
+    }
     bool table_synced = false;
 
     for (uint32_t tile = 0; tile < ntiles; ++tile) {
@@ -223,7 +253,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                     for (int h = 0; h < 2; ++h) {
                         const u32x4 wh = h == 0 ? w0 : w1;
                         const uint32_t wd[4] = {wh.x, wh.y, wh.z, wh.w};
-                        constexpr int DS = NT == 2 ? 2 : 4;                // dwords decoded per batch of table reads
+                        constexpr int DS = HALF ? 4 : 2;                   // dwords decoded per batch of table reads (register budget)
 #pragma unroll
                         for (int d0 = 0; d0 < 4; d0 += DS) {
                             uint32_t ah[4 * DS], al[4 * DS];
@@ -257,13 +287,19 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                             __builtin_amdgcn_sched_barrier(0);
                         }
                     }
+                    // 2^-e of this lane's token column for this block (per token tile), left in LDS by the prologue
+                    float unscale[NT];
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+                        unscale[t] = undo[((uint32_t)t * (blk_hi - blk_lo) + pass * PB + wave * BPW + b2) * 16u + li];
                     // the block's FP16 scale of row r sits in the low half of the first dword of lane r (kq = 0)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
                         const uint32_t sbits = (uint32_t)__builtin_amdgcn_ds_bpermute((int)((4u * kq + v) * 4u), (int)w0.x) & 0xFFFFu;
                         const float scale = __half2float(__ushort_as_half((unsigned short)sbits));
 #pragma unroll
-                        for (int t = 0; t < NT; ++t) acc[g * NT + t][v] = __fmaf_rn(t0[t][v] + t1[t][v], scale, acc[g * NT + t][v]);
+                        for (int t = 0; t < NT; ++t)
+                            acc[g * NT + t][v] = __fmaf_rn((t0[t][v] + t1[t][v]) * unscale[t], scale, acc[g * NT + t][v]);
                     }
                 }
             }
@@ -344,7 +380,8 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
     uint32_t* xp = d_pack;
     if (!xp)
         if (int rc = stream_scratch(s, kScratchGemvPack, kPackBytes, reinterpret_cast<void**>(&xp))) return rc;
-    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + 64;            // table, then partial sums
+    int* xp_exp = reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(xp) + kGemvPackBytes - kGemvPackExpBytes);   // exponents behind the packed data
+    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;   // table, partial sums, the activations' scale factors
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
     // rows wider than one K-pass (16 blocks, 8 for passes of 32 tokens): the row is cut into parts of at most one pass
     // that go to different workgroups, so that a workgroup fetches the split activations of its part once instead of
@@ -360,7 +397,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         uint32_t slabs = (uint32_t)device_cu_count() / ks;
         if (slabs > groups) slabs = groups;
         auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
-        hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, y, (uint32_t)t.rows,
+        hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, xp_exp, y, (uint32_t)t.rows,
                            (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
     };
     for (int m0 = 0; m0 < M;) {       // passes of 32 tokens while more than 16 are left, then one of 16 or of 8
@@ -368,7 +405,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         const int kind = left <= 8 ? 0 : left <= 16 ? 1 : 2;
         const int m1 = left <= 32 ? M : m0 + 32;
         const bool cut = split_of(kind == 2 ? 8u : 16u) > 1u;
-        hipLaunchKernelGGL(pack_x_kernel, dim3(bpr * 8u * (kind == 2 ? 2u : 1u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp,
+        hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
                            (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, cut ? d_y : nullptr, (uint32_t)w.rows, ldy,
                            w2 && cut ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
         OILHIP_HIP(hipGetLastError());

@@ -95,7 +95,7 @@ gemv_oil8_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, flo
     u32x4 wv[NL];
     auto issue_load = [&](int n, uint32_t rel) {           // rel: first row of the chunk, counted from r0
         const int it = n / CS, cs = n % CS;
-        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, 0);
+        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, 2);
     };
 #pragma unroll
     for (int n = 0; n < PFA; ++n) issue_load(n, 0u);

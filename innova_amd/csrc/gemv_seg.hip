@@ -204,7 +204,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t piece = j * 64u + lane < A.blind16 ? j * 64u + lane : A.blind16 - 1u;
-        wreg[j] = *reinterpret_cast<const u32x4*>(sp + (size_t)piece * 16u);
+        wreg[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(sp + (size_t)piece * 16u));
     }
 
     build_level_tables(smem, tid);
@@ -284,7 +284,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t piece = j * 64u + lane < used16 ? j * 64u + lane : used16 - 1u;
-                wreg[j] = *reinterpret_cast<const u32x4*>(np + (size_t)piece * 16u);
+                wreg[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(np + (size_t)piece * 16u));
             }
         }
         const uint32_t ne = uniform(hdr[0]);

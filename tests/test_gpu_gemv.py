@@ -225,3 +225,27 @@ def test_shape_errors():
     with ia.DeviceWeights.from_blocks(payload, blocks, 1, w.size) as dw:
         with pytest.raises(ia.OilHipError):
             dw.gemv(torch.zeros(1, w.size, device="cuda"))        # ragged block: matmul refuses
+
+
+# The multi-row kernel splits activations into two FP16 parts after scaling each token row by a power of two, so its
+# accuracy must not depend on the magnitude of the activations: tiny rows, huge rows (beyond the FP16 range), rows that
+# mix magnitudes, a zero row, and tokens of very different scale in one batch.
+@pytest.mark.parametrize("rows,cols,M", [(130, 4096, 5), (61, 11008, 16), (300, 2048, 24)])
+def test_oil4_multi_token_activation_ranges(rows, cols, M):
+    w = gaussian_weights(rows * cols, rows + cols)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    rng = np.random.default_rng(M)
+    X = rng.standard_normal((M, cols)).astype(np.float32)
+    X[0] *= np.float32(1e-6)
+    X[1] *= np.float32(1e5)
+    X[2] *= np.float32(3e-30)
+    X[3] *= np.float32(2e30)
+    X[4, ::3] *= np.float32(1e-7)                         # one row with magnitudes 14 decades apart
+    X[4, 1::3] *= np.float32(1e7)
+    if M > 5:
+        X[5] = 0.0
+    want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        got = dw.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
+    for m in range(M):                                    # row by row: a large row must not hide a small one
+        assert rel_l2(got[m], want[m]) <= TOL, m
