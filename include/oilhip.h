@@ -178,6 +178,14 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
  * threads) race on it and must be serialized by the caller. */
 int oilhip_gemv_oil4_f32_noalloc(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream);
 
+/* Rows too wide for one workgroup pass of the multi-row OIL4 kernel (more than 16 blocks, 8 for batches beyond 16 rows)
+ * are cut into parts whose partial sums have to meet.  ordered = 1 (the default): three or more parts are added in a
+ * fixed order through a workspace, so a call returns the same bits every time, like the reference's sequential loop
+ * (src/adapters/tools/qwen35_engine.cpp:71-78).  ordered = 0: float atomics, a few microseconds faster, last bits may
+ * differ from run to run (within the 1e-5 bound).  Process-wide. */
+int oilhip_set_ordered_sums(int ordered);
+
+
 /* Prefill form of the same contraction: activations as bf16 bit patterns,
  * weights dequantized to bf16 in LDS, MFMA with FP32 accumulation, FP32 out.
  * (The reference has no bf16 path; its FP32 prefill loop is

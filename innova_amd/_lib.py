@@ -73,6 +73,7 @@ _SIGNATURES = {
     "oilhip_gemv_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_gemv_f32_general": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_gemv_oil4_f32_noalloc": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_set_ordered_sums": (C.c_int, [C.c_int]),
     "oilhip_gemm_bf16": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_flat_oil8_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_flat_oil4_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),

@@ -114,7 +114,9 @@ int launch_gemv_flat8(const uint8_t* d_idx, const float* d_cb, const float* d_ac
 // several activation rows at once (FP32 MFMA); x row tok[m] (or m) of an [xrows][ldx] matrix, y row stride ldy
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2 = nullptr,
-                           float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr, uint32_t* d_pack = nullptr);
+                           float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr, uint32_t* d_pack = nullptr,
+                           size_t pack_cap = 0);
+void g_ordered_sums_set(int v);
 // widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
 constexpr uint32_t kGemvPackMaxCols = 32768;
 constexpr size_t kGemvPackExpBytes = (size_t)(kGemvPackMaxCols >> 8) * 2u * 16u * 4u;    // one scale exponent per (token tile, block, column)

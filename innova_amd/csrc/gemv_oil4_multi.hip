@@ -23,6 +23,7 @@
 // shared), a row tile is 32 rows.
 #include <hip/hip_fp16.h>
 
+#include <algorithm>
 #include <mutex>
 
 #include "common.h"
@@ -74,7 +75,7 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
               int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
               float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld) {
     const uint32_t bpr = cols >> 8, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    // outputs that the main kernel accumulates into (rows cut along K between workgroups) start at zero
+    // outputs that the main kernel's two row parts add into start at zero
     const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
     if (yc0)
         for (uint32_t i = gid; i < yc0_rows * (uint32_t)(M - m0); i += gn) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
@@ -141,7 +142,7 @@ template <bool HALF, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
                        uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
-                       uint32_t ksplit) {
+                       uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
@@ -151,7 +152,9 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     const uint32_t li = lane & 15u, kq = lane >> 4;
     const uint32_t bpr = cols >> 8, row_bytes = bpr * 128u;
     // ksplit > 1: workgroup blockIdx.x takes part blockIdx.x % ksplit of every row (at most 16 blocks, so its
-    // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit, and adds into y
+    // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit.  Two parts add into a zeroed
+    // y with float atomics (two addends: the sum does not depend on their order); three or more parts write their sums
+    // to `partial` and the workgroup that arrives last at the slab's counter adds them in ascending order
     const uint32_t slab = ksplit > 1u ? blockIdx.x / ksplit : blockIdx.x, part = ksplit > 1u ? blockIdx.x % ksplit : 0u;
     static_assert(NT == 1 || !HALF, "passes of 8 tokens have one token tile");
     constexpr int BPW = NT == 2 ? 1 : 2;                                   // blocks of the row per wavefront and pass
@@ -325,11 +328,60 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                     s += cell[j * 4u];
                     if (HALF) s += cell[(j + 8u) * 4u];
                 }
-                if (ksplit > 1u) unsafeAtomicAdd(y + (size_t)(m0 + jj) * ldy + r, s);
+                if (ksplit == 2u || (ksplit > 2u && !ordered)) unsafeAtomicAdd(y + (size_t)(m0 + jj) * ldy + r, s);
+                else if (ksplit > 2u)
+                    __hip_atomic_store(&partial[((size_t)part * (uint32_t)(M - m0) + jj) * rows + r], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 else y[(size_t)(m0 + jj) * ldy + r] = s;
             }
         }
         if (tile + 1 < ntiles) __syncthreads();                            // red is rewritten by the next tile
+    }
+    if (ksplit <= 2u || !ordered) return;
+    // ---- rows cut into three or more parts: the last workgroup of the slab adds the parts in ascending order, so the result does
+    // not depend on the order in which workgroups run.  The parts' sums are written and read with device-scope
+    // accesses that go through to memory (no cache of another XCD can hold a stale copy), so no cache-wide write-back
+    // or invalidate is needed: every thread waits until its own stores are acknowledged, the barrier collects the
+    // workgroup, then one thread counts the workgroup in.  The last one leaves the counter at zero for the next launch.
+    volatile uint32_t* last = reinterpret_cast<volatile uint32_t*>(lds + kRedBase + kRedBytes + 8192);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (tid == 0) {
+        const uint32_t seen = __hip_atomic_fetch_add(&counter[slab], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *last = seen == ksplit - 1u ? 1u : 0u;
+        if (seen == ksplit - 1u) __hip_atomic_store(&counter[slab], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!*last) return;
+    const uint32_t r_lo = g0 * 16u, r_hi = g1 * 16u < rows ? g1 * 16u : rows, nr = r_hi - r_lo, Mp = (uint32_t)(M - m0);
+    // 8 outputs x 8 parts of loads in flight per thread (device scope: sc1), so the slab's sums cost one round trip
+    const uint64_t pbytes = (uint64_t)ksplit * Mp * rows * 4u;
+    const __amdgpu_buffer_rsrc_t prsrc = __builtin_amdgcn_make_buffer_rsrc((void*)partial, 0, (int)(uint32_t)(pbytes < 0xFFFFFFFFull ? pbytes : 0xFFFFFFFFull), 0x00020000);
+    for (uint32_t o0 = tid; o0 < nr * Mp; o0 += 512u * 8u) {
+        float sum[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) sum[q] = 0.0f;
+        for (uint32_t p0 = 0; p0 < ksplit; p0 += 8u) {
+            float v[8][8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) {
+                const uint32_t o = o0 + 512u * q, jj = o / nr, r = r_lo + o % nr;
+#pragma unroll
+                for (int p2 = 0; p2 < 8; ++p2) {
+                    const bool ok = o < nr * Mp && p0 + p2 < ksplit;
+                    const uint32_t off = ok ? (uint32_t)((((size_t)(p0 + p2) * Mp + jj) * rows + r) * 4u) : kOobOffset;
+                    v[q][p2] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(prsrc, off, 0, 16));
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 8; ++q)
+#pragma unroll
+                for (int p2 = 0; p2 < 8; ++p2) sum[q] += v[q][p2];   // parts in ascending order (absent ones read as zero)
+        }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const uint32_t o = o0 + 512u * q, jj = o / nr, r = r_lo + o % nr;
+            if (o < nr * Mp) y[(size_t)(m0 + jj) * ldy + r] = sum[q];
+        }
     }
 }
 
@@ -343,7 +395,12 @@ constexpr size_t kPackBytes = kGemvPackBytes;
 // GPU the library runs on until the process ends).  In host code the array's name is only a stand-in: the device
 // address comes from hipGetSymbolAddress, once per device with that device current, and only that pointer is ever
 // handed to a kernel.
-static __device__ __align__(256) uint8_t scratch[kPackBytes];
+// rows cut into three or more parts: sums added in a fixed order through the workspace (default), or with float atomics
+std::atomic<int> g_ordered_sums{1};
+
+constexpr size_t kStaticScratchBytes = 8u << 20;
+static_assert(kStaticScratchBytes > kPackBytes + 4096u, "the static scratch holds the packed activations and the counters");
+static __device__ __align__(256) uint8_t scratch[kStaticScratchBytes];
 std::mutex g_static_mu;
 uint32_t* g_static_ptr[64] = {};
 
@@ -364,33 +421,46 @@ int static_pack_buffer(uint32_t** out) {
 
 }  // namespace
 
+void g_ordered_sums_set(int v) { g_ordered_sums.store(v ? 1 : 0, std::memory_order_relaxed); }
+
 // Y[m][r] for m < M: x row tok[m] (or m when tok is null) of an [xrows][ldx] activation matrix; with w2 the same
 // activations also go through a second tensor of the same width into d_y2 (the gate and up projections of an expert):
 // they are split and ordered once per pass for both.  With d_x2 (same layout as d_x) the activations are silu(x) * x2.
 // Returns 1 when the shape is outside what this kernel covers.
 int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int* d_tok, float* d_y, int M,
                            uint32_t ldx, uint32_t ldy, uint32_t xrows, hipStream_t s, const oilhip_weights* w2, float* d_y2,
-                           uint32_t ldy2, const float* d_x2, uint32_t* d_pack) {
+                           uint32_t ldy2, const float* d_x2, uint32_t* d_pack, size_t pack_cap) {
     if (w.rows == 0 || w.rows > 0x7FFFFFFFull || w.cols > kMaxPackCols || (w.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
     if (w2 && (w2->cols != w.cols || w2->rows == 0 || w2->rows > 0x7FFFFFFFull || !plain_oil4(*w2) || !d_y2)) return 1;
     static std::atomic<uint64_t> attr_done[3];
     if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>), kMaxLds)) return rc;
     if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>), kMaxLds)) return rc;
     if (int rc = ensure_max_lds(attr_done[2], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>), kMaxLds)) return rc;
-    uint32_t* xp = d_pack;
-    if (!xp)
-        if (int rc = stream_scratch(s, kScratchGemvPack, kPackBytes, reinterpret_cast<void**>(&xp))) return rc;
-    int* xp_exp = reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(xp) + kGemvPackBytes - kGemvPackExpBytes);   // exponents behind the packed data
-    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;   // table, partial sums, the activations' scale factors
     const uint32_t bpr = (uint32_t)(w.cols >> 8);
     // rows wider than one K-pass (16 blocks, 8 for passes of 32 tokens): the row is cut into parts of at most one pass
     // that go to different workgroups, so that a workgroup fetches the split activations of its part once instead of
-    // once per pass and tile (the parts' sums meet through float atomics: with three or more parts the order of the
-    // additions, and with it the last bits of y, can differ between launches)
+    // once per pass and tile; the parts' sums meet in a workspace behind the packed activations (4096 bytes of
+    // counters, then [parts][tokens of the pass][rows] floats)
     auto split_of = [&](uint32_t pass_blocks) -> uint32_t {
         const uint32_t np = (bpr + pass_blocks - 1u) / pass_blocks;
         return np >= 2u && np <= (uint32_t)device_cu_count() ? np : 1u;
     };
+    const bool ordered = g_ordered_sums.load(std::memory_order_relaxed) != 0;
+    const uint64_t max_rows = w2 && w2->rows > w.rows ? w2->rows : w.rows;
+    size_t need = kPackBytes;
+    {
+        const uint32_t ks16 = split_of(16u), ks8 = split_of(8u);
+        const uint64_t parts_tokens = M > 16 ? std::max<uint64_t>((uint64_t)ks8 * 32u, (uint64_t)ks16 * 16u) : (uint64_t)ks16 * (uint64_t)(M < 16 ? M : 16);
+        if (ordered && (M > 16 ? ks8 : ks16) > 2u) need += 4096u + (size_t)(parts_tokens * max_rows * 4u);
+    }
+    uint32_t* xp = d_pack;
+    if (xp && pack_cap < need) return 1;                                   // the caller's buffer cannot take this shape
+    if (!xp)
+        if (int rc = stream_scratch(s, kScratchGemvPack, need, reinterpret_cast<void**>(&xp))) return rc;
+    uint32_t* counter = reinterpret_cast<uint32_t*>(reinterpret_cast<uint8_t*>(xp) + kPackBytes);
+    float* partial = reinterpret_cast<float*>(reinterpret_cast<uint8_t*>(xp) + kPackBytes + 4096u);
+    int* xp_exp = reinterpret_cast<int*>(reinterpret_cast<uint8_t*>(xp) + kGemvPackBytes - kGemvPackExpBytes);   // exponents behind the packed data
+    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;   // table, partial sums, the activations' scale factors
     auto main_launch = [&](const oilhip_weights& t, float* y, uint32_t ld, int kind, int m0, int m1) {
         const uint32_t groups = ((uint32_t)t.rows + 15u) / 16u;
         const uint32_t ks = split_of(kind == 2 ? 8u : 16u);
@@ -398,16 +468,17 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         if (slabs > groups) slabs = groups;
         auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
         hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, xp_exp, y, (uint32_t)t.rows,
-                           (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks);
+                           (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0);
     };
     for (int m0 = 0; m0 < M;) {       // passes of 32 tokens while more than 16 are left, then one of 16 or of 8
         const int left = M - m0;
         const int kind = left <= 8 ? 0 : left <= 16 ? 1 : 2;
         const int m1 = left <= 32 ? M : m0 + 32;
-        const bool cut = split_of(kind == 2 ? 8u : 16u) > 1u;
+        const uint32_t ksp = split_of(kind == 2 ? 8u : 16u);
+        const bool two = ksp == 2u || (ksp > 2u && !ordered);              // row parts that add into y, which then starts at zero
         hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
-                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, cut ? d_y : nullptr, (uint32_t)w.rows, ldy,
-                           w2 && cut ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
+                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
+                           w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, kind, m0, m1);
         OILHIP_HIP(hipGetLastError());
@@ -436,10 +507,14 @@ extern "C" int oilhip_gemv_oil4_f32_noalloc(const oilhip_weights* w, const float
         uint32_t* pack = nullptr;
         if (int e = static_pack_buffer(&pack)) return e;
         rc = launch_gemv_oil4_multi(*w, d_x, nullptr, d_y, M, (uint32_t)w->cols, (uint32_t)w->rows, (uint32_t)M, s, nullptr, nullptr, 0,
-                                    nullptr, pack);
+                                    nullptr, pack, kStaticScratchBytes);
     }
     if (rc == 1 && M > 2 && M <= 4) rc = launch_gemv_oil4(*w, d_x, d_y, M, s);
     if (rc == 1) return fail(OILHIP_E_ARG, "gemv_oil4_f32_noalloc: this shape needs a kernel that allocates; use oilhip_gemv_f32");
     return rc;
 }
 
+extern "C" int oilhip_set_ordered_sums(int ordered) {
+    oilhip::g_ordered_sums_set(ordered);
+    return OILHIP_OK;
+}

@@ -171,7 +171,7 @@ def test_moe_step_full_size():
                 d.close()
     want, zw, dw = O.moe_dispatch(x, dense[0], dense[1], dense[2], idx, wgt, wide=True)
     assert rel_l2(out.cpu().numpy(), want) <= TOL
-    assert rel_l2(out2.cpu().numpy(), out.cpu().numpy()) <= 1e-6
+    assert np.array_equal(out.cpu().numpy().view(np.uint32), out2.cpu().numpy().view(np.uint32))   # the same bits from run to run
     assert dropped == dw == 1
     # the reference adds the 5e5 squared contributions in one FP32 chain (fmaf), the device in double: the chain's own
     # rounding is what separates the two

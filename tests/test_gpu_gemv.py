@@ -121,8 +121,9 @@ def test_oil4_multi_token_counts(rows, cols, M):
     assert err <= TOL
 
 
-# rows wider than 16 blocks are cut along K between workgroups that add into y: the output buffer is cleared by the
-# launch itself (it holds NaNs here), several row tiles per workgroup, parts of unequal length, both pass widths
+# rows wider than 16 blocks are cut along K between workgroups whose sums meet in a workspace and are added in a fixed
+# order (the output buffer holds NaNs before the call), several row tiles per workgroup, parts of unequal length, both
+# pass widths
 @pytest.mark.parametrize("rows,cols,M", [(9000, 8192, 5), (9000, 8192, 17), (5000, 11008, 16), (700, 8448, 24)])
 def test_oil4_multi_token_rows_cut_along_k(rows, cols, M):
     w = gaussian_weights(rows * cols, rows + M)
@@ -131,9 +132,14 @@ def test_oil4_multi_token_rows_cut_along_k(rows, cols, M):
     want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
     with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
         out = torch.full((M, rows), float("nan"), device="cuda")
-        for _ in range(2):                                   # the second call finds the first call's sums in y
+        runs = []
+        for _ in range(3):                                   # later calls find the earlier calls' sums in y and in the workspace
             got = dw.gemv(torch.from_numpy(X).cuda(), out=out).cpu().numpy()
             assert rel_l2(got, want) <= TOL
+            runs.append(got.copy())
+        # the parts are added in a fixed order: the same bits from every launch
+        assert np.array_equal(runs[0].view(np.uint32), runs[1].view(np.uint32))
+        assert np.array_equal(runs[0].view(np.uint32), runs[2].view(np.uint32))
 
 
 # the OIL8 kernel: one and several slabs per row, rows not a multiple of the wave count, several chunks per
