@@ -70,11 +70,37 @@ __device__ __forceinline__ float pack_value(const float* __restrict__ x, const f
     return v;
 }
 
+__global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* __restrict__ p, uint32_t n) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i < n) p[i] = 0u;
+}
+
+// Several batches in one launch (the experts of a mixture-of-experts step): batch j packs M[j] rows of x into
+// xp + xp_off[j] (exponents at xp_exp + exp_off[j]); its rows are list[row0[j] + m] when use_list is set, else
+// row0[j] + m.  The list travels by value with the launch, so the host needs no copy and no synchronisation.
+constexpr int kMaxJobs = 16, kMaxListed = 448;
+struct PackJobs {
+    uint32_t n, wgs_per_job;
+    int M[kMaxJobs], row0[kMaxJobs];
+    uint32_t xp_off[kMaxJobs], exp_off[kMaxJobs];
+    int use_list;
+    int list[kMaxListed];
+};
+
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
               int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
-              float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld) {
+              float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld,
+              const PackJobs jobs) {
     const uint32_t bpr = cols >> 8, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    uint32_t bid = blockIdx.x;
+    int row0 = 0;
+    if (jobs.n) {                                                          // workgroup -> (batch, index within the batch)
+        const uint32_t job = bid / jobs.wgs_per_job;
+        bid -= job * jobs.wgs_per_job;
+        M = jobs.M[job]; row0 = jobs.row0[job];
+        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+    }
     // outputs that the main kernel's two row parts add into start at zero
     const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
     if (yc0)
@@ -85,11 +111,12 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
     // behind the first's); passes of 8 tokens have 8 token columns: columns 0..7 of the operand carry their high
     // parts and columns 8..15 their low parts, in the pieces that otherwise hold the high parts of 16 tokens
     const uint32_t ncol = half ? 8u : 16u, nbg = (bpr + 3u) / 4u;
-    const uint32_t blk = (blockIdx.x % nbg) * 4u + wave, t = (blockIdx.x / nbg) % ncol, tile = blockIdx.x / (nbg * ncol);
+    const uint32_t blk = (bid % nbg) * 4u + wave, t = (bid / nbg) % ncol, tile = bid / (nbg * ncol);
     if (blk >= bpr) return;
     const int m = m0 + 16 * (int)tile + (int)t;
     xp += (size_t)tile * bpr * 4096u;
-    const uint32_t src = m < M ? (tok ? (uint32_t)tok[m] : (uint32_t)m) : 0xFFFFFFFFu;
+    uint32_t src = 0xFFFFFFFFu;
+    if (m < M) src = jobs.n ? (jobs.use_list ? (uint32_t)jobs.list[row0 + m] : (uint32_t)(row0 + m)) : (tok ? (uint32_t)tok[m] : (uint32_t)m);
     const bool live = src < xrows;
     const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u : 0;
     // this lane's two pairs: pair id = lane + 64 k holds positions 2c, 2c+1 of chunk kq + 4h
@@ -138,11 +165,29 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
 // NT = 2: passes of 32 tokens.  A wavefront then owns one block of the row per K-pass (8 blocks per pass) and keeps
 // the split activations of two token tiles of it, so a decoded weight operand serves two matrix instructions per
 // product term; a row tile is two groups of 16 rows.
+// Several tensors of one shape in one launch (the experts of a mixture-of-experts step): workgroup blockIdx.x serves
+// tensor blockIdx.x / wgs_per_job with that tensor's packed activations, batch size and output.
+struct MultiJobs {
+    uint32_t n, wgs_per_job;
+    const uint8_t* W[kMaxJobs];
+    float* y[kMaxJobs];
+    int M[kMaxJobs];
+    uint32_t xp_off[kMaxJobs], exp_off[kMaxJobs], partial_off[kMaxJobs], counter_off[kMaxJobs];
+};
+
 template <bool HALF, int NT>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
                        uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
-                       uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered) {
+                       uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, const MultiJobs jobs) {
+    uint32_t bid = blockIdx.x;
+    if (jobs.n) {
+        const uint32_t job = bid / jobs.wgs_per_job;
+        bid -= job * jobs.wgs_per_job;
+        W = jobs.W[job]; y = jobs.y[job]; M = jobs.M[job];
+        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+        partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
+    }
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
@@ -155,7 +200,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit.  Two parts add into a zeroed
     // y with float atomics (two addends: the sum does not depend on their order); three or more parts write their sums
     // to `partial` and the workgroup that arrives last at the slab's counter adds them in ascending order
-    const uint32_t slab = ksplit > 1u ? blockIdx.x / ksplit : blockIdx.x, part = ksplit > 1u ? blockIdx.x % ksplit : 0u;
+    const uint32_t slab = ksplit > 1u ? bid / ksplit : bid, part = ksplit > 1u ? bid % ksplit : 0u;
     static_assert(NT == 1 || !HALF, "passes of 8 tokens have one token tile");
     constexpr int BPW = NT == 2 ? 1 : 2;                                   // blocks of the row per wavefront and pass
     constexpr uint32_t PB = 8u * BPW;                                      // blocks per pass
@@ -468,7 +513,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         if (slabs > groups) slabs = groups;
         auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
         hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, xp_exp, y, (uint32_t)t.rows,
-                           (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0);
+                           (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0, MultiJobs{});
     };
     for (int m0 = 0; m0 < M;) {       // passes of 32 tokens while more than 16 are left, then one of 16 or of 8
         const int left = M - m0;
@@ -478,7 +523,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         const bool two = ksp == 2u || (ksp > 2u && !ordered);              // row parts that add into y, which then starts at zero
         hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
                            (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
-                           w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2);
+                           w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2, PackJobs{});
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, kind, m0, m1);
         OILHIP_HIP(hipGetLastError());
@@ -488,6 +533,89 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         }
         m0 = m1;
     }
+    return OILHIP_OK;
+}
+
+
+// ---- several batches in one launch (the experts of a mixture-of-experts step) ---------------------------------------
+// Batch b multiplies M[b] <= (8, 16, 32 for kind 0, 1, 2) activation rows with tensor wa[b] (and, with wb, with a
+// second tensor of the same shape: an expert's gate and up projections share their activations).  All tensors have
+// one shape.  The activation rows of batch b are rows list[row0[b] + m] of x when `list` is given (the list is passed
+// by value with the launch), else rows row0[b] + m; with x2 they are silu(x) * x2.  Outputs: ya[b][m * ldy + r].
+// Workspace layout: packed activations and exponents per batch, one counter block and one partial-sum area per job.
+size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t cols) {
+    const uint32_t bpr = (uint32_t)(cols >> 8), NT = kind == 2 ? 2u : 1u, tokens = kind == 0 ? 8u : kind == 1 ? 16u : 32u;
+    const uint32_t pb = kind == 2 ? 8u : 16u, ks = (bpr + pb - 1u) / pb;
+    size_t per_batch = (size_t)NT * bpr * 16384u + (size_t)NT * bpr * 64u;
+    size_t per_job = 4096u + (ks > 2u ? (size_t)ks * tokens * rows * 4u : 0u);
+    return (size_t)nb * per_batch + (size_t)2 * nb * per_job + 256u;
+}
+
+int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const* wa, float* const* ya,
+                                   const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
+                                   const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
+                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s) {
+    if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || kind < 0 || kind > 2 || nlist > kMaxListed) return 1;
+    const oilhip_weights& w0 = *wa[0];
+    if (w0.rows == 0 || w0.rows > 0x7FFFFFFFull || w0.cols > kMaxPackCols || (w0.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
+    if (ws_bytes < gemv_oil4_multi_batches_bytes(kind, nb, w0.rows, w0.cols)) return 1;
+    static std::atomic<uint64_t> attr_done[3];
+    if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>), kMaxLds)) return rc;
+    if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>), kMaxLds)) return rc;
+    if (int rc = ensure_max_lds(attr_done[2], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>), kMaxLds)) return rc;
+    const bool ordered = g_ordered_sums.load(std::memory_order_relaxed) != 0;
+    const uint32_t bpr = (uint32_t)(w0.cols >> 8), NT = kind == 2 ? 2u : 1u, tokens = kind == 0 ? 8u : kind == 1 ? 16u : 32u;
+    const uint32_t pb = kind == 2 ? 8u : 16u;
+    uint32_t ks = (bpr + pb - 1u) / pb;
+    if (ks < 2u || ks > (uint32_t)device_cu_count()) ks = 1u;
+    const size_t xp_dwords = (size_t)NT * bpr * 4096u, exp_ints = (size_t)NT * bpr * 16u;
+    uint8_t* base = static_cast<uint8_t*>(d_ws);
+    uint32_t* xp = reinterpret_cast<uint32_t*>(base);
+    int* xp_exp = reinterpret_cast<int*>(base + (size_t)nb * xp_dwords * 4u);
+    const int njobs = wb ? 2 * nb : nb;
+    uint8_t* jobs_base = base + (size_t)nb * (xp_dwords * 4u + exp_ints * 4u);
+    const size_t part_floats = ks > 2u ? (size_t)ks * tokens * w0.rows : 0u;
+    uint32_t* counter = reinterpret_cast<uint32_t*>(jobs_base);
+    float* partial = reinterpret_cast<float*>(jobs_base + (size_t)njobs * 4096u);
+    if (xp_dwords * (size_t)nb > 0xFFFFFFFFull || part_floats * (size_t)njobs > 0xFFFFFFFFull) return 1;
+
+    PackJobs pj{};
+    pj.n = (uint32_t)nb;
+    pj.wgs_per_job = (kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u);
+    pj.use_list = list ? 1 : 0;
+    for (int i = 0; i < nlist; ++i) pj.list[i] = list[i];
+    MultiJobs mj{};
+    mj.n = (uint32_t)njobs;
+    const uint32_t groups = ((uint32_t)w0.rows + 15u) / 16u;
+    // workgroups per tensor: the launch as a whole fills the device about twice over, so that a workgroup keeps its
+    // table and its activations for many row groups
+    uint32_t slabs = std::max<uint32_t>(1u, 2u * (uint32_t)device_cu_count() / ((uint32_t)njobs * ks));
+    if (slabs > groups) slabs = groups;
+    if (slabs > 1024u) slabs = 1024u;
+    mj.wgs_per_job = slabs * ks;
+    for (int b = 0; b < nb; ++b) {
+        if (M[b] < 1 || M[b] > (int)tokens) return fail(OILHIP_E_ARG, "multi-row batches: a batch exceeds the pass size");
+        pj.M[b] = M[b]; pj.row0[b] = row0[b];
+        pj.xp_off[b] = (uint32_t)(b * xp_dwords); pj.exp_off[b] = (uint32_t)(b * exp_ints);
+        for (int t = 0; t < (wb ? 2 : 1); ++t) {
+            const int j = t * nb + b;
+            const oilhip_weights* w = t ? wb[b] : wa[b];
+            if (!plain_oil4(*w) || w->rows != w0.rows || w->cols != w0.cols) return 1;
+            mj.W[j] = w->d_payload; mj.y[j] = t ? yb[b] : ya[b]; mj.M[j] = M[b];
+            mj.xp_off[j] = pj.xp_off[b]; mj.exp_off[j] = pj.exp_off[b];
+            mj.partial_off[j] = (uint32_t)(j * part_floats); mj.counter_off[j] = (uint32_t)(j * 1024);
+        }
+    }
+    if (ks > 2u && ordered)                                               // the caller's workspace is not known to be zero
+        hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
+    hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
+                       (uint32_t)w0.cols, 0, 0, ldx, xrows, kind == 0 ? 1 : 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
+    OILHIP_HIP(hipGetLastError());
+    const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;
+    auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
+    hipLaunchKernelGGL(kern, dim3(mj.wgs_per_job * (uint32_t)njobs), dim3(512), lds_bytes, s, (const uint8_t*)nullptr, xp, xp_exp, (float*)nullptr,
+                       (uint32_t)w0.rows, (uint32_t)w0.cols, 0, 0, ldy, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0, mj);
+    OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }
 

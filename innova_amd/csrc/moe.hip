@@ -76,12 +76,56 @@ __global__ void __launch_bounds__(256) combine_distinct_kernel(const float* __re
     if (threadIdx.x == 0) atomicAdd(zacc, (part[0] + part[1]) + (part[2] + part[3]));
 }
 
+// The grouped path's combine: every token's contributions in the order the reference adds them (ascending expert,
+// then list order), out[t][d] written once.  The lists travel by value with the launch.
+constexpr int kMaxPairs = 448;
+struct CombineLists {
+    int K;
+    int pair[kMaxPairs];        // pair[t * K + k]: row of o behind the k-th contribution of token t, or -1
+    float wgt[kMaxPairs];       // its weight (<= 0: dropped)
+};
+
+__global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __restrict__ o, uint32_t D, float* __restrict__ out,
+                                                              double* __restrict__ zacc, const CombineLists L) {
+    __shared__ double part[4];
+    const uint32_t d = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
+    double z = 0.0;
+    if (d < D) {
+        float sum = 0.0f;
+        for (int k = 0; k < L.K; ++k) {
+            const int i = L.pair[t * L.K + k];
+            const float w = L.wgt[t * L.K + k];
+            if (i < 0 || !(w > 0.0f)) continue;
+            const float v = w * o[(size_t)i * D + d];
+            sum += v;
+            z += (double)v * (double)v;
+        }
+        out[(size_t)t * D + d] = sum;
+    }
+    for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = z;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicAdd(zacc, (part[0] + part[1]) + (part[2] + part[3]));
+}
+
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
-    int* tok; float* wgt; float* g; float* u; float* o; float* xg; double* z;
-    size_t bytes;
+    int* tok; float* wgt; float* g; float* u; float* o; float* xg; double* z; uint8_t* batch;
+    size_t bytes, batch_bytes;
 };
+
+constexpr int kChunk = 8;       // expert batches per grouped launch (gate and up together are 16 tensors)
+
+// scratch of one grouped launch: the larger of the gate/up side (rows F, cols D) and the down side (rows D, cols F)
+size_t batch_scratch_bytes(int64_t D, int64_t F) {
+    size_t m = 0;
+    for (int kind = 0; kind < 3; ++kind) {
+        m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)F, (uint64_t)D));
+        m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)D, (uint64_t)F));
+    }
+    return m;
+}
 
 Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
     Workspace w{};
@@ -95,6 +139,8 @@ Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
     w.u = (float*)take((size_t)pairs * F * 4);
     w.o = (float*)take((size_t)pairs * D * 4);
     w.xg = (float*)take((size_t)pairs * D * 4);
+    w.batch_bytes = (D % 256 == 0 && F % 256 == 0 && D <= 32768 && F <= 32768) ? batch_scratch_bytes(D, F) : 0;
+    w.batch = take(w.batch_bytes);
     w.bytes = off;
     return w;
 }
@@ -193,6 +239,71 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
     for (int e = 0; e < E; ++e)
         for (int i = begin[(size_t)e] + 1; i < begin[(size_t)e + 1]; ++i)
             if (tok[(size_t)i] == tok[(size_t)i - 1]) distinct[(size_t)e] = 0;
+    if (dropped) *dropped = drop;
+    // ---- grouped path: uniform OIL4 experts, lists small enough to travel with the launches ---------------------
+    // Per pass size (32, 16 or 8 tokens) and chunk of experts: one launch that splits the gathered activations, one
+    // launch over the gate and up projections of all those experts, one that forms silu(gate) * up while splitting it,
+    // one over their down projections; then one combine.  No copy, no synchronisation: the step can be captured.
+    bool grouped = ws.batch_bytes > 0 && (int64_t)tok.size() <= kMaxPairs && T * K <= kMaxPairs && !tok.empty();
+    for (int e = 0; e < E && grouped; ++e) grouped = plain_oil4(*gate[e]) && plain_oil4(*up[e]) && plain_oil4(*down[e]);
+    if (grouped) {
+        const int64_t pairs = (int64_t)tok.size();
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(256), 0, s, (float*)ws.z, (size_t)2);
+        // outputs of row parts that meet through atomics start at zero
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, s, ws.g, (size_t)(pairs * (2 * F + D)));
+        OILHIP_HIP(hipGetLastError());
+        struct Batch { int e, pair0, m; };
+        std::vector<Batch> byKind[3];
+        for (int e = 0; e < E; ++e) {
+            int n = begin[(size_t)e + 1] - begin[(size_t)e], pos = begin[(size_t)e];
+            while (n > 0) {
+                const int take = n > 32 ? 32 : n;
+                byKind[take <= 8 ? 0 : take <= 16 ? 1 : 2].push_back(Batch{e, pos, take});
+                pos += take; n -= take;
+            }
+        }
+        for (int kind = 2; kind >= 0; --kind)
+            for (size_t c0 = 0; c0 < byKind[kind].size(); c0 += kChunk) {
+                const int nb = (int)std::min<size_t>(kChunk, byKind[kind].size() - c0);
+                const oilhip_weights *wg[kChunk], *wu[kChunk], *wd[kChunk];
+                float *yg[kChunk], *yu[kChunk], *yo[kChunk];
+                int Mb[kChunk], r0[kChunk];
+                for (int b = 0; b < nb; ++b) {
+                    const Batch& B = byKind[kind][c0 + b];
+                    wg[b] = gate[B.e]; wu[b] = up[B.e]; wd[b] = down[B.e];
+                    yg[b] = ws.g + (size_t)B.pair0 * F; yu[b] = ws.u + (size_t)B.pair0 * F; yo[b] = ws.o + (size_t)B.pair0 * D;
+                    Mb[b] = B.m; r0[b] = B.pair0;
+                }
+                int rc = launch_gemv_oil4_multi_batches(kind, nb, wg, yg, wu, yu, Mb, r0, tok.data(), (int)tok.size(), d_x, nullptr,
+                                                        (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s);
+                if (rc == 0)
+                    rc = launch_gemv_oil4_multi_batches(kind, nb, wd, yo, nullptr, nullptr, Mb, r0, nullptr, 0, ws.g, ws.u,
+                                                        (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s);
+                if (rc < 0) return rc;
+                if (rc == 1) return fail(OILHIP_E_ARG, "moe_forward: the grouped launch refused a shape it was planned for");
+            }
+        CombineLists L{};
+        L.K = (int)K;
+        for (int64_t i = 0; i < T * K; ++i) { L.pair[i] = -1; L.wgt[i] = 0.0f; }
+        std::vector<int> filled((size_t)T, 0);
+        for (int e = 0; e < E; ++e)                      // ascending expert, list order: the order of the reference's additions
+            for (int i = begin[(size_t)e]; i < begin[(size_t)e + 1]; ++i) {
+                const int t = tok[(size_t)i];
+                L.pair[t * K + filled[(size_t)t]] = i;
+                L.wgt[t * K + filled[(size_t)t]] = wgt[(size_t)i];
+                filled[(size_t)t]++;
+            }
+        hipLaunchKernelGGL(combine_grouped_kernel, dim3((uint32_t)((D + 255) / 256), (uint32_t)T), dim3(256), 0, s, ws.o, (uint32_t)D,
+                           d_out, ws.z, L);
+        OILHIP_HIP(hipGetLastError());
+        if (z_loss) {
+            double z = 0.0;
+            OILHIP_HIP(hipMemcpyAsync(&z, ws.z, 8, hipMemcpyDeviceToHost, s));
+            OILHIP_HIP(hipStreamSynchronize(s));
+            *z_loss = (float)z;
+        }
+        return OILHIP_OK;
+    }
     if (!tok.empty()) {
         OILHIP_HIP(hipMemcpyAsync(ws.tok, tok.data(), tok.size() * 4, hipMemcpyHostToDevice, s));
         OILHIP_HIP(hipMemcpyAsync(ws.wgt, wgt.data(), wgt.size() * 4, hipMemcpyHostToDevice, s));
