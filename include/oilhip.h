@@ -212,6 +212,21 @@ int oilhip_prod_gemv_oil4(const uint8_t* d_w, const uint16_t* d_cb16, float scal
 int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb256, float scale, const float* d_x,
                           float* d_y, int M, int K, int batch, void* stream);
 
+/* oil::adapters::prod::KernelPerf + profile_gemv_{spark,oil4,oil8} (include/oil/kernel_production.h:68-82,
+ * src/kernel_production.cpp:433-485): `repeats` launches of the tiled GEMV (batch 1) timed between two events on
+ * `stream`, after one untimed launch.  kind 0 SPARK (d_cb unused), 4 OIL4 (d_cb = 16 FP16 entries), 8 OIL8 (d_cb =
+ * 256 floats).  bytes_read / bytes_written / gflops use the reference's formulas; `cycles` is the time per launch in
+ * shader clocks at the device's peak frequency, where the reference reads the CPU's timestamp counter.  Waits for
+ * the stream; cannot be captured into a graph. */
+typedef struct oilhip_kernel_perf {
+    uint64_t cycles;
+    uint64_t bytes_read;
+    uint64_t bytes_written;
+    double gflops;
+} oilhip_kernel_perf_t;
+int oilhip_profile_gemv(int kind, const uint8_t* d_w, const void* d_cb, float scale, const float* d_x, float* d_y,
+                        int M, int K, int repeats, oilhip_kernel_perf_t* out, void* stream);
+
 /* oil::engines::OIL{8,4,2}Engine::quant_gemm (include/oil/oil_engines.h:49,78,151;
  * src/oil_engines_oil8.cpp:197-216, oil4.cpp:238-261, oil2.cpp:210-229):
  *   C[m*N+n] = sum_k A[m*K+k] * cb[code(k*N+n)],  [K][N] packed codes, bits in {2,4,8} */
@@ -234,6 +249,31 @@ int oilhip_engine_dequant(int bits, const uint8_t* d_idx, const float* d_cb, int
                           int64_t block, float* d_out, void* stream);
 int oilhip_engine_dense_gemm(int kind, const float* d_a, const void* d_b, const float* d_scales, int64_t block,
                              float* d_c, int64_t M, int64_t N, int64_t K, void* stream);
+
+/* oil::kernel::tl1_gemm (kind 1) / tl2_gemm (kind 2) (include/oil/kernel.h:11-18, src/kernel_tl.cpp:32-90,124-184):
+ * d_w holds one packed row of K two-bit ternary codes per (m, n) pair -- (K+3)/4 bytes for TL1, ((K+11)/12)*3 for
+ * TL2 --, d_act is [N][K] FP32, quantized per row to int8 with scale 127 / max|a| as the reference does;
+ * d_out[m*N+n] = (sum of products) / scale[n], TL1 with every pair sum clamped to int8 first.  Bit-identical to the
+ * reference.  TL2 needs K % 3 == 0 (beyond that the reference reads past the activation row): OILHIP_E_ARG otherwise. */
+int oilhip_tl_gemm(int kind, const uint8_t* d_w, const float* d_act, float* d_out, int M, int N, int K, void* stream);
+
+/* backend::ComputeBackend's dense FP32 operations (include/oil/backend.h:49-80) on device pointers, with the meaning
+ * of their CPU bodies in src/math.cpp (gemv :50-70, gemm :72-95, relu/gelu/silu :97-126, layer_norm :146-178,
+ * rms_norm :180-203, softmax :205-247, add/mul/scale :249-283): what a gfx950 backend object behind
+ * ComputeBackend::create runs.  Row-major, contiguous.
+ *   gemm    : C[M][N] = alpha * A[M][K] . B[K][N] + beta * C      gemv : y[M] = alpha * A[M][N] . x + beta * y
+ *   norm    : kind 0 layer_norm (mean/variance in double, gamma and beta), kind 1 rms_norm (gamma only, d_beta
+ *             unused), over `rows` rows of n
+ *   softmax : over `dim` entries that lie `inner` apart, for each of outer x inner lines
+ *   map     : op 0 relu, 1 gelu (erf form), 2 silu, 3 a + b, 4 a * b, 5 s * a, 6 fill with s                  */
+int oilhip_dense_gemm_f32(float alpha, const float* d_a, const float* d_b, float beta, float* d_c,
+                          int64_t M, int64_t N, int64_t K, void* stream);
+int oilhip_dense_gemv_f32(float alpha, const float* d_a, const float* d_x, float beta, float* d_y,
+                          int64_t M, int64_t N, void* stream);
+int oilhip_dense_norm_f32(int kind, const float* d_x, const float* d_gamma, const float* d_beta, float eps,
+                          float* d_y, int64_t rows, int64_t n, void* stream);
+int oilhip_dense_softmax_f32(const float* d_x, float* d_y, int64_t outer, int64_t dim, int64_t inner, void* stream);
+int oilhip_dense_map_f32(int op, const float* d_a, const float* d_b, float s, float* d_y, int64_t n, void* stream);
 
 /* ------------------------------------------------------------ decode-step pieces
  * oilhip_weights_stack_rows : several uploaded tensors of one width (full 256-weight blocks only) as one tensor of

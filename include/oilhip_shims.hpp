@@ -16,7 +16,12 @@
 #include <vector>
 
 #if __has_include("oil/types.h")
+// Inside the reference tree: the reference's own declarations are the interface, and the shim sources define them.
+#define OILHIP_REFERENCE_TREE 1
 #include "oil/types.h"
+#include "oil/block_codec.h"
+#include "oil/kernel.h"
+#include "oil/kernel_production.h"
 #else
 namespace oil {
 // include/oil/types.h:19-35 (values pinned by tests/test_format.cpp:183-186)
@@ -30,10 +35,6 @@ class Error : public std::runtime_error {
 public:
     explicit Error(const std::string& msg) : std::runtime_error(msg) {}
 };
-}  // namespace oil
-#endif
-
-namespace oil {
 
 // include/oil/block_codec.h:55-63
 bool quantize_block_all(Format fmt, const float* w, int n, std::vector<uint8_t>& indices, std::vector<uint8_t>& codebook);
@@ -55,7 +56,23 @@ void gemv_oil8_tiled(const uint8_t* indices, const float* codebook, float scale,
 void gemv_spark_batch(const uint8_t* packed_w, float scale, const float* X, float* Y, int M, int N, int K);
 void gemv_oil4_batch(const uint8_t* packed_indices, const uint16_t* codebook, float scale, const float* X, float* Y, int M, int N, int K);
 void gemv_oil8_batch(const uint8_t* indices, const float* codebook, float scale, const float* X, float* Y, int M, int N, int K);
+// include/oil/kernel_production.h:68-82.  `cycles` is the time per launch in shader clocks at the device's peak
+// frequency (the reference reads the CPU's timestamp counter); the byte counts and gflops follow the reference's
+// formulas (src/kernel_production.cpp:433-485).
+struct KernelPerf {
+    uint64_t cycles = 0;
+    uint64_t bytes_read = 0;
+    uint64_t bytes_written = 0;
+    double   gflops = 0.0;
+};
+KernelPerf profile_gemv_spark(const uint8_t* packed_w, float scale, const float* x, float* y, int M, int K, int repeats = 100);
+KernelPerf profile_gemv_oil4(const uint8_t* packed_indices, const uint16_t* codebook, float scale, const float* x, float* y, int M, int K, int repeats = 100);
+KernelPerf profile_gemv_oil8(const uint8_t* indices, const float* codebook, float scale, const float* x, float* y, int M, int K, int repeats = 100);
 }  // namespace adapters::prod
+}  // namespace oil
+#endif
+
+namespace oil {
 
 namespace gfx950 {
 
@@ -63,6 +80,19 @@ namespace gfx950 {
 // C[m*N+n] = sum_k A[m*K+k] * codebook[code(k*N+n)].
 void engine_quant_gemm(int bits, const float* a, const uint8_t* b_idx, const float* codebook, float* c,
                        int64_t M, int64_t N, int64_t K);
+// Bodies of OIL{8,4,2}Engine::dequant_tensor (oil_engines.h:48,77,150; scales == nullptr: n packed codes ->
+// codebook values) and of OIL8Engine / OIL4Engine::dequantize_per_block (:43-44, :72-73; one index byte per weight,
+// OIL8: one scale per block, OIL4: {center, half_range} per block).
+void engine_dequant(int bits, const uint8_t* indices, const float* codebook, int64_t n, const float* scales,
+                    int64_t block_size, float* out);
+// Bodies of the engines whose B operand is not a codebook index, [K][N] flat layout: kind 1 Oil1Engine::quant_gemm
+// (oil_engines.h:123; b = one float per 32 flat positions), 3 SparkEngine::quant_gemm (:103; b = 2-bit codes, scales[flat /
+// block_size]), 16 OIL16Engine::quant_gemm (:167; b = FP16 bits), 32 OIL32Engine::quant_gemm (:183; b = FP32).
+void engine_dense_gemm(int kind, const float* a, const void* b, const float* scales, int64_t block_size, float* c,
+                       int64_t M, int64_t N, int64_t K);
+// Bodies of tl1_gemm (kind 1) / tl2_gemm (kind 2) (include/oil/kernel.h:11-18) on host pointers: weights = one packed
+// row of K ternary codes per (m, n), activations [N][K], output [M][N].
+void tl_gemm(int kind, const uint8_t* weights, const float* activations, float* output, int M, int N, int K);
 
 // One block as the .oil file stores it (OILWriter::write_block, src/oil_format.cpp:219-233).
 struct BlockRef {

@@ -6,10 +6,10 @@ include/oilhip.h); importing works without a GPU, calling a kernel does not.
 """
 from .formats import Format, format_bpw, FULL_BLOCK_BYTES, WIRE_BLOCK  # noqa: F401
 from ._lib import OilHipError, lib, probe  # noqa: F401
-from . import block_codec, format_planner, kernel, layers, moe  # noqa: F401
+from . import backend, block_codec, format_planner, kernel, layers, moe  # noqa: F401
 from .kv_cache import OIL4KVCache  # noqa: F401
 from .weights import DeviceWeights  # noqa: F401
 from .oil_format import OILReader, write_oil  # noqa: F401
 
 __all__ = ["Format", "format_bpw", "FULL_BLOCK_BYTES", "WIRE_BLOCK", "OilHipError", "lib", "probe",
-           "block_codec", "format_planner", "kernel", "layers", "moe", "DeviceWeights", "OILReader", "write_oil"]
+           "backend", "block_codec", "format_planner", "kernel", "layers", "moe", "DeviceWeights", "OILReader", "write_oil"]

@@ -75,6 +75,13 @@ _SIGNATURES = {
     "oilhip_gemv_oil4_f32_noalloc": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_set_ordered_sums": (C.c_int, [C.c_int]),
     "oilhip_gemm_bf16": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_profile_gemv": (C.c_int, [C.c_int, vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp]),
+    "oilhip_tl_gemm": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
+    "oilhip_dense_gemm_f32": (C.c_int, [C.c_float, vp, vp, C.c_float, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
+    "oilhip_dense_gemv_f32": (C.c_int, [C.c_float, vp, vp, C.c_float, vp, C.c_int64, C.c_int64, vp]),
+    "oilhip_dense_norm_f32": (C.c_int, [C.c_int, vp, vp, vp, C.c_float, vp, C.c_int64, C.c_int64, vp]),
+    "oilhip_dense_softmax_f32": (C.c_int, [vp, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
+    "oilhip_dense_map_f32": (C.c_int, [C.c_int, vp, vp, C.c_float, vp, C.c_int64, vp]),
     "oilhip_flat_oil8_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_flat_oil4_gemm": (C.c_int, [vp, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_prod_gemv_spark": (C.c_int, [vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp]),

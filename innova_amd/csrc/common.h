@@ -46,7 +46,7 @@ int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes);
 // one and the old one stays allocated.  No allocation can happen while the stream is being captured, so the first
 // call of a given size on a stream has to be made outside capture; otherwise the call fails with OILHIP_E_ARG.
 // New buffers are zero-filled.
-enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1 };
+enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1, kScratchTl = 2 };
 int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
 // Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream

@@ -465,6 +465,49 @@ int oilhip_prod_gemv_oil8(const uint8_t* d_w, const float* d_cb, float scale, co
     return OILHIP_OK;
 }
 
+// profile_gemv_{spark,oil4,oil8} (src/kernel_production.cpp:433-485): `repeats` launches of the tiled GEMV between two
+// events on `stream`; waits for them.  Not capturable.
+int oilhip_profile_gemv(int kind, const uint8_t* d_w, const void* d_cb, float scale, const float* d_x, float* d_y,
+                        int M, int K, int repeats, oilhip_kernel_perf_t* out, void* stream) {
+    if (!out) return fail(OILHIP_E_ARG, "profile_gemv: null result");
+    if (kind != 0 && kind != 4 && kind != 8) return fail(OILHIP_E_ARG, "profile_gemv: kind must be 0 (SPARK), 4 (OIL4) or 8 (OIL8)");
+    if (repeats < 1) repeats = 1;
+    auto run = [&]() {
+        return kind == 0 ? oilhip_prod_gemv_spark(d_w, scale, d_x, d_y, M, K, 1, stream)
+             : kind == 4 ? oilhip_prod_gemv_oil4(d_w, static_cast<const uint16_t*>(d_cb), scale, d_x, d_y, M, K, 1, stream)
+                         : oilhip_prod_gemv_oil8(d_w, static_cast<const float*>(d_cb), scale, d_x, d_y, M, K, 1, stream);
+    };
+    if (int rc = run()) return rc;                    // first-use set-up stays outside the timed launches
+    auto s = static_cast<hipStream_t>(stream);
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    OILHIP_HIP(hipEventCreate(&e0));
+    if (hipError_t e = hipEventCreate(&e1); e != hipSuccess) {
+        (void)hipEventDestroy(e0);
+        return fail(OILHIP_E_DEVICE, std::string("hipEventCreate: ") + hipGetErrorString(e));
+    }
+    int rc = OILHIP_OK;
+    float ms = 0.f;
+    hipError_t he = hipEventRecord(e0, s);
+    for (int r = 0; r < repeats && rc == OILHIP_OK && he == hipSuccess; ++r) rc = run();
+    if (he == hipSuccess) he = hipEventRecord(e1, s);
+    if (he == hipSuccess) he = hipEventSynchronize(e1);
+    if (he == hipSuccess) he = hipEventElapsedTime(&ms, e0, e1);
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    if (rc != OILHIP_OK) return rc;
+    if (he != hipSuccess) return fail(OILHIP_E_DEVICE, std::string("profile_gemv: ") + hipGetErrorString(he));
+    int dev = 0, khz = 0;
+    OILHIP_HIP(hipGetDevice(&dev));
+    OILHIP_HIP(hipDeviceGetAttribute(&khz, hipDeviceAttributeClockRate, dev));
+    const double sec = (double)ms * 1e-3 / repeats;
+    const uint64_t m = (uint64_t)(M > 0 ? M : 0), k = (uint64_t)(K > 0 ? K : 0);
+    out->cycles = (uint64_t)(sec * (double)khz * 1e3);            // shader clocks at the device's peak frequency
+    out->bytes_read = kind == 0 ? m * k * 2 : kind == 4 ? m * k / 2 + m * k * 4 : m * k + m * 1024;   // the reference's formulas
+    out->bytes_written = m * 4;
+    out->gflops = sec > 0.0 ? 2.0 * (double)m * (double)k / (sec * 1.0e9) : 0.0;
+    return OILHIP_OK;
+}
+
 int oilhip_engine_quant_gemm(int bits, const float* d_a, const uint8_t* d_b, const float* d_cb, float* d_c,
                              int64_t M, int64_t N, int64_t K, void* stream) {
     if (int rc = check(d_a, d_b, d_cb, d_c, M, N, K)) return rc;

@@ -135,9 +135,83 @@ void gemv_oil8_tiled(const uint8_t* w, const float* cb, float scale, const float
     gemv_oil8_batch(w, cb, scale, x, y, M, 1, K);
 }
 
+
+namespace {
+KernelPerf profile(int kind, const uint8_t* w, size_t w_bytes, const void* cb, size_t cb_bytes, float scale,
+                   const float* x, float* y, int M, int K, int repeats) {
+    KernelPerf p;
+    if (M <= 0) return p;
+    Dev<uint8_t> dw(w, w_bytes), dc(static_cast<const uint8_t*>(cb), cb_bytes);
+    Dev<float> dx(x, sz(K)), dy(nullptr, sz(M));
+    oilhip_kernel_perf_t r{};
+    ok(oilhip_profile_gemv(kind, dw.get(), dc.get(), scale, dx.get(), dy.get(), M, K, repeats, &r, nullptr), "profile_gemv");
+    dy.to_host(y);
+    p.cycles = r.cycles;
+    p.bytes_read = r.bytes_read;
+    p.bytes_written = r.bytes_written;
+    p.gflops = r.gflops;
+    return p;
+}
+}  // namespace
+
+KernelPerf profile_gemv_spark(const uint8_t* w, float scale, const float* x, float* y, int M, int K, int repeats) {
+    return profile(0, w, sz(M) * ((sz(K) + 3) / 4), nullptr, 0, scale, x, y, M, K, repeats);
+}
+KernelPerf profile_gemv_oil4(const uint8_t* w, const uint16_t* cb, float scale, const float* x, float* y, int M, int K, int repeats) {
+    return profile(4, w, sz(M) * ((sz(K) + 1) / 2), cb, 32, scale, x, y, M, K, repeats);
+}
+KernelPerf profile_gemv_oil8(const uint8_t* w, const float* cb, float scale, const float* x, float* y, int M, int K, int repeats) {
+    return profile(8, w, sz(M) * sz(K), cb, 1024, scale, x, y, M, K, repeats);
+}
+
 }  // namespace adapters::prod
 
 namespace gfx950 {
+
+void engine_dequant(int bits, const uint8_t* indices, const float* codebook, int64_t n, const float* scales,
+                    int64_t block_size, float* out) {
+    if (n <= 0) return;
+    if (bits != 2 && bits != 4 && bits != 8) throw Error("engine_dequant: bits must be 2, 4 or 8");
+    const size_t idx_bytes = scales ? sz(n) : (sz(n) * (size_t)bits + 7) / 8;
+    const size_t nblocks = scales && block_size > 0 ? (sz(n) + sz(block_size) - 1) / sz(block_size) : 0;
+    Dev<uint8_t> di(indices, idx_bytes);
+    Dev<float> dc(codebook, (size_t)1 << bits), ds(scales, nblocks * (bits == 4 ? 2 : 1)), dout(nullptr, sz(n));
+    ok(oilhip_engine_dequant(bits, di.get(), dc.get(), n, scales ? ds.get() : nullptr, block_size, dout.get(), nullptr),
+       "engine_dequant");
+    dout.to_host(out);
+}
+
+void engine_dense_gemm(int kind, const float* a, const void* b, const float* scales, int64_t block_size, float* c,
+                       int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0) return;
+    const size_t flat = sz(K) * sz(N);
+    size_t b_bytes = 0, nscales = 0;
+    switch (kind) {
+        case 1: b_bytes = ((flat + 31) / 32) * 4; break;
+        case 3:
+            if (block_size <= 0) throw Error("engine_dense_gemm: the SPARK engine needs a block size");
+            b_bytes = (flat + 3) / 4;
+            nscales = (flat + sz(block_size) - 1) / sz(block_size);
+            break;
+        case 16: b_bytes = flat * 2; break;
+        case 32: b_bytes = flat * 4; break;
+        default: throw Error("engine_dense_gemm: kind must be 1, 3, 16 or 32");
+    }
+    Dev<float> da(a, sz(M) * sz(K)), ds(scales, nscales), out(nullptr, sz(M) * sz(N));
+    Dev<uint8_t> db(static_cast<const uint8_t*>(b), b_bytes);
+    ok(oilhip_engine_dense_gemm(kind, da.get(), db.get(), nscales ? ds.get() : nullptr, block_size, out.get(), M, N, K, nullptr),
+       "engine_dense_gemm");
+    out.to_host(c);
+}
+
+void tl_gemm(int kind, const uint8_t* weights, const float* activations, float* output, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return;
+    const size_t row = kind == 1 ? (sz(K) + 3) / 4 : ((sz(K) + 11) / 12) * 3;
+    Dev<uint8_t> dw(weights, sz(M) * sz(N) * row);
+    Dev<float> da(activations, sz(N) * sz(K)), dout(nullptr, sz(M) * sz(N));
+    ok(oilhip_tl_gemm(kind, dw.get(), da.get(), dout.get(), M, N, K, nullptr), "tl_gemm");
+    dout.to_host(output);
+}
 
 void engine_quant_gemm(int bits, const float* a, const uint8_t* b_idx, const float* codebook, float* c,
                        int64_t M, int64_t N, int64_t K) {

@@ -5,6 +5,8 @@ per call, as the reference's host-pointer signatures imply) or cuda tensors
 (used in place); results come back in the same kind."""
 from __future__ import annotations
 
+import ctypes as C
+
 import numpy as np
 
 from . import _lib
@@ -141,3 +143,68 @@ def engine_dequant(bits: int, indices, codebook, n: int, scales=None, block_size
     _lib.check(_lib.lib().oilhip_engine_dequant(bits, i.data_ptr(), c.data_ptr(), n, sd.data_ptr() if sd is not None else None,
                                                 int(block_size), out.data_ptr(), _lib.current_stream()))
     return _ret(out, d1)
+
+
+def _tl(kind, weights, activations, M, N, K):
+    import torch
+    w, d1 = _dev(weights, np.uint8)
+    a, d2 = _dev(activations, np.float32)
+    out = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    _lib.check(_lib.lib().oilhip_tl_gemm(kind, w.data_ptr(), a.data_ptr(), out.data_ptr(), M, N, K, _lib.current_stream()))
+    return _ret(out, d1 and d2)
+
+
+def tl1_gemm(weights, activations, M: int, N: int, K: int):
+    """SPARK lookup kernel, pairs (kernel.h:11-12, src/kernel_tl.cpp:32-90): one packed row of K ternary codes per
+    (m, n), activations [N][K] quantized per row to int8; every pair sum is clamped to int8 before it is added."""
+    return _tl(1, weights, activations, M, N, K)
+
+
+def tl2_gemm(weights, activations, M: int, N: int, K: int):
+    """SPARK lookup kernel, triples (kernel.h:17-18, src/kernel_tl.cpp:124-184); K must be a multiple of 3."""
+    return _tl(2, weights, activations, M, N, K)
+
+
+class KernelPerf:
+    """include/oil/kernel_production.h:68-73.  `cycles` counts shader clocks at the device's current frequency
+    (the reference counts CPU timestamp ticks); the byte formulas are the reference's own
+    (src/kernel_production.cpp:433-485)."""
+
+    def __init__(self, cycles=0, bytes_read=0, bytes_written=0, gflops=0.0):
+        self.cycles, self.bytes_read, self.bytes_written, self.gflops = cycles, bytes_read, bytes_written, gflops
+
+    def __repr__(self):
+        return (f"KernelPerf(cycles={self.cycles}, bytes_read={self.bytes_read}, "
+                f"bytes_written={self.bytes_written}, gflops={self.gflops:.3f})")
+
+
+class _Perf(C.Structure):            # oilhip_kernel_perf_t
+    _fields_ = [("cycles", C.c_uint64), ("bytes_read", C.c_uint64), ("bytes_written", C.c_uint64), ("gflops", C.c_double)]
+
+
+def _profile(kind, w, cb, cb_dtype, scale, x, M, K, repeats):
+    import torch
+    wd, _ = _dev(w, np.uint8)
+    xd, _ = _dev(x, np.float32)
+    cd = _dev(cb, cb_dtype)[0] if cb is not None else None
+    y = torch.empty(M, dtype=torch.float32, device="cuda")
+    p = _Perf()
+    _lib.check(_lib.lib().oilhip_profile_gemv(kind, wd.data_ptr(), cd.data_ptr() if cd is not None else None, float(scale),
+                                              xd.data_ptr(), y.data_ptr(), M, K, int(repeats), C.addressof(p),
+                                              _lib.current_stream()))
+    return KernelPerf(p.cycles, p.bytes_read, p.bytes_written, p.gflops), y
+
+
+def profile_gemv_spark(packed_w, scale, x, M: int, K: int, repeats: int = 100):
+    """kernel_production.h:75-76: `repeats` launches of gemv_spark_tiled between two events."""
+    return _profile(0, packed_w, None, None, scale, x, M, K, repeats)[0]
+
+
+def profile_gemv_oil4(packed_indices, codebook, scale, x, M: int, K: int, repeats: int = 100):
+    """kernel_production.h:78-79."""
+    return _profile(4, packed_indices, codebook, np.uint16, scale, x, M, K, repeats)[0]
+
+
+def profile_gemv_oil8(indices, codebook, scale, x, M: int, K: int, repeats: int = 100):
+    """kernel_production.h:81-82."""
+    return _profile(8, indices, codebook, np.float32, scale, x, M, K, repeats)[0]

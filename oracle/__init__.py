@@ -92,6 +92,8 @@ def lib():
         L.orc_engine_quant_gemm.restype = None
         L.orc_engine_quant_gemm.argtypes = [C.c_int, _f32p, _u8p, _f32p, _f32p,
                                             C.c_int64, C.c_int64, C.c_int64, C.c_int]
+        L.orc_tl_gemm.restype = None
+        L.orc_tl_gemm.argtypes = [C.c_int, _u8p, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
         _lib = L
     return _lib
 
@@ -129,6 +131,8 @@ def ref(simd: bool = True):
             R.ref_engine_quant_gemm.restype = None
             R.ref_engine_quant_gemm.argtypes = [C.c_int, _f32p, _u8p, _f32p,
                                                 C.c_int64, C.c_int64, C.c_int64]
+            R.ref_tl_gemm.restype = None
+            R.ref_tl_gemm.argtypes = [C.c_int, _u8p, C.c_size_t, _f32p, _f32p, C.c_int, C.c_int, C.c_int]
             _ref[key] = R
     return _ref[key]
 
@@ -278,6 +282,23 @@ def engine_quant_gemm(bits, A, b_idx, cb, M, N, K, as_double=False):
     out = np.zeros(M * N, dtype=np.float32)
     lib().orc_engine_quant_gemm(bits, _p(A, _f32p), _p(b_idx, _u8p), _p(cb, _f32p), _p(out, _f32p),
                                 M, N, K, int(as_double))
+    return out.reshape(M, N)
+
+
+def tl_row_bytes(kind: int, K: int) -> int:
+    return (K + 3) // 4 if kind == 1 else ((K + 11) // 12) * 3
+
+
+def tl_gemm(kind, w, a, M, N, K, fn=None):
+    """tl1_gemm (kind 1) / tl2_gemm (kind 2); fn = ref().ref_tl_gemm runs the compiled reference instead."""
+    w = np.ascontiguousarray(w, dtype=np.uint8)
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    assert w.size >= M * N * tl_row_bytes(kind, K) and a.size == N * K
+    out = np.zeros(M * N, dtype=np.float32)
+    if fn is None:
+        lib().orc_tl_gemm(kind, _p(w, _u8p), _p(a, _f32p), _p(out, _f32p), M, N, K)
+    else:
+        fn(kind, _p(w, _u8p), w.size, _p(a, _f32p), _p(out, _f32p), M, N, K)
     return out.reshape(M, N)
 
 

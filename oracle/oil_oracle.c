@@ -26,6 +26,10 @@
  *   orc_gemv_*                           compiled reference built without SIMD
  *                                        flags (its scalar bodies).
  *   orc_engine_quant_gemm                compiled reference engines.
+ *   orc_tl_gemm                          compiled reference (golden fixture incl.
+ *                                        the shape of tests/test_protected.cpp:177-
+ *                                        192); plain integer matrix product when
+ *                                        no pair sum leaves int8 (brute force).
  *
  * Compile with -ffp-contract=off: fusions the reference build performs are
  * written out as fmaf()/fma() below.
@@ -1243,4 +1247,45 @@ void orc_kv_get_range(const uint8_t* idx, const uint16_t* cb, int64_t idx_bytes,
             left -= chunk; flat += chunk; dst += chunk;
         }
     }
+}
+
+/* ------------------------------------------------------------ SPARK lookup kernels */
+/* src/kernel_tl.cpp:32-90 (TL1) and :124-184 (TL2). */
+void orc_tl_gemm(int kind, const uint8_t* w, const float* a, float* out, int M, int N, int K) {
+    if (M <= 0 || N <= 0 || K < 0) return;
+    const size_t row_bytes = kind == 1 ? (size_t)((K + 3) / 4) : (size_t)(((K + 11) / 12) * 3);
+    int8_t* q = (int8_t*)malloc((size_t)N * (size_t)(K > 0 ? K : 1));
+    float* scales = (float*)malloc(sizeof(float) * (size_t)N);
+    for (int n = 0; n < N; ++n) {                          /* :39-50 / :131-143 */
+        float mx = 0.f;
+        for (int k = 0; k < K; ++k) { const float v = fabsf(a[(size_t)n * K + k]); if (v > mx) mx = v; }
+        if (mx < 1e-10f) mx = 1e-10f;
+        scales[n] = 127.0f / mx;
+        for (int k = 0; k < K; ++k) q[(size_t)n * K + k] = (int8_t)roundf(a[(size_t)n * K + k] * scales[n]);
+    }
+    for (int m = 0; m < M; ++m)
+        for (int n = 0; n < N; ++n) {
+            const uint8_t* wr = w + ((size_t)m * N + n) * row_bytes;
+            const int8_t* ar = q + (size_t)n * K;
+            int64_t total = 0;
+            for (int k = 0; k < K; ++k) {
+                const int c = (wr[k / 4] >> ((k % 4) * 2)) & 3;   /* 0 -> -1, 1 -> 0, else +1 (:68-71, :112-117) */
+                const int wv = c == 0 ? -1 : (c == 1 ? 0 : 1);
+                if (kind == 1 && k + 1 < K && (k & 1) == 0) {     /* pair sum stored as int8 (:22-24) */
+                    const int c1 = (wr[k / 4] >> ((k % 4) * 2 + 2)) & 3;
+                    const int w1 = c1 == 0 ? -1 : (c1 == 1 ? 0 : 1);
+                    int sum = (int)ar[k] * wv + (int)ar[k + 1] * w1;
+                    if (sum < -128) sum = -128;
+                    if (sum > 127) sum = 127;
+                    total += sum;
+                    ++k;
+                } else {
+                    total += (int)ar[k] * wv;                     /* odd tail of TL1 (:75-81); every term of TL2 */
+                }
+            }
+            if (kind == 1) total = (int32_t)total;
+            out[(size_t)m * N + n] = (float)total / scales[n];
+        }
+    free(q);
+    free(scales);
 }

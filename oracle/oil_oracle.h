@@ -136,6 +136,12 @@ void orc_engine_quant_gemm(int bits, const float* A, const uint8_t* b_idx,
                            const float* cb, float* C,
                            int64_t M, int64_t N, int64_t K, int as_double);
 
+/* SPARK lookup-table kernels tl1_gemm (kind 1, src/kernel_tl.cpp:32-90) and tl2_gemm (kind 2, :124-184): one packed
+ * row of K two-bit ternary codes per (m, n) pair, activations [N][K] quantized per row to int8 with scale
+ * 127 / max|a|; out[m*N+n] = (sum of products) / scale[n].  TL1 stores every pair sum as int8 (clamped) before it
+ * is added; TL2 does not, and is defined here for K % 3 == 0 (beyond that the reference reads past the row). */
+void orc_tl_gemm(int kind, const uint8_t* w, const float* a, float* out, int M, int N, int K);
+
 /* Engines with a dense or sign-coded B operand, [K][N] flat layout, k ascending, a == 0 skipped, each
  * multiply-add fused as in the -mfma build: kind 1 Oil1Engine (src/oil_engines_oil1.cpp:61-82), 3 SparkEngine
  * (src/oil_engines_spark.cpp:154-186), 16 OIL16Engine (src/oil_engines_fp.cpp:433-451, widening as

@@ -278,6 +278,16 @@ void ref_engine_dequant(int bits, const uint8_t* idx, int64_t n, const float* sc
     }
 }
 
+// include/oil/kernel.h:11-18: tl1_gemm (kind 1) / tl2_gemm (kind 2) over host arrays wrapped in tensors
+void ref_tl_gemm(int kind, const uint8_t* w, size_t w_bytes, const float* a, float* out, int M, int N, int K) {
+    oil::Tensor wt(oil::Shape{(int64_t)w_bytes}, oil::DType::U8), at(oil::Shape{(int64_t)N, (int64_t)K}), ot(oil::Shape{(int64_t)M, (int64_t)N});
+    std::memcpy(wt.data<uint8_t>(), w, w_bytes);
+    std::memcpy(at.data<float>(), a, sizeof(float) * (size_t)N * (size_t)K);
+    if (kind == 1) oil::kernel::tl1_gemm(wt, at, ot, M, N, K);
+    else oil::kernel::tl2_gemm(wt, at, ot, M, N, K);
+    std::memcpy(out, ot.data<float>(), sizeof(float) * (size_t)M * (size_t)N);
+}
+
 // CodebookOIL4::half_to_float / float_to_half (include/oil/codebook.h:79-80)
 float ref_kv_half_to_float(uint16_t h) { return oil::CodebookOIL4::half_to_float(h); }
 uint16_t ref_kv_float_to_half(float f) { return oil::CodebookOIL4::float_to_half(f); }

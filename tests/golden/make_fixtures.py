@@ -553,8 +553,37 @@ def kv_f2h_inputs():
     return bits[~np.isnan(f)]
 
 
+# ---------------------------------------------------------------- SPARK lookup kernels
+# (kind, M, N, K): the shape of the reference's own test (tests/test_protected.cpp:177-192), odd K for TL1's tail,
+# K that is not a multiple of 12 for TL2's last group, a long row, one output
+TL_CASES = [(1, 4, 4, 16), (1, 3, 5, 33), (1, 2, 3, 7), (1, 5, 2, 255), (1, 1, 1, 1), (1, 2, 2, 1200), (1, 6, 9, 4096),
+            (2, 4, 4, 36), (2, 3, 5, 33), (2, 2, 3, 9), (2, 5, 2, 255), (2, 1, 1, 3), (2, 2, 2, 1200), (2, 6, 9, 4095)]
+
+
+def tl_inputs(i):
+    kind, M, N, K = TL_CASES[i]
+    rng = np.random.default_rng(5100 + i)
+    w = rng.integers(0, 256, size=M * N * O.tl_row_bytes(kind, K), dtype=np.uint8)
+    a = (rng.standard_normal((N, K)) * rng.choice([1e-3, 1.0, 50.0], size=(N, 1))).astype(np.float32)
+    a[0, :] = np.where(rng.random(K) < 0.5, -1.0, 1.0) * np.abs(a[0, :]).max()   # a saturated row: TL1's pair sums clamp
+    if N > 1:
+        a[1, :] = 0.0                                                            # all-zero row: the 1e-10 floor
+    return w, a
+
+
+def make_tl():
+    R = O.ref()
+    out = {"cases": np.array(TL_CASES, dtype=np.int32)}
+    for i, (kind, M, N, K) in enumerate(TL_CASES):
+        w, a = tl_inputs(i)
+        out[f"w{i}"], out[f"a{i}"] = w, a
+        out[f"out{i}"] = O.tl_gemm(kind, w, a, M, N, K, fn=R.ref_tl_gemm).view(np.uint32)
+    np.savez_compressed(os.path.join(HERE, "tl.npz"), **out)
+    print("tl.npz written")
+
+
 if __name__ == "__main__":
-    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe", "engines", "kv"]
+    which = sys.argv[1:] or ["codec", "gemv", "flat", "planner", "container", "moe", "engines", "kv", "tl"]
     for name in which:
         {"codec": make_codec, "gemv": make_gemv, "flat": make_flat, "planner": make_planner,
-         "container": make_container, "moe": make_moe, "engines": make_engines, "kv": make_kv}[name]()
+         "container": make_container, "moe": make_moe, "engines": make_engines, "kv": make_kv, "tl": make_tl}[name]()

@@ -180,3 +180,59 @@ def test_engine_dense_gemm_matches_reference(kind):
         dense = np.where(code == 2, 1.0, np.where(code == 0, -1.0, 0.0)) * scales[flat // sh["block"]]
     want = A.astype(np.float64) @ np.asarray(dense, np.float64).reshape(sh["K"], sh["N"])
     assert np.linalg.norm(got - want) / np.linalg.norm(want) < 1e-5
+
+
+# ------------------------------------------------------------------ SPARK lookup kernels (tl1_gemm / tl2_gemm)
+TL = np.load(os.path.join(HERE, "golden", "tl.npz"))
+
+
+@pytest.mark.parametrize("i", range(len(TL["cases"])))
+def test_tl_gemm_matches_golden(i):
+    """Outputs of the compiled reference's tl1_gemm / tl2_gemm (src/kernel_tl.cpp:32-90,124-184), bit for bit."""
+    kind, M, N, K = (int(v) for v in TL["cases"][i])
+    got = O.tl_gemm(kind, TL[f"w{i}"], TL[f"a{i}"], M, N, K)
+    assert np.array_equal(got.view(np.uint32), TL[f"out{i}"])
+
+
+@pytest.mark.parametrize("kind", [1, 2])
+def test_tl_gemm_is_an_integer_matrix_product(kind):
+    """With activations small enough that no pair sum leaves int8, both kernels are an integer matrix product of the
+    int8 activations with the ternary weights, divided by the row's scale."""
+    rng = np.random.default_rng(77 + kind)
+    M, N, K = 5, 4, 48
+    rb = O.tl_row_bytes(kind, K)
+    w = rng.integers(0, 256, size=M * N * rb, dtype=np.uint8)
+    a = rng.uniform(-0.45, 0.45, size=(N, K)).astype(np.float32)
+    a[:, 0], a[:, 1] = 1.0, 0.0                                # the row maximum beside a zero: every other |code| < 64
+    codes = (w.reshape(M * N, rb)[:, :, None] >> (2 * np.arange(4))[None, None, :]) & 3
+    tern = np.where(codes == 0, -1, np.where(codes == 1, 0, 1)).reshape(M * N, rb * 4)[:, :K].reshape(M, N, K)
+    scale = np.float32(127.0) / np.abs(a).max(axis=1).astype(np.float32)
+    v = (a * scale[:, None]).astype(np.float32)
+    q = (np.sign(v) * np.floor(np.abs(v) + np.float32(0.5))).astype(np.int64)      # round half away from zero
+    want = (np.einsum("mnk,nk->mn", tern, q).astype(np.float32) / scale[None, :]).astype(np.float32)
+    got = O.tl_gemm(kind, w, a, M, N, K)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def test_tl1_pair_sums_saturate():
+    """Two full-scale activations under two +1 weights: 127 + 127 is stored as 127 (the table entry is an int8)."""
+    a = np.array([[1.0, 1.0, -1.0, -1.0]], dtype=np.float32)
+    w = np.array([0b10101010], dtype=np.uint8)                  # four +1 weights
+    assert O.tl_gemm(1, w, a, 1, 1, 4)[0, 0] == np.float32((127 - 128) / 127.0)
+    assert O.tl_gemm(2, np.array([0b10101010, 0, 0], np.uint8), np.array([[1.0, 1.0, -1.0]], np.float32), 1, 1, 3)[0, 0] == np.float32(1.0)
+
+
+def test_tl_gemm_matches_compiled_reference():
+    R = O.ref()
+    if R is None:
+        pytest.skip("compiled reference not built")
+    rng = np.random.default_rng(99)
+    for kind in (1, 2):
+        for _ in range(6):
+            M, N = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+            K = int(rng.integers(1, 400)) if kind == 1 else 3 * int(rng.integers(1, 130))
+            w = rng.integers(0, 256, size=M * N * O.tl_row_bytes(kind, K), dtype=np.uint8)
+            a = (rng.standard_normal((N, K)) * 10.0 ** rng.integers(-4, 3)).astype(np.float32)
+            got = O.tl_gemm(kind, w, a, M, N, K)
+            ref = O.tl_gemm(kind, w, a, M, N, K, fn=R.ref_tl_gemm)
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (kind, M, N, K)
