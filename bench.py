@@ -449,6 +449,68 @@ def bench_prefill(torch, ia, payload, blocks):
     return out
 
 
+def bench_read_probe(torch, ia):
+    """What a pure reader reaches on this device with the GEMVs' load pattern (oilhip_read_probe): (a) steady state, one
+    launch over a 902 MB buffer, swept over waves per SIMD (2 / 4 / 8) and loads in flight (2 / 4 / 8), plain and
+    non-temporal loads; (b) the headline's shape of work, 22.5 MB per launch as a graph of 40 dependent launches over
+    40 different slices, which adds the launch gap and the ramp the GEMV pays too."""
+    L = ia._lib.lib()
+    one, copies = 22544384, 40
+    buf = torch.empty(one * copies, dtype=torch.uint8, device="cuda").fill_(1)
+    sink = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
+
+    def launch(ptr, nbytes, u, nt, pat, wgs, thr):
+        ia._lib.check(L.oilhip_read_probe(ptr, nbytes, u, nt, pat, wgs, thr, sink.data_ptr(), ia._lib.current_stream()))
+
+    out, table = {}, {}
+    best = 0.0
+    for wps, (wgs, thr) in ((2, (256, 512)), (4, (512, 512)), (8, (1024, 512))):
+        for u in (2, 4, 8):
+            for nt in (0, 1):
+                for pat in (0, 1):
+                    for _ in range(2):
+                        launch(buf.data_ptr(), buf.numel(), u, nt, pat, wgs, thr)
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(4):
+                        launch(buf.data_ptr(), buf.numel(), u, nt, pat, wgs, thr)
+                    e1.record()
+                    e1.synchronize()
+                    gbs = buf.numel() / (e0.elapsed_time(e1) * 1e-3 / 4) / 1e9
+                    key = f"w{wps}_u{u}_{'nt' if nt else 'ld'}_{'il' if pat else 'ct'}"
+                    table[key] = round(gbs)
+                    best = max(best, gbs)
+    out["read_only_probe_GBps"] = round(best, 1)
+    out["read_only_probe_steady_table_GBps"] = table
+    # the headline's launch pattern
+    stream = torch.cuda.Stream()
+    best_us = None
+    for (wgs, thr, u) in ((256, 512, 4), (512, 512, 4), (1024, 512, 2), (1024, 512, 4)):
+        with torch.cuda.stream(stream):
+            for c in range(copies):
+                launch(buf.data_ptr() + c * one, one, u, 1, 0, wgs, thr)
+            stream.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for c in range(copies):
+                    launch(buf.data_ptr() + c * one, one, u, 1, 0, wgs, thr)
+            for _ in range(3):
+                g.replay()
+            stream.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            for _ in range(50):
+                g.replay()
+            e1.record(stream)
+            e1.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (50 * copies)
+        best_us = us if best_us is None else min(best_us, us)
+    out["read_only_probe_22MB_per_launch_us"] = round(best_us, 2)
+    out["read_only_probe_22MB_per_launch_GBps"] = round(one / best_us / 1e3, 1)
+    return out
+
+
 def bench_dequant_and_engine(torch, ia, payload, blocks):
     """dequantize_block_all over the whole headline tensor (180 MB of FP32 written) and OIL8Engine::quant_gemm at M=1
     (B laid out [K][N], k-ordered FMA chain per output: bit-identical to the reference loop)."""
@@ -703,6 +765,7 @@ def main():
         extra["qkvo_4096x4096_M1_GBps"] = round(pq.size / t_qkvo / 1e9, 1)
         extra["decode_tok_per_s_7B_weight_gemvs_only"] = round(1.0 / (32 * per_layer), 1)
         extra.update(bench_fused_layer(torch, ia, 32 * per_layer))
+        extra.update(bench_read_probe(torch, ia))
         extra.update(bench_tall(torch, ia))
         extra.update(bench_oil8(torch, ia))
         extra.update(bench_dequant_and_engine(torch, ia, payload, blocks))

@@ -255,3 +255,39 @@ def test_oil4_multi_token_activation_ranges(rows, cols, M):
         got = dw.gemv(torch.from_numpy(X).cuda()).cpu().numpy()
     for m in range(M):                                    # row by row: a large row must not hide a small one
         assert rel_l2(got[m], want[m]) <= TOL, m
+
+
+def test_two_streams_run_multi_token_gemvs_concurrently():
+    """Calls on different streams keep separate activation scratch: M = 16 GEMVs of two tensors issued back and forth
+    on two streams, all in flight together, the first and last round checked against the oracle, one in between
+    against a quiet rerun."""
+    shapes = [(2048, 4096), (1024, 11008)]
+    rng = np.random.default_rng(21)
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    handles, wants, outs, xs = [], [], [], []
+    rounds = 12
+    for i, (rows, cols) in enumerate(shapes):
+        w = gaussian_weights(rows * cols, 50 + i)
+        payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+        handles.append(ia.DeviceWeights.from_blocks(payload, blocks, rows, cols))
+        X = rng.standard_normal((rounds, 16, cols)).astype(np.float32)
+        xs.append(torch.from_numpy(X).cuda())
+        wants.append([O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X[r], wide=True) for r in (0, rounds - 1)])
+        outs.append([None] * rounds)
+    torch.cuda.synchronize()
+    for r in range(rounds):
+        for i in (0, 1):
+            with torch.cuda.stream(streams[i]):
+                outs[i][r] = handles[i].gemv(xs[i][r])
+    torch.cuda.synchronize()
+    for i in (0, 1):
+        for r, want in zip((0, rounds - 1), wants[i]):
+            assert rel_l2(outs[i][r].cpu().numpy(), want) <= TOL, (i, r)
+        # the rounds in between: same weights, so linear in the activations
+        mid = outs[i][5].cpu().numpy()
+        with torch.cuda.stream(streams[i]):
+            again = handles[i].gemv(xs[i][5])
+        streams[i].synchronize()
+        assert np.array_equal(mid, again.cpu().numpy()), i
+    for h in handles:
+        h.close()
