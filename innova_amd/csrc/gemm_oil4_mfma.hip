@@ -20,6 +20,7 @@
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
+#include <type_traits>
 
 #include "common.h"
 
@@ -193,32 +194,43 @@ __global__ void __launch_bounds__(256) zero_y_kernel(float* __restrict__ y, size
     for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (size_t)gridDim.x * 256u) y[i] = 0.f;
 }
 
-// Pipelined kernel for larger M: 256 tokens x 128 weight rows per workgroup, 8 wavefronts (4 x 2, each
-// 64 x 64 outputs), 64 columns per step, two LDS tile buffers: while the matrix cores work on step kt, the
-// same wavefronts decode the weights of step kt+1 into the other buffer and the global loads of the
-// following steps are in flight, with one barrier per step.  Per step a thread stages 64 bytes of X' and
-// decodes 8 bytes (16 nibbles) of weights.
-#ifndef OILHIP_GEMM_DEPTH
-#define OILHIP_GEMM_DEPTH 2
-#endif
+// Pipelined kernel for larger M: TBM (256 or 128) tokens x 128 weight rows per workgroup, 8 wavefronts (TBM = 256:
+// 4 x 2 wavefronts of 64 x 64 outputs; TBM = 128: 2 x 4 of 64 x 32), 64 columns per step, two LDS tile buffers.
+// Per step a thread stages TBM / 4 bytes of X' and decodes 8 bytes (16 nibbles) of weights; the global loads of two
+// further steps are in flight.
+//
+// The eight wavefronts work as two groups of four (one per SIMD each), half a step apart: while one group reads
+// its fragments of a step from LDS, the other multiplies, finishes the decode of a later tile and stores it, so
+// the LDS pipe and the matrix cores are busy at the same time instead of one after the other.  Slots are
+// separated by workgroup barriers; group g reads step r in slot 2r + g and multiplies in slot 2r + 1 + g, and
+// during that product stores its share of tile r + 1 + g (buffer (r + 1 + g) & 1): group 0's target was last read
+// in slot 2r - 1 and is needed from slot 2r + 2, group 1's was last read in slot 2r + 1 and is needed from
+// slot 2r + 4.  Both groups pass 2 * steps + 1 barriers after the prologue.
 constexpr int PK = 64;                      // columns per step
 constexpr int PLD = PK;                     // LDS row pitch in bf16: 128 bytes = 8 chunks of 16 bytes; the chunk index of a
                                             // row is XOR-swizzled with (row / 2) % 8 so that the tile stores (2 rows x 8
                                             // chunks per 16 lanes) and the fragment reads (16 rows x 1 chunk) touch every bank once
-constexpr int PBM = 256, PBN = 128;
+constexpr int PBN = 128;
+constexpr int PD = 2;                       // steps of global loads in flight: even, divides K / 64 / 2 (4 measured the same)
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> 1) & 7u; }
 
+template <int TBM>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
                            uint32_t M, uint32_t N, uint32_t K, uint32_t ksplit) {
+    static_assert(TBM == 256 || TBM == 128, "workgroup tiles of 256 or 128 tokens");
+    constexpr int WN = TBM == 256 ? 2 : 4;              // wavefronts along the weight rows
+    constexpr int NJ = PBN / WN / 32;                   // 32-row fragments per wavefront along the weight rows
+    constexpr int AC = TBM / 64;                        // 16-byte pieces of the X' tile per thread
+    constexpr int D = PD;
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);
-    __bf16* As = reinterpret_cast<__bf16*>(lds + kTabBytes);                      // [2][PBM][PLD]
-    __bf16* Bs = As + 2 * PBM * PLD;                                              // [2][PBN][PLD]
+    __bf16* As = reinterpret_cast<__bf16*>(lds + kTabBytes);                      // [2][TBM][PLD]
+    __bf16* Bs = As + 2 * TBM * PLD;                                              // [2][PBN][PLD]
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t wm = wave >> 1, wn = wave & 1u;
-    const uint32_t m0 = blockIdx.y * PBM, n0 = blockIdx.x * PBN;
+    const uint32_t wm = wave / WN, wn = wave % WN;
+    const uint32_t m0 = blockIdx.y * TBM, n0 = blockIdx.x * PBN;
     const uint32_t bpr = K >> 8, KT = K / PK;
 
     {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 512*k
@@ -238,12 +250,11 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     const uint32_t brow = tid >> 2, bq = tid & 3u;                               // weight row of the tile, 8-byte piece of the 32 bytes of a step
     const uint32_t lanebase = (lane & 31u) * 8u;
 
-    constexpr int D = OILHIP_GEMM_DEPTH;        // steps of global loads in flight: even, divides K / 64
-    u32x4 ar[D][4];
+    u32x4 ar[D][AC];
     uint32_t br[D][2], sr[D];
     auto load_regs = [&](int set, uint32_t kt) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < AC; ++c) {
             const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
             ar[set][c] = *reinterpret_cast<const u32x4*>(xa + (size_t)row * K + kt * PK + kc * 8u);
         }
@@ -253,8 +264,8 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
         br[set][1] = __builtin_amdgcn_raw_buffer_load_b32(wrs, off + 4u, 0, 0);
         sr[set] = __builtin_amdgcn_raw_buffer_load_b16(wrs, blk_off, 0, 0);
     };
-    // decode of the next step, split so that its table reads are issued before the fragment reads of the
-    // current step and its arithmetic runs in the shadow of the MFMAs
+    // decode of a later step, split so that its table reads are issued with the fragment reads and its arithmetic
+    // runs in the shadow of the MFMAs
     auto lookup_tiles = [&](int set, f32x2 (&t)[8]) {
 #pragma unroll
         for (int d = 0; d < 2; ++d)
@@ -266,9 +277,9 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     };
     auto finish_tiles = [&](int set, int buf, const f32x2 (&t)[8]) {
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int c = 0; c < AC; ++c) {
             const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
-            *reinterpret_cast<u32x4*>(As + (buf * PBM + row) * PLD + ((kc ^ swz(row)) * 8u)) = ar[set][c];
+            *reinterpret_cast<u32x4*>(As + (buf * TBM + row) * PLD + ((kc ^ swz(row)) * 8u)) = ar[set][c];
         }
         const float scale = __half2float(__ushort_as_half((unsigned short)sr[set]));
         uint32_t packed[8];
@@ -292,73 +303,84 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
         finish_tiles(set, buf, t);
     };
 
-    f32x16 acc[2][2];
+    f32x16 acc[2][NJ];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NJ; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
 
     const uint32_t sw = swz(lane & 31u);
-    auto step_mfmas = [&](int buf) {
-        const __bf16* ap = As + (buf * PBM + wm * 64u + (lane & 31u)) * PLD;
-        const __bf16* bp = Bs + (buf * PBN + wn * 64u + (lane & 31u)) * PLD;
-        bf16x8 a[4][2], b[4][2];
+    bf16x8 fa[4][2], fb[4][NJ];
+    auto read_frags = [&](int buf) {
+        const __bf16* ap = As + (buf * TBM + wm * 64u + (lane & 31u)) * PLD;
+        const __bf16* bp = Bs + (buf * PBN + wn * (NJ * 32u) + (lane & 31u)) * PLD;
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             const uint32_t ch = (((uint32_t)kk * 2u + (lane >> 5)) ^ sw) * 8u;
 #pragma unroll
-            for (int i = 0; i < 2; ++i) a[kk][i] = *reinterpret_cast<const bf16x8*>(ap + i * 32 * PLD + ch);
+            for (int i = 0; i < 2; ++i) fa[kk][i] = *reinterpret_cast<const bf16x8*>(ap + i * 32 * PLD + ch);
 #pragma unroll
-            for (int j = 0; j < 2; ++j) b[kk][j] = *reinterpret_cast<const bf16x8*>(bp + j * 32 * PLD + ch);
+            for (int j = 0; j < NJ; ++j) fb[kk][j] = *reinterpret_cast<const bf16x8*>(bp + j * 32 * PLD + ch);
         }
-        __builtin_amdgcn_sched_barrier(0);
+    };
+    auto do_mfmas = [&]() {
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
             for (int i = 0; i < 2; ++i)
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[kk][i], b[kk][j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < NJ; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[kk][i], fb[kk][j], acc[i][j], 0, 0, 0);
     };
 
-    // K is a multiple of 256, so KT is a multiple of 4 and of D.  Every load and every decode below is issued
-    // unconditionally (steps past the end are clamped to the last one and decoded into a buffer nobody reads):
-    // the number of loads in flight is then a compile-time fact and each wait covers exactly the step it needs.
-    static_assert(D == 2 || D == 4, "D must be even and divide 4");
+    // K is a multiple of 256, so KT is a multiple of 4; a workgroup's share of the steps (all, a half or a quarter of
+    // them) is a multiple of D.  Every load and every decode below is issued unconditionally (steps past the end are
+    // clamped to the last one and decoded into a buffer nobody reads any more): the number of loads in flight is then
+    // a compile-time fact and each wait covers exactly the step it needs.
     // ksplit > 1: workgroup blockIdx.z takes the steps [kbeg, kend) of the row and adds its partial sums to a zeroed Y
     // (two parts at most, so the sum does not depend on which arrives first)
     const uint32_t kbeg = KT / ksplit * blockIdx.z, kend = blockIdx.z + 1u == ksplit ? KT : kbeg + KT / ksplit;
-    const uint32_t last = kend - 1u;
+    const uint32_t last = kend - 1u, nk = kend - kbeg;
     auto clampk = [&](uint32_t k) { return k < last ? k : last; };
 #pragma unroll
     for (int u = 0; u < D; ++u) load_regs(u, clampk(kbeg + (uint32_t)u));
     __syncthreads();                                   // table complete
     store_tiles(0, 0);
     load_regs(0, clampk(kbeg + (uint32_t)D));
-    __syncthreads();
-    // register set s holds the steps congruent to s modulo D.  Iteration kt issues the table reads of step kt+1,
-    // then the fragment reads of step kt (buffer kt & 1), multiplies, finishes the decode of step kt+1 into the
-    // other buffer in the shadow of the MFMAs and refills that register set with step kt+1+D.
-    for (uint32_t kt0 = kbeg; kt0 < kend; kt0 += D) {
-#pragma unroll
-        for (int u = 0; u < D; ++u) {
-            const uint32_t kt = kt0 + u;
-            f32x2 t[8];
-            lookup_tiles((u + 1) % D, t);
-            step_mfmas(u & 1);
-            finish_tiles((u + 1) % D, (u + 1) & 1, t);
-            load_regs((u + 1) % D, clampk(kt + 1u + D));
-            __syncthreads();
+    auto run = [&](auto gc) {
+        constexpr int G = decltype(gc)::value;
+        if constexpr (G == 1) {                        // the late group also brings its share of tile 1
+            store_tiles(1 % D, 1);
+            load_regs(1 % D, clampk(kbeg + 1u + (uint32_t)D));
         }
-    }
+        __syncthreads();                               // tile 0 (and the late group's share of tile 1) in place
+        if constexpr (G == 1) __syncthreads();         // slot 0 belongs to the early group
+        for (uint32_t r0 = 0; r0 < nk; r0 += D) {
+#pragma unroll
+            for (int u = 0; u < D; ++u) {
+                const int set = (u + 1 + G) % D, buf = (u + 1 + G) & 1;
+                f32x2 t[8];
+                lookup_tiles(set, t);
+                read_frags(u & 1);
+                __syncthreads();
+                do_mfmas();
+                finish_tiles(set, buf, t);
+                load_regs(set, clampk(kbeg + r0 + (uint32_t)(u + 1 + G + D)));
+                __syncthreads();
+            }
+        }
+        if constexpr (G == 0) __syncthreads();
+    };
+    if (wave < 4u) run(std::integral_constant<int, 0>{});
+    else run(std::integral_constant<int, 1>{});
 
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const uint32_t col = n0 + (wn * 2 + j) * 32u + (lane & 31u);
+        for (int j = 0; j < NJ; ++j) {
+            const uint32_t col = n0 + (wn * NJ + j) * 32u + (lane & 31u);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t row = m0 + (wm * 2 + i) * 32u + 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u);
@@ -390,7 +412,11 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
     const uint32_t K = (uint32_t)w.cols;
     const bool big = M > 256;
-    const uint32_t BM = big ? 256 : 128;
+    const uint32_t N = (uint32_t)w.rows, ntn = (N + PBN - 1) / PBN, cus = (uint32_t)device_cu_count();
+    // M > 256 runs the pipelined kernel.  Its 256-token tiles decode each weight tile once per 256 tokens; when they
+    // leave more than half of the compute units without a workgroup, 128-token tiles put twice as many to work.
+    const bool wide = big && ntn * (((uint32_t)M + 255u) / 256u) * 2u > cus;
+    const uint32_t BM = wide ? 256 : 128;
     const uint32_t Mpad = ((uint32_t)M + BM - 1) / BM * BM;
     uint16_t* xp = nullptr;
     if (int rc = stream_scratch(s, kScratchGemmX, (size_t)Mpad * K * 2, reinterpret_cast<void**>(&xp))) return rc;
@@ -399,19 +425,25 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
     hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
     OILHIP_HIP(hipGetLastError());
     if (big) {
-        static std::atomic<uint64_t> attr_done{0};
-        if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel), 160 * 1024)) return rc;
-        const uint32_t N = (uint32_t)w.rows;
-        const size_t lds_bytes = (size_t)kTabBytes + 2ull * (PBM + PBN) * PLD * 2;
-        // a grid that leaves half of the compute units idle is cut in two along K (two partial sums into a zeroed Y)
-        const uint32_t tiles = (N + PBN - 1) / PBN * (Mpad / PBM);
-        const uint32_t ksplit = tiles * 2u <= (uint32_t)device_cu_count() && (K / PK) % 8u == 0u ? 2u : 1u;
+        static std::atomic<uint64_t> attr_done[2];
+        // a grid that still leaves half of the units idle is cut in two along K (two partial sums into a zeroed Y)
+        const uint32_t tbm = BM;
+        const uint32_t tiles = ntn * (Mpad / tbm);
+        const uint32_t ksplit = tiles * 2u <= cus && (K / PK) % 8u == 0u ? 2u : 1u;
         if (ksplit > 1u) {
             hipLaunchKernelGGL(zero_y_kernel, dim3((uint32_t)std::min<size_t>(((size_t)M * N + 255) / 256, 4096)), dim3(256), 0, s, d_y, (size_t)M * N);
             OILHIP_HIP(hipGetLastError());
         }
-        hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel, dim3((N + PBN - 1) / PBN, Mpad / PBM, ksplit), dim3(512), lds_bytes, s,
-                           w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
+        const size_t lds_bytes = (size_t)kTabBytes + 2ull * (tbm + PBN) * PLD * 2;
+        if (wide) {
+            if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel<256>), 160 * 1024)) return rc;
+            hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel<256>, dim3(ntn, Mpad / 256u, ksplit), dim3(512), lds_bytes, s,
+                               w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
+        } else {
+            if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel<128>), 160 * 1024)) return rc;
+            hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel<128>, dim3(ntn, Mpad / 128u, ksplit), dim3(512), lds_bytes, s,
+                               w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
+        }
         OILHIP_HIP(hipGetLastError());
         return OILHIP_OK;
     }
