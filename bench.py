@@ -420,6 +420,22 @@ def bench_prefill(torch, ia, payload, blocks):
                 torch.cuda.synchronize()
                 t = e0.elapsed_time(e1) * 1e-3 / 20
                 out[f"prefill_M{M}_N{rows}_TFLOPs"] = round(2.0 * M * rows * cols / t / 1e12, 1)
+    # a tensor that is not uniform OIL4 (here SPARK_Q0): decoded to bf16 slab by slab, then the same kernel over a dense operand
+    ws = make_weights(11008, 4096, seed=12)
+    ps, bs = ia.block_codec.quantize_tensor(ws, ia.Format.SPARK_Q0)
+    with ia.DeviceWeights.from_blocks(ps, bs, 11008, 4096) as d:
+        x = torch.randn(2048, 4096, device="cuda").to(torch.bfloat16)
+        y = torch.empty((2048, 11008), dtype=torch.float32, device="cuda")
+        for _ in range(3):
+            d.gemm_bf16(x, out=y)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            d.gemm_bf16(x, out=y)
+        e1.record()
+        torch.cuda.synchronize()
+        out["prefill_spark_q0_M2048_N11008_TFLOPs"] = round(2.0 * 2048 * 11008 * 4096 / (e0.elapsed_time(e1) * 1e-3 / 10) / 1e12, 1)
     # what this box reaches with a plain bf16 GEMM of the largest shape (rocBLAS / hipBLASLt through torch), and with a
     # plain device-to-device copy: the practical ceilings next to the vendor peaks
     a = torch.randn(2048, 4096, device="cuda").to(torch.bfloat16)

@@ -187,9 +187,13 @@ int oilhip_set_ordered_sums(int ordered);
 
 
 /* Prefill form of the same contraction: activations as bf16 bit patterns,
- * weights dequantized to bf16 in LDS, MFMA with FP32 accumulation, FP32 out.
+ * weights dequantized to bf16 (each value rounded once), MFMA with FP32 accumulation, FP32 out.
  * (The reference has no bf16 path; its FP32 prefill loop is
- * qwen35_engine.cpp:630-753 over the same gemm.) */
+ * qwen35_engine.cpp:630-753 over the same gemm.)  Uniform OIL4 tensors are decoded tile by tile in LDS inside the
+ * GEMM kernel.  Tensors of any other format, or that mix formats, are decoded to bf16 in slabs of weight rows (at
+ * most 64 MB, a scratch buffer of the stream: the first call of a size on a stream allocates, so make it outside
+ * graph capture) and multiplied by the same kernel reading a dense operand; they need full 256-weight blocks with
+ * the channel sizes the quantizer writes (OILHIP_E_ARG otherwise). */
 int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x_bf16, float* d_y, int M, void* stream);
 
 /* ---------------------------------------------------- flat-codebook kernels

@@ -544,9 +544,11 @@ int oilhip_gemv_f32_general(const oilhip_weights* w, const float* d_x, float* d_
 
 int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x, float* d_y, int M, void* stream) {
     if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
-    if (!plain_oil4(*w))
-        return fail(OILHIP_E_ARG, "bf16 prefill GEMM is implemented for uniform OIL4 tensors");
-    return launch_gemm_oil4_bf16(*w, d_x, d_y, M, (hipStream_t)stream);
+    if (plain_oil4(*w)) return launch_gemm_oil4_bf16(*w, d_x, d_y, M, (hipStream_t)stream);
+    // any other tensor of full blocks: decoded to bf16 slab by slab, then the same kernel over a dense operand
+    const int rc = launch_gemm_any_bf16(*w, d_x, d_y, M, (hipStream_t)stream);
+    if (rc == 1) return fail(OILHIP_E_ARG, "bf16 prefill GEMM needs full blocks with the channel sizes the quantizer writes");
+    return rc;
 }
 
 }  // extern "C"

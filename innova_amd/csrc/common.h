@@ -46,7 +46,7 @@ int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes);
 // one and the old one stays allocated.  No allocation can happen while the stream is being captured, so the first
 // call of a given size on a stream has to be made outside capture; otherwise the call fails with OILHIP_E_ARG.
 // New buffers are zero-filled.
-enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1, kScratchTl = 2 };
+enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1, kScratchTl = 2, kScratchGemmW = 3 };
 int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
 // Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream
@@ -101,6 +101,7 @@ inline bool plain_oil8(const oilhip_weights& w) {
 
 // kernels (each returns an OILHIP_* code and sets the error text)
 int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
+int launch_dequant_bf16_blocks(const oilhip_weights& w, uint32_t b0, uint32_t nb, uint16_t* d_out, hipStream_t s);
 int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
@@ -132,4 +133,5 @@ int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M
 // every format, a lane per run of 32 weights
 int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
+int launch_gemm_any_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
 }  // namespace oilhip

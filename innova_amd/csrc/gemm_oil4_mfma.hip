@@ -194,6 +194,12 @@ __global__ void __launch_bounds__(256) zero_y_kernel(float* __restrict__ y, size
     for (size_t i = (size_t)blockIdx.x * 256u + threadIdx.x; i < n; i += (size_t)gridDim.x * 256u) y[i] = 0.f;
 }
 
+// Y[m][0..n) <- 0 for rows of ldy floats
+__global__ void __launch_bounds__(256) zero_y2d_kernel(float* __restrict__ y, uint32_t n, uint32_t ldy) {
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x;
+    if (c < n) y[(size_t)blockIdx.y * ldy + c] = 0.f;
+}
+
 // Pipelined kernel for larger M: TBM (256 or 128) tokens x 128 weight rows per workgroup, 8 wavefronts (TBM = 256:
 // 4 x 2 wavefronts of 64 x 64 outputs; TBM = 128: 2 x 4 of 64 x 32), 64 columns per step, two LDS tile buffers.
 // Per step a thread stages TBM / 4 bytes of X' and decodes 8 bytes (16 nibbles) of weights; the global loads of two
@@ -214,10 +220,14 @@ constexpr int PBN = 128;
 constexpr int PD = 2;                       // steps of global loads in flight: even, divides K / 64 / 2 (4 measured the same)
 __device__ __forceinline__ uint32_t swz(uint32_t row) { return (row >> 1) & 7u; }
 
-template <int TBM>
+//
+// DENSE: the weight operand is a bf16 matrix [N][K] in natural column order (a tensor of any format, decoded to
+// bf16 beforehand) and Xp is X itself, [M][K]; rows past M and N read as zero through the buffer bounds.  Y has ldy
+// floats per row.
+template <int TBM, bool DENSE>
 __global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
 gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xp, float* __restrict__ Y,
-                           uint32_t M, uint32_t N, uint32_t K, uint32_t ksplit) {
+                           uint32_t M, uint32_t N, uint32_t K, uint32_t ksplit, uint32_t ldy) {
     static_assert(TBM == 256 || TBM == 128, "workgroup tiles of 256 or 128 tokens");
     constexpr int WN = TBM == 256 ? 2 : 4;              // wavefronts along the weight rows
     constexpr int NJ = PBN / WN / 32;                   // 32-row fragments per wavefront along the weight rows
@@ -233,7 +243,7 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     const uint32_t m0 = blockIdx.y * TBM, n0 = blockIdx.x * PBN;
     const uint32_t bpr = K >> 8, KT = K / PK;
 
-    {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 512*k
+    if constexpr (!DENSE) {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 512*k
         const float lv_lane = level_literal(lane & 15u);
         const float lo = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
 #pragma unroll
@@ -243,20 +253,32 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
         }
     }
 
+    const uint32_t nrows = N - n0 < (uint32_t)PBN ? N - n0 : (uint32_t)PBN;
     const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
-        (void*)(W + (size_t)n0 * bpr * 128u), 0,
-        (int)((uint64_t)(N - n0 < (uint32_t)PBN ? N - n0 : (uint32_t)PBN) * bpr * 128u), 0x00020000);
+        (void*)(W + (size_t)n0 * (DENSE ? (size_t)K * 2u : (size_t)bpr * 128u)), 0,
+        (int)((uint64_t)nrows * (DENSE ? (uint64_t)K * 2u : (uint64_t)bpr * 128u)), 0x00020000);
     const uint16_t* xa = Xp + (size_t)m0 * K;
+    const uint32_t mrows = DENSE ? (M - m0 < (uint32_t)TBM ? M - m0 : (uint32_t)TBM) : (uint32_t)TBM;
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc((void*)xa, 0, (int)((uint64_t)mrows * K * 2u), 0x00020000);
     const uint32_t brow = tid >> 2, bq = tid & 3u;                               // weight row of the tile, 8-byte piece of the 32 bytes of a step
     const uint32_t lanebase = (lane & 31u) * 8u;
 
-    u32x4 ar[D][AC];
+    u32x4 ar[D][AC], bd[D][DENSE ? 2 : 1];
     uint32_t br[D][2], sr[D];
     auto load_regs = [&](int set, uint32_t kt) {
 #pragma unroll
         for (int c = 0; c < AC; ++c) {
             const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
-            ar[set][c] = *reinterpret_cast<const u32x4*>(xa + (size_t)row * K + kt * PK + kc * 8u);
+            if constexpr (DENSE) ar[set][c] = __builtin_amdgcn_raw_buffer_load_b128(xrs, (row * K + kt * PK + kc * 8u) * 2u, 0, 0);
+            else ar[set][c] = *reinterpret_cast<const u32x4*>(xa + (size_t)row * K + kt * PK + kc * 8u);
+        }
+        if constexpr (DENSE) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
+                bd[set][c] = __builtin_amdgcn_raw_buffer_load_b128(wrs, (row * K + kt * PK + kc * 8u) * 2u, 0, 0);
+            }
+            return;
         }
         const uint32_t blk_off = (brow * bpr + (kt >> 2)) * 128u;
         const uint32_t off = blk_off + (kt & 3u) * 32u + bq * 8u;
@@ -267,6 +289,7 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     // decode of a later step, split so that its table reads are issued with the fragment reads and its arithmetic
     // runs in the shadow of the MFMAs
     auto lookup_tiles = [&](int set, f32x2 (&t)[8]) {
+        if constexpr (DENSE) return;
 #pragma unroll
         for (int d = 0; d < 2; ++d)
 #pragma unroll
@@ -280,6 +303,14 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
         for (int c = 0; c < AC; ++c) {
             const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
             *reinterpret_cast<u32x4*>(As + (buf * TBM + row) * PLD + ((kc ^ swz(row)) * 8u)) = ar[set][c];
+        }
+        if constexpr (DENSE) {
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const uint32_t id = tid + c * 512u, row = id >> 3, kc = id & 7u;
+                *reinterpret_cast<u32x4*>(Bs + (buf * PBN + row) * PLD + ((kc ^ swz(row)) * 8u)) = bd[set][c];
+            }
+            return;
         }
         const float scale = __half2float(__ushort_as_half((unsigned short)sr[set]));
         uint32_t packed[8];
@@ -385,8 +416,8 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
             for (int v = 0; v < 16; ++v) {
                 const uint32_t row = m0 + (wm * 2 + i) * 32u + 8u * (v >> 2) + 4u * (lane >> 5) + (v & 3u);
                 if (row < M && col < N) {
-                    if (ksplit > 1u) unsafeAtomicAdd(Y + (size_t)row * N + col, acc[i][j][v]);
-                    else Y[(size_t)row * N + col] = acc[i][j][v];
+                    if (ksplit > 1u) unsafeAtomicAdd(Y + (size_t)row * ldy + col, acc[i][j][v]);
+                    else Y[(size_t)row * ldy + col] = acc[i][j][v];
                 }
             }
         }
@@ -406,7 +437,58 @@ int launch(const oilhip_weights& w, const uint16_t* xp, float* d_y, uint32_t M, 
     return OILHIP_OK;
 }
 
+// The pipelined kernel over Nc weight rows (OIL4 blocks, or DENSE: bf16 [Nc][K]); Y + column offset already applied,
+// ldy floats per output row.  A grid that leaves half of the compute units idle is cut in two along K (two partial
+// sums into a zeroed Y: the order of two addends does not matter).
+template <bool DENSE>
+int launch_pipe(const uint8_t* wmat, const uint16_t* x, float* d_y, uint32_t M, uint32_t Nc, uint32_t K, uint32_t ldy, hipStream_t s) {
+    static std::atomic<uint64_t> attr_done[2];
+    const uint32_t ntn = (Nc + PBN - 1) / PBN, cus = (uint32_t)device_cu_count();
+    const bool wide = M > 256u && ntn * ((M + 255u) / 256u) * 2u > cus;
+    const uint32_t tbm = wide ? 256u : 128u, mt = (M + tbm - 1) / tbm;
+    const uint32_t ksplit = ntn * mt * 2u <= cus && (K / PK) % 8u == 0u ? 2u : 1u;
+    if (ksplit > 1u) {
+        if (ldy == Nc) {
+            hipLaunchKernelGGL(zero_y_kernel, dim3((uint32_t)std::min<size_t>(((size_t)M * Nc + 255) / 256, 4096)), dim3(256), 0, s, d_y, (size_t)M * Nc);
+        } else {
+            hipLaunchKernelGGL(zero_y2d_kernel, dim3((Nc + 255u) / 256u, M), dim3(256), 0, s, d_y, Nc, ldy);
+        }
+        OILHIP_HIP(hipGetLastError());
+    }
+    const size_t lds_bytes = (size_t)kTabBytes + 2ull * (tbm + PBN) * PLD * 2;
+    if (wide) {
+        auto kern = gemm_oil4_bf16_pipe_kernel<256, DENSE>;
+        if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
+        hipLaunchKernelGGL(kern, dim3(ntn, mt, ksplit), dim3(512), lds_bytes, s, wmat, x, d_y, M, Nc, K, ksplit, ldy);
+    } else {
+        auto kern = gemm_oil4_bf16_pipe_kernel<128, DENSE>;
+        if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
+        hipLaunchKernelGGL(kern, dim3(ntn, mt, ksplit), dim3(512), lds_bytes, s, wmat, x, d_y, M, Nc, K, ksplit, ldy);
+    }
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
 }  // namespace
+
+// Prefill over a tensor of any format (full 256-weight blocks): slabs of weight rows are decoded to bf16 in a scratch
+// buffer of the stream (dequantize_block_all's values, each rounded once to bf16) and multiplied by the same pipelined
+// kernel reading a dense operand.  Returns 1 when the tensor's layout is not covered.
+int launch_gemm_any_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s) {
+    if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
+    const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols, bpr = K >> 8;
+    if ((uint64_t)M * K * 2u >= 0x80000000ull) return fail(OILHIP_E_ARG, "activation matrix too large for the prefill kernel");
+    // slab: at most 64 MB of bf16, a multiple of 128 rows
+    uint32_t slab = (uint32_t)std::min<uint64_t>(N, std::max<uint64_t>(128, ((64ull << 20) / ((uint64_t)K * 2u)) & ~127ull));
+    uint16_t* wd = nullptr;
+    if (int rc = stream_scratch(s, kScratchGemmW, (size_t)slab * K * 2, reinterpret_cast<void**>(&wd))) return rc;
+    for (uint32_t n0 = 0; n0 < N; n0 += slab) {
+        const uint32_t nc = std::min(slab, N - n0);
+        if (int rc = launch_dequant_bf16_blocks(w, n0 * bpr, nc * bpr, wd, s)) return rc;
+        if (int rc = launch_pipe<true>(reinterpret_cast<const uint8_t*>(wd), d_x, d_y + n0, (uint32_t)M, nc, K, N, s)) return rc;
+    }
+    return OILHIP_OK;
+}
 
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
@@ -424,29 +506,7 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
     if (gx > 64) gx = 64;
     hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
     OILHIP_HIP(hipGetLastError());
-    if (big) {
-        static std::atomic<uint64_t> attr_done[2];
-        // a grid that still leaves half of the units idle is cut in two along K (two partial sums into a zeroed Y)
-        const uint32_t tbm = BM;
-        const uint32_t tiles = ntn * (Mpad / tbm);
-        const uint32_t ksplit = tiles * 2u <= cus && (K / PK) % 8u == 0u ? 2u : 1u;
-        if (ksplit > 1u) {
-            hipLaunchKernelGGL(zero_y_kernel, dim3((uint32_t)std::min<size_t>(((size_t)M * N + 255) / 256, 4096)), dim3(256), 0, s, d_y, (size_t)M * N);
-            OILHIP_HIP(hipGetLastError());
-        }
-        const size_t lds_bytes = (size_t)kTabBytes + 2ull * (tbm + PBN) * PLD * 2;
-        if (wide) {
-            if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel<256>), 160 * 1024)) return rc;
-            hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel<256>, dim3(ntn, Mpad / 256u, ksplit), dim3(512), lds_bytes, s,
-                               w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
-        } else {
-            if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemm_oil4_bf16_pipe_kernel<128>), 160 * 1024)) return rc;
-            hipLaunchKernelGGL(gemm_oil4_bf16_pipe_kernel<128>, dim3(ntn, Mpad / 128u, ksplit), dim3(512), lds_bytes, s,
-                               w.d_payload, xp, d_y, (uint32_t)M, N, K, ksplit);
-        }
-        OILHIP_HIP(hipGetLastError());
-        return OILHIP_OK;
-    }
+    if (big) return launch_pipe<false>(w.d_payload, xp, d_y, (uint32_t)M, N, K, N, s);
     return launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
 }
 

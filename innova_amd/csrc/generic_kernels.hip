@@ -128,10 +128,11 @@ __device__ __forceinline__ float4 decode_full4(const uint8_t* __restrict__ p, ui
 #define OILHIP_ALL_FORMATS(X) X(0) X(1) X(2) X(3) X(4) X(5) X(6) X(7) X(8) X(9) X(10) X(11) X(12) X(13) X(14)
 
 // FMT >= 0: every block has that format; FMT < 0: each block's format from its descriptor (tensors that mix formats)
-template <int FMT>
+// BF16: the blocks [b0, b0 + nblocks) as bf16 (each FP32 value rounded once, to nearest even), for the prefill GEMM
+template <int FMT, bool BF16 = false>
 __global__ void __launch_bounds__(256)
 dequant_full_kernel(const uint8_t* __restrict__ base, uint32_t stride, const DevBlock* __restrict__ blocks,
-                    const DecodeTables* __restrict__ T, float* __restrict__ out, uint32_t nblocks) {
+                    const DecodeTables* __restrict__ T, void* __restrict__ out_, uint32_t nblocks, uint32_t b0 = 0) {
     __shared__ float tb[256 * 3 + 20];
     {
         const uint32_t t = threadIdx.x;
@@ -142,7 +143,8 @@ dequant_full_kernel(const uint8_t* __restrict__ base, uint32_t stride, const Dev
     __syncthreads();
     const FullTables L{tb, tb + 256, tb + 512, tb + 768, tb + 784};
     const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
-    for (uint32_t b = blockIdx.x * 4u + wave; b < nblocks; b += gridDim.x * 4u) {
+    for (uint32_t bi = blockIdx.x * 4u + wave; bi < nblocks; bi += gridDim.x * 4u) {
+        const uint32_t b = b0 + bi;
         const uint8_t* p = base + (blocks ? (size_t)blocks[b].off16 * 16u : (size_t)b * stride);
         float4 o = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         if constexpr (FMT >= 0) {
@@ -153,7 +155,14 @@ dequant_full_kernel(const uint8_t* __restrict__ base, uint32_t stride, const Dev
             switch (f) { OILHIP_ALL_FORMATS(OILHIP_CASE) default: break; }
 #undef OILHIP_CASE
         }
-        reinterpret_cast<float4*>(out + (size_t)b * 256u)[lane] = o;
+        if constexpr (BF16) {
+            typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+            const bf2 lo = bf2{(__bf16)o.x, (__bf16)o.y}, hi = bf2{(__bf16)o.z, (__bf16)o.w};
+            reinterpret_cast<uint2*>(static_cast<uint16_t*>(out_) + (size_t)bi * 256u)[lane] =
+                make_uint2(__builtin_bit_cast(uint32_t, lo), __builtin_bit_cast(uint32_t, hi));
+        } else {
+            reinterpret_cast<float4*>(static_cast<float*>(out_) + (size_t)bi * 256u)[lane] = o;
+        }
     }
 }
 
@@ -227,30 +236,61 @@ int launch_block_mse(const oilhip_weights& w, const float* d_orig, const uint64_
     return OILHIP_OK;
 }
 
+// full blocks of nominal size: one format at a regular stride (1), or (window streams, one format or several) the place
+// and format of every block from its descriptor (2); 0: neither
+static int full_block_layout(const oilhip_weights& w) {
+    if (!w.all_full || w.d_out_off) return 0;
+    const bool by_stride = w.uniform_fmt >= 0 && w.uniform_stride > 0 && (w.uniform_base & 3u) == 0 &&
+                           w.uniform_stride == full_block_bytes(w.uniform_fmt) &&
+                           w.uniform_cb == full_block_cb_bytes(w.uniform_fmt) &&
+                           w.uniform_cb + w.uniform_idx == w.uniform_stride;
+    if (by_stride) return 1;
+    bool by_desc = w.seg.nstreams > 0;
+    for (uint32_t i = 0; by_desc && i < w.seg.nf; ++i)
+        by_desc = w.seg.cb_bytes[i] == full_block_cb_bytes((int)w.seg.fmt[i]) &&
+                  w.seg.cb_bytes[i] + w.seg.idx_bytes[i] == full_block_bytes((int)w.seg.fmt[i]);
+    return by_desc ? 2 : 0;
+}
+
+// The blocks [b0, b0 + nb) decoded to bf16 at d_out (nb * 256 values).  Returns 1 when the tensor's blocks are not
+// full blocks of nominal size.
+int launch_dequant_bf16_blocks(const oilhip_weights& w, uint32_t b0, uint32_t nb, uint16_t* d_out, hipStream_t s) {
+    const DecodeTables* T = nullptr;
+    if (int rc = get_tables(&T)) return rc;
+    const int layout = full_block_layout(w);
+    if (!layout) return 1;
+    if (nb == 0) return OILHIP_OK;
+    const uint32_t g = std::min<uint32_t>((nb + 3u) / 4u, (uint32_t)device_cu_count() * 16u);
+    const bool by_stride = layout == 1;
+    const uint8_t* base = w.d_payload + (by_stride ? w.uniform_base : 0u);
+    const DevBlock* bl = by_stride ? nullptr : w.d_blocks;
+    const int f = by_stride || w.seg.nf == 1 ? w.uniform_fmt : -1;
+#define OILHIP_CASE(F) case F: hipLaunchKernelGGL((dequant_full_kernel<F, true>), dim3(g), dim3(256), 0, s, base, w.uniform_stride, bl, T, (void*)d_out, nb, b0); break;
+    switch (f) {
+        OILHIP_ALL_FORMATS(OILHIP_CASE)
+        default: hipLaunchKernelGGL((dequant_full_kernel<-1, true>), dim3(g), dim3(256), 0, s, base, 0u, bl, T, (void*)d_out, nb, b0); break;
+    }
+#undef OILHIP_CASE
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
 int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s) {
     const DecodeTables* T = nullptr;
     if (int rc = get_tables(&T)) return rc;
     if (w.nblocks == 0) return OILHIP_OK;
-    // full blocks of nominal size: one format at a regular stride, or (window streams, one format or several) the place
-    // and format of every block from its descriptor
-    if (w.all_full && !w.d_out_off) {
+    {
         const uint32_t g = std::min<uint32_t>((w.nblocks + 3u) / 4u, (uint32_t)device_cu_count() * 16u);
-        const bool by_stride = w.uniform_fmt >= 0 && w.uniform_stride > 0 && (w.uniform_base & 3u) == 0 &&
-                               w.uniform_stride == full_block_bytes(w.uniform_fmt) &&
-                               w.uniform_cb == full_block_cb_bytes(w.uniform_fmt) &&
-                               w.uniform_cb + w.uniform_idx == w.uniform_stride;
-        bool by_desc = !by_stride && w.seg.nstreams > 0;
-        for (uint32_t i = 0; by_desc && i < w.seg.nf; ++i)
-            by_desc = w.seg.cb_bytes[i] == full_block_cb_bytes((int)w.seg.fmt[i]) &&
-                      w.seg.cb_bytes[i] + w.seg.idx_bytes[i] == full_block_bytes((int)w.seg.fmt[i]);
-        if (by_stride || by_desc) {
+        const int layout = full_block_layout(w);
+        const bool by_stride = layout == 1;
+        if (layout) {
             const uint8_t* base = w.d_payload + (by_stride ? w.uniform_base : 0u);
             const DevBlock* bl = by_stride ? nullptr : w.d_blocks;
             const int f = by_stride || w.seg.nf == 1 ? w.uniform_fmt : -1;
-#define OILHIP_CASE(F) case F: hipLaunchKernelGGL(dequant_full_kernel<F>, dim3(g), dim3(256), 0, s, base, w.uniform_stride, bl, T, d_out, w.nblocks); break;
+#define OILHIP_CASE(F) case F: hipLaunchKernelGGL((dequant_full_kernel<F, false>), dim3(g), dim3(256), 0, s, base, w.uniform_stride, bl, T, (void*)d_out, w.nblocks, 0u); break;
             switch (f) {
                 OILHIP_ALL_FORMATS(OILHIP_CASE)
-                default: hipLaunchKernelGGL(dequant_full_kernel<-1>, dim3(g), dim3(256), 0, s, base, 0u, bl, T, d_out, w.nblocks); break;
+                default: hipLaunchKernelGGL((dequant_full_kernel<-1, false>), dim3(g), dim3(256), 0, s, base, 0u, bl, T, (void*)d_out, w.nblocks, 0u); break;
             }
 #undef OILHIP_CASE
             OILHIP_HIP(hipGetLastError());

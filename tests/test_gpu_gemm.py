@@ -66,9 +66,44 @@ def test_config_shapes(rows, cols, M):
     assert np.all(np.isfinite(y))
 
 
-def test_rejects_non_oil4():
-    w = gaussian_weights(256 * 4, 1)
-    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL8)
-    with ia.DeviceWeights.from_blocks(payload, blocks, 4, 256) as dw:
-        with pytest.raises(ia.OilHipError):
-            dw.gemm_bf16(torch.zeros(2, 256, dtype=torch.bfloat16, device="cuda"))
+def _check_any_format(fmts, rows, cols, M, seed):
+    """bf16 prefill over a tensor that is not uniform OIL4: sampled token rows against the float64 product of the
+    dequantized weights (the oracle's dequantize, bit-equal to the device's) with the bf16 activations."""
+    w = gaussian_weights(rows * cols, seed, outlier_every=97)
+    payload, blocks = ia.block_codec.quantize_tensor(w, fmts)
+    rng = np.random.default_rng(seed)
+    X = torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).cuda().to(torch.bfloat16)
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        y = dw.gemm_bf16(X).cpu().numpy()
+    wd = O.dequant_blocks(payload, to_orc_blocks(blocks)).reshape(rows, cols).astype(np.float64)
+    sel = np.unique(np.concatenate([[0, M - 1], rng.integers(0, M, 14)]))
+    want = X.float().cpu().numpy()[sel].astype(np.float64) @ wd.T
+    assert rel_l2(y[sel], want) <= TOL, rel_l2(y[sel], want)
+    assert np.all(np.isfinite(y))
+
+
+@pytest.mark.parametrize("fmt", [ia.Format.OIL8, ia.Format.SPARK_Q0, ia.Format.OIL1, ia.Format.OIL2, ia.Format.OIL16,
+                                 ia.Format.OIL4_GRP, ia.Format.SPARK_SPARSE])
+def test_other_formats(fmt):
+    _check_any_format(fmt, 640, 1024, 300, 40 + int(fmt))
+
+
+@pytest.mark.parametrize("rows,cols,M", [(4096, 4096, 512), (1000, 2048, 70), (4096, 11008, 257)])
+def test_mixed_formats(rows, cols, M):
+    """Formats drawn per block (all fifteen), and the planner's 1.50-bpw routing of a whole matrix."""
+    rng = np.random.default_rng(rows)
+    _check_any_format(rng.integers(0, 15, rows * cols // 256).astype(np.uint8), rows, cols, M, rows + M)
+
+
+def test_planner_routed_matrix_prefill():
+    from innova_amd.format_planner import FormatPlanner
+    rows, cols, M = 4096, 4096, 640
+    w = gaussian_weights(rows * cols, 5, outlier_every=100)
+    pl = FormatPlanner(1.50)
+    pl.score_importance(w)
+    _check_any_format(np.asarray(pl.allocate(rows * cols // 256).formats, dtype=np.uint8), rows, cols, M, 5)
+
+
+def test_slabs_of_a_tall_tensor():
+    """More rows than one 64 MB slab of bf16 holds (8192 at 4096 columns): two slabs, the second partial."""
+    _check_any_format(ia.Format.SPARK_Q0, 8192 + 384, 4096, 260, 77)
