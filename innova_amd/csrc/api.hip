@@ -6,6 +6,7 @@
 #include <algorithm>
 #include <map>
 #include <tuple>
+#include <queue>
 #include <vector>
 
 #include "common.h"
@@ -180,68 +181,97 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
             return;
         }
     }
-    const uint32_t ns = (uint32_t)std::min<uint64_t>(rows, (uint64_t)device_cu_count() * 8);   // streams: two per SIMD
-    struct Entry { uint32_t slot, flags, nblk, data_off, tag_off, row0, nrows; };
-    struct Window { std::vector<Entry> ent; std::vector<uint16_t> tags; std::vector<uint32_t> src; uint32_t data = 0; };
-    auto bytes_of = [](size_t ne, size_t nb, uint32_t data) { return 16 + 16 * ne + ((2 * nb + 15) & ~(size_t)15) + data; };
-    std::vector<std::vector<Window>> streams(ns);
-    // The first window of every stream is fetched blind at the size of the fullest one, so its capacity is held near
-    // the average stream: what does not fit goes to a second window, fetched while the first is worked on.
-    uint64_t all_bytes = 0, widest = 0;
-    for (const DevBlock& d : db) {
-        all_bytes += g.stride[slot_of[d.fmt]] + 2u;
-        widest = std::max<uint64_t>(widest, g.stride[slot_of[d.fmt]]);
+    // streams: at most two per SIMD, and as many as give every stream the same number of rows (or one less): streams of
+    // five and six rows side by side would leave the fixed-size first windows a sixth empty
+    const uint64_t max_streams = (uint64_t)device_cu_count() * 8, rows_each = (rows + max_streams - 1) / max_streams;
+    const uint32_t ns = (uint32_t)((rows + rows_each - 1) / rows_each);
+    // a block's tag is its row of the tile and its column block: one byte while a row has at most 64 blocks
+    const uint32_t tagw = bpr <= 64 ? 1u : 2u, tag_shift = bpr <= 64 ? 6u : 12u;
+    // `rec` counts the 8-byte units of the window's records: one per entry, and two (four row numbers) behind every
+    // entry that closes a tile
+    struct Entry { uint32_t slot, flags, nblk, data_off, tag_off, rows[kSegTileRows], nrows; };
+    struct Window { std::vector<Entry> ent; std::vector<uint16_t> tags; std::vector<uint32_t> src; uint32_t data = 0, rec = 0; };
+    auto bytes_of = [&](size_t nrec, size_t nb, uint32_t data) { return ((8 + 8 * nrec + tagw * nb + 15) & ~(size_t)15) + data; };
+    // Rows go to streams by weight, heaviest first, each to the stream that is lightest so far: streams end up with
+    // nearly the same number of bytes, so the first windows (fetched blind, all at the size of the fullest) carry
+    // little slack and the wavefronts finish together.  A stream's rows need not be neighbours.
+    std::vector<uint32_t> row_bytes(rows, 0);
+    uint64_t widest = 0;
+    for (uint64_t r = 0; r < rows; ++r)
+        for (uint64_t c = 0; c < bpr; ++c) {
+            const uint32_t st = g.stride[slot_of[db[r * bpr + c].fmt]];
+            row_bytes[r] += st + tagw;
+            widest = std::max<uint64_t>(widest, st);
+        }
+    std::vector<uint32_t> order(rows);
+    for (uint32_t r = 0; r < rows; ++r) order[r] = r;
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t x, uint32_t y) { return row_bytes[x] > row_bytes[y]; });
+    std::vector<std::vector<uint32_t>> rows_of(ns);
+    {
+        using Load = std::pair<uint64_t, uint32_t>;                 // (bytes so far, stream)
+        std::priority_queue<Load, std::vector<Load>, std::greater<Load>> light;
+        for (uint32_t st = 0; st < ns; ++st) light.push({0, st});
+        for (uint32_t r : order) {
+            Load l = light.top();
+            light.pop();
+            rows_of[l.second].push_back(r);
+            l.first += row_bytes[r];
+            light.push(l);
+        }
     }
-    const uint64_t first_cap = std::min<uint64_t>(kSegWindow, std::max((all_bytes / ns * 9 / 8 + 96 + 63) & ~63ull, (widest + 64 + 63) & ~63ull));
+    std::vector<std::vector<Window>> streams(ns);
     for (uint32_t st = 0; st < ns; ++st) {
         std::vector<Window>& ws = streams[st];
         ws.emplace_back();
-        // the stream's rows in tiles of at most kSegTileRows, as even as they come
-        const uint64_t ra = (uint64_t)st * rows / ns, rb = (uint64_t)(st + 1) * rows / ns;
-        const uint64_t nt = (rb - ra + kSegTileRows - 1) / kSegTileRows;
-        for (uint64_t t = 0; t < nt; ++t) {
-            const uint64_t r0 = ra + t * (rb - ra) / nt, r1 = ra + (t + 1) * (rb - ra) / nt;
+        std::vector<uint32_t>& mine = rows_of[st];
+        std::sort(mine.begin(), mine.end());
+        for (size_t t0 = 0; t0 < mine.size(); t0 += kSegTileRows) {
+            const uint32_t nr = (uint32_t)std::min<size_t>(kSegTileRows, mine.size() - t0);
             Entry* last = nullptr;
             for (uint32_t s = 0; s < nf; ++s) {
                 bool open = false;                     // an entry of this tile and slot is open in the current window
-                for (uint64_t r = r0; r < r1; ++r)
+                for (uint32_t j = 0; j < nr; ++j)
                     for (uint64_t c = 0; c < bpr; ++c) {
-                        const uint32_t b = (uint32_t)(r * bpr + c);
+                        const uint32_t b = (uint32_t)((uint64_t)mine[t0 + j] * bpr + c);
                         if (slot_of[db[b].fmt] != (int)s) continue;
                         Window* w = &ws.back();
-                        if (bytes_of(w->ent.size() + (open ? 0 : 1), w->tags.size() + 1, w->data + g.stride[s]) >
-                            (ws.size() == 1 ? first_cap : kSegWindow)) {
+                        // room for the block, its tag, its entry if a new one opens, and the row record of a closing entry
+                        if (bytes_of(w->rec + (open ? 0 : 1) + 2, w->tags.size() + 1, w->data + g.stride[s]) > kSegWindow) {
                             ws.emplace_back();
                             w = &ws.back();
                             open = false;
                         }
                         if (!open) {
-                            w->ent.push_back(Entry{s, 0u, 0u, w->data, (uint32_t)w->tags.size(), (uint32_t)r0, (uint32_t)(r1 - r0)});
+                            Entry e{s, 0u, 0u, w->data, (uint32_t)w->tags.size(), {0, 0, 0, 0}, nr};
+                            for (uint32_t q = 0; q < nr; ++q) e.rows[q] = mine[t0 + q];
+                            w->ent.push_back(e);
+                            ++w->rec;
                             open = true;
                         }
                         last = &w->ent.back();
                         ++last->nblk;
-                        w->tags.push_back((uint16_t)(((r - r0) << 12) | c));
+                        w->tags.push_back((uint16_t)((j << tag_shift) | c));
                         w->src.push_back(b);
                         w->data += g.stride[s];
                     }
             }
             last->flags |= 1u;                         // every tile has blocks: its last entry closes it
+            ws.back().rec += 2;                        // ... and is followed by the tile's row numbers
         }
     }
     // first windows at a fixed stride (the fullest of them decides it), so that a wavefront finds its own from its
     // number alone; the windows after them packed one behind the other, each found through its predecessor's header
-    auto used = [&](const Window& w) { return bytes_of(w.ent.size(), w.tags.size(), w.data); };
+    auto used = [&](const Window& w) { return bytes_of(w.rec, w.tags.size(), w.data); };
     size_t first_used = 0;
     for (const auto& ws : streams) first_used = std::max(first_used, used(ws[0]));
-    const uint64_t stride = (first_used + 63) & ~(size_t)63;
+    const uint64_t stride = (first_used + 15) & ~(size_t)15;
     uint64_t total = stride * ns;
     std::vector<std::vector<uint64_t>> at_of(ns);
     for (uint32_t st = 0; st < ns; ++st) {
         at_of[st].push_back(st * stride);
         for (size_t wi = 1; wi < streams[st].size(); ++wi) {
             at_of[st].push_back(total);
-            total += (used(streams[st][wi]) + 63) & ~(size_t)63;
+            total += (used(streams[st][wi]) + 15) & ~(size_t)15;
         }
     }
     if ((total >> 4) > 0xFFFFFFFFull) return;
@@ -250,20 +280,25 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
         for (size_t wi = 0; wi < streams[st].size(); ++wi) {
             const Window& w = streams[st][wi];
             uint8_t* base = out.data() + at_of[st][wi];
-            const uint32_t tag_base = 16u + 16u * (uint32_t)w.ent.size();
-            const uint32_t data_base = tag_base + (uint32_t)((2 * w.tags.size() + 15) & ~(size_t)15);
+            const uint32_t tag_base = 8u + 8u * w.rec;
+            const uint32_t data_base = (tag_base + tagw * (uint32_t)w.tags.size() + 15u) & ~15u;
             const bool more = wi + 1 < streams[st].size();
-            const uint32_t hdr[4] = {(uint32_t)w.ent.size(), more ? 1u : 0u,
-                                     more ? (uint32_t)((used(streams[st][wi + 1]) + 15) >> 4) : 0u,
+            const uint32_t hdr[2] = {w.rec | (more ? 1u << 12 : 0u) | (more ? (uint32_t)((used(streams[st][wi + 1]) + 15) >> 4) << 16 : 0u),
                                      more ? (uint32_t)(at_of[st][wi + 1] >> 4) : 0u};
-            std::memcpy(base, hdr, 16);
-            for (size_t i = 0; i < w.ent.size(); ++i) {
-                const Entry& e = w.ent[i];
-                const uint32_t rec[4] = {e.slot | (g.fmt[e.slot] << 4) | (e.flags << 8) | (e.nblk << 16),
-                                         (data_base + e.data_off) | ((tag_base + 2u * e.tag_off) << 16), e.row0, e.nrows};
-                std::memcpy(base + 16 + 16 * i, rec, 16);
+            std::memcpy(base, hdr, 8);
+            uint32_t at_rec = 8;
+            for (const Entry& e : w.ent) {
+                const uint32_t rec[2] = {e.slot | (g.fmt[e.slot] << 4) | (e.flags << 8) | (e.nrows << 9) | (e.nblk << 16),
+                                         (data_base + e.data_off) | ((tag_base + tagw * e.tag_off) << 16)};
+                std::memcpy(base + at_rec, rec, 8);
+                at_rec += 8;
+                if (e.flags & 1u) {
+                    std::memcpy(base + at_rec, e.rows, 16);
+                    at_rec += 16;
+                }
             }
-            std::memcpy(base + tag_base, w.tags.data(), 2 * w.tags.size());
+            if (tagw == 1) for (size_t i = 0; i < w.tags.size(); ++i) base[tag_base + i] = (uint8_t)w.tags[i];
+            else std::memcpy(base + tag_base, w.tags.data(), 2 * w.tags.size());
             uint32_t at = data_base;
             for (uint32_t b : w.src) {
                 DevBlock& d = db[b];
@@ -272,6 +307,7 @@ static void pack_window_streams(std::vector<uint8_t>& pay, std::vector<DevBlock>
                 at += g.stride[slot_of[d.fmt]];
             }
         }
+    g.tag_bytes = tagw;
     pay.swap(out);
     g.nf = nf;
     g.nstreams = ns;

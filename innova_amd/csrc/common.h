@@ -51,18 +51,20 @@ int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
 // Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream
 // (gemv_seg.hip).  The first window of stream s sits at byte s * stream_bytes of the payload buffer, the later ones
-// behind all first windows, each found through its predecessor.  A stream covers a contiguous range of rows in tiles
-// of at most kSegTileRows; inside a tile the blocks are ordered by format (in the order of `fmt`), inside a format by
-// row and column.  Window: 4 dwords {entries, 1 if another window follows, 16-byte pieces that window fills, its byte
-// offset / 16 in the buffer}; per entry 4 dwords {slot | format << 4 | closes its tile << 8 | blocks << 16, byte offset
-// of the blocks | byte offset of their tags << 16, first row of the tile, rows of the tile}; the tags (per block: row
-// of the tile << 12 | column block); the blocks, 16-byte aligned, whole.  `blind16` = 16-byte pieces the fullest first
+// behind all first windows, each found through its predecessor.  A stream covers a set of rows (chosen so that all
+// streams weigh about the same) in tiles of at most kSegTileRows; inside a tile the blocks are ordered by format (in the
+// order of `fmt`), inside a format by row and column.  Window: 2 dwords {8-byte units of records | 1 << 12 if another
+// window follows | 16-byte pieces that window fills << 16, its byte offset / 16 in the buffer}; the records: per entry
+// 2 dwords {slot | format << 4 | closes its tile << 8 | rows of the tile << 9 | blocks << 16, byte offset of the blocks |
+// byte offset of their tags << 16}, and behind an entry that closes its tile 4 dwords with the tile's row numbers; the
+// tags (per block: row of the tile and column block, in one byte (row << 6 | column) while a row has at most 64 blocks,
+// else two (row << 12 | column)); the blocks, 16-byte aligned, whole.  `blind16` = 16-byte pieces the fullest first
 // window fills.
 constexpr int kSegMaxFormats = 15;
 constexpr uint32_t kSegWindow = 4096;
 constexpr int kSegTileRows = 4;
 struct SegLayout {
-    uint32_t nf = 0, nstreams = 0, blind16 = 0;
+    uint32_t nf = 0, nstreams = 0, blind16 = 0, tag_bytes = 2;
     uint64_t stream_bytes = 0;
     uint32_t fmt[kSegMaxFormats] = {}, cb_bytes[kSegMaxFormats] = {}, idx_bytes[kSegMaxFormats] = {}, stride[kSegMaxFormats] = {};
 };

@@ -7,7 +7,7 @@
 // dependent memory round trips, not by bandwidth.  The upload therefore stores it as one stream of windows (at most
 // 4 KB each) per wavefront, the first at an address that follows from the wavefront's number alone: it is fetched
 // blind together with the activations, and a window describes itself and says where the next one is (entries: format, block count, where the blocks and their tags
-// sit in the window, which rows they belong to).  A stream covers a contiguous range of rows in tiles of up to four;
+// sit in the window, which rows they belong to).  A stream covers rows chosen so that all streams weigh about the same, in tiles of up to four;
 // inside a tile the blocks are ordered by format, inside a format by row and column, so a step of 8 blocks has one
 // format for all 64 lanes.  The wavefront copies a window to LDS with plain 16-byte loads, fetches the next one while it works,
 // and decodes from LDS: a lane owns one run of 32 weights and adds its dot product to its accumulator of the run's
@@ -31,7 +31,7 @@ typedef _Float16 h2v __attribute__((ext_vector_type(2)));
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 struct SegArgs {
-    uint32_t nstreams, blind16;
+    uint32_t nstreams, blind16, tag_bytes;
     uint64_t stream_bytes;
     uint32_t cb_bytes[kSegMaxFormats], idx_bytes[kSegMaxFormats], stride[kSegMaxFormats];
 };
@@ -51,26 +51,31 @@ __device__ __forceinline__ void add_to_row(float (&acc)[MB][TR], uint32_t rowl, 
 }
 
 template <int FMT, int MB>
-__device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* tags, uint32_t nblk, uint32_t stride,
+__device__ __forceinline__ void run_entry(const uint8_t* data, const uint8_t* tags, uint32_t tagw, uint32_t nblk, uint32_t stride,
                                           uint32_t cb_bytes, uint32_t idx_bytes, const DecodeTables* __restrict__ T,
                                           const LdsTables& L, const float* xs, const float* rs, float (&acc)[MB][TR],
                                           uint32_t xpad, uint32_t nruns, uint32_t lane) {
     constexpr int N = run_raw_dwords(FMT);
     const uint32_t steps = (nblk + 7u) >> 3, r = lane & 7u, g = lane >> 3;
+    // a block's tag: row of the tile and column block, one byte (row << 6 | column) or two (row << 12 | column)
+    const uint32_t tshift = tagw == 1u ? 6u : 12u, tmask = tagw == 1u ? 0x3Fu : 0xFFFu;
+    auto tag_of = [&](uint32_t b) -> uint32_t {
+        return tagw == 1u ? (uint32_t)tags[b] : (uint32_t)reinterpret_cast<const uint16_t*>(tags)[b];
+    };
     if constexpr (FMT == 0) {
         // a block is 8 FP16 run means: a lane takes a whole block, 16 bytes of means against 8 run sums
         for (uint32_t b0 = 0; b0 < nblk; b0 += 64u) {
             const uint32_t blk = b0 + lane;
             const bool live = blk < nblk;
             const uint32_t bc = live ? blk : nblk - 1u;
-            const uint32_t tag = tags[bc];
+            const uint32_t tag = tag_of(bc);
             const u32x4 mv = *reinterpret_cast<const u32x4*>(data + bc * stride);
             const float mean[8] = {f16_bits(mv.x), f16_bits(mv.x >> 16), f16_bits(mv.y), f16_bits(mv.y >> 16),
                                    f16_bits(mv.z), f16_bits(mv.z >> 16), f16_bits(mv.w), f16_bits(mv.w >> 16)};
             float part[MB];
 #pragma unroll
             for (int m = 0; m < MB; ++m) {
-                const float4* sp = reinterpret_cast<const float4*>(rs + (size_t)m * nruns + (tag & 0xFFFu) * 8u);
+                const float4* sp = reinterpret_cast<const float4*>(rs + (size_t)m * nruns + (tag & tmask) * 8u);
                 const float4 s0 = sp[0], s1 = sp[1];
                 float a0 = mean[0] * s0.x, a1 = mean[1] * s0.y;
                 a0 = __fmaf_rn(mean[2], s0.z, a0);
@@ -81,18 +86,18 @@ __device__ __forceinline__ void run_entry(const uint8_t* data, const uint16_t* t
                 a1 = __fmaf_rn(mean[7], s1.w, a1);
                 part[m] = live ? a0 + a1 : 0.f;
             }
-            add_to_row<MB>(acc, tag >> 12, part);
+            add_to_row<MB>(acc, tag >> tshift, part);
         }
     } else {
     for (uint32_t st = 0; st < steps; ++st) {
         const uint32_t blk = st * 8u + g;
         const bool live = blk < nblk;
         const uint32_t bc = live ? blk : nblk - 1u;                     // past the end: the last block again, result unused
-        const uint32_t tag = tags[bc];
+        const uint32_t tag = tag_of(bc);
         const uint8_t* cb = data + bc * stride;
         uint32_t raw[N];
         fetch_run<FMT>(cb, cb_bytes, r, raw);
-        const uint32_t rowl = tag >> 12, run = (tag & 0xFFFu) * 8u + r;
+        const uint32_t rowl = tag >> tshift, run = (tag & tmask) * 8u + r;
         float part[MB];
         if constexpr (FMT == 1) {
             // weight k = bit k ? +scale : -scale; as FP16: |scale| with the sign bit from the (inverted) sign word.
@@ -277,31 +282,34 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
     for (uint32_t wi = 0;; ++wi) {
         const uint8_t* cur = win + (wi & 1u) * kSegWindow;
         const uint32_t* hdr = reinterpret_cast<const uint32_t*>(cur);
-        const bool more = uniform(hdr[1]) != 0u;
+        const uint32_t h0 = uniform(hdr[0]);           // 8-byte units of records | another window follows << 12 | its 16-byte pieces << 16
+        const bool more = (h0 >> 12) & 1u;
         if (more) {                                    // the next window: its size and place are in this one's header
-            const uint32_t used16 = uniform(hdr[2]);
-            const uint8_t* np = streams + (size_t)uniform(hdr[3]) * 16u;
+            const uint32_t used16 = h0 >> 16;
+            const uint8_t* np = streams + (size_t)uniform(hdr[1]) * 16u;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t piece = j * 64u + lane < used16 ? j * 64u + lane : used16 - 1u;
                 wreg[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(np + (size_t)piece * 16u));
             }
         }
-        const uint32_t ne = uniform(hdr[0]);
+        const uint32_t ne = h0 & 0xFFFu;               // an entry is one unit, the row numbers behind a closing entry two
         for (uint32_t i = 0; i < ne; ++i) {
-            const uint32_t* rec = reinterpret_cast<const uint32_t*>(cur) + 4u + 4u * i;
-            const uint32_t r0 = uniform(rec[0]), r1 = uniform(rec[1]), row0 = uniform(rec[2]), nrows = uniform(rec[3]);
-            const uint32_t sl = r0 & 15u, nblk = r0 >> 16;
+            const uint32_t* rec = reinterpret_cast<const uint32_t*>(cur) + 2u + 2u * i;
+            const uint32_t r0 = uniform(rec[0]), r1 = uniform(rec[1]);
+            const uint32_t sl = r0 & 15u, nblk = r0 >> 16, nrows = (r0 >> 9) & 7u;
             const uint8_t* data = cur + (r1 & 0xFFFFu);
-            const uint16_t* tags = reinterpret_cast<const uint16_t*>(cur + (r1 >> 16));
+            const uint8_t* tags = cur + (r1 >> 16);
 #define OILHIP_SEG_CASE(F)                                                                                              \
     case F:                                                                                                             \
-        run_entry<F, MB>(data, tags, nblk, A.stride[sl], A.cb_bytes[sl], A.idx_bytes[sl], T, L, xs, rs, acc, xpad,  \
+        run_entry<F, MB>(data, tags, A.tag_bytes, nblk, A.stride[sl], A.cb_bytes[sl], A.idx_bytes[sl], T, L, xs, rs, acc, xpad,  \
                          nruns, lane);                                                                                  \
         break;
             switch ((r0 >> 4) & 15u) { OILHIP_SEG_FORMATS(OILHIP_SEG_CASE) default: break; }
 #undef OILHIP_SEG_CASE
             if ((r0 >> 8) & 1u) {                      // the tile is complete: sum each row across the wavefront
+                i += 2;                                // the two units behind a closing entry: the tile's row numbers
+                const uint32_t trow[TR] = {uniform(rec[2]), uniform(rec[3]), uniform(rec[4]), uniform(rec[5])};
 #pragma unroll
                 for (int m = 0; m < MB; ++m)
 #pragma unroll
@@ -314,7 +322,7 @@ gemv_seg_kernel(const uint8_t* __restrict__ streams, const DecodeTables* __restr
                         v += oil4::dpp_row_mirror(v);
                         v += oil4::dpp_row_bcast15(v);
                         v += oil4::dpp_row_bcast31(v);
-                        if (lane == 63 && (uint32_t)j < nrows && m0 + m < M) y[(size_t)(m0 + m) * rows + row0 + j] = v * yscale;
+                        if (lane == 63 && (uint32_t)j < nrows && m0 + m < M) y[(size_t)(m0 + m) * rows + trow[j]] = v * yscale;
                     }
             }
         }
@@ -344,7 +352,7 @@ int launch_seg(const oilhip_weights& w, const DecodeTables* T, const float* d_x,
     if (lds > 160 * 1024) return 1;
     if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
     SegArgs A{};
-    A.nstreams = g.nstreams; A.blind16 = g.blind16; A.stream_bytes = g.stream_bytes;
+    A.nstreams = g.nstreams; A.blind16 = g.blind16; A.tag_bytes = g.tag_bytes; A.stream_bytes = g.stream_bytes;
     for (uint32_t i = 0; i < g.nf; ++i) { A.cb_bytes[i] = g.cb_bytes[i]; A.idx_bytes[i] = g.idx_bytes[i]; A.stride[i] = g.stride[i]; }
     hipLaunchKernelGGL(kern, dim3((g.nstreams + kWaves - 1) / kWaves), dim3(64 * kWaves), lds, s, w.d_payload, T, d_x, d_xw,
                        d_y, (uint32_t)w.rows, (uint32_t)w.cols, m0, M, A);
