@@ -27,7 +27,7 @@ ROWS, COLS = 11008, 4096       # W is [N rows][K cols]: y = W x
 RING = 40                      # distinct weight copies: 40 x 22.5 MB = 902 MB > 256 MB cache
 # HBM bytes per GEMV launch, cited from the rocprofv3 counter runs summarised in profiles/oil4_gemv_4096x11008_m1.md
 # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0 KiB per dispatch, factors from a plain 1 GiB copy); not measured in this run
-HBM_TRAFFIC_BYTES_PER_LAUNCH = 22881894
+HBM_TRAFFIC_BYTES_PER_LAUNCH = 22881280
 
 
 def log(*a):
