@@ -172,7 +172,7 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
 
 /* The same product for uniform OIL4 tensors, for callers that cannot allocate device memory (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no
- * hipMalloc/hipFree: the scratch its multi-row kernel needs (packed activations, 4 MB) is a fixed array in the
+ * hipMalloc/hipFree: the scratch its multi-row kernel needs (packed activations and their exponents, 8 MB) is a fixed array in the
  * library's code object, one per GPU.  Limits: uniform OIL4 in the plain block layout, cols <= 32768; anything else
  * returns OILHIP_E_ARG.  All calls on one GPU share that array: calls that overlap on one GPU (two streams, two
  * threads) race on it and must be serialized by the caller. */

@@ -436,7 +436,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 constexpr uint32_t kMaxPackCols = kGemvPackMaxCols;
 constexpr size_t kPackBytes = kGemvPackBytes;
 
-// The same scratch for the entry point that allocates nothing: a fixed array in the code object (4 MB, held by every
+// The same scratch for the entry point that allocates nothing: a fixed array in the code object (8 MB, held by every
 // GPU the library runs on until the process ends).  In host code the array's name is only a stand-in: the device
 // address comes from hipGetSymbolAddress, once per device with that device current, and only that pointer is ever
 // handed to a kernel.
