@@ -125,7 +125,9 @@ size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t c
 int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
-                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s);
+                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean = false);
+// clears the slab counters at the start of a batch workspace; launches over it may then be told that they are clean
+int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s);
 // widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
 constexpr uint32_t kGemvPackMaxCols = 32768;
 constexpr size_t kGemvPackExpBytes = (size_t)(kGemvPackMaxCols >> 8) * 2u * 16u * 4u;    // one scale exponent per (token tile, block, column)

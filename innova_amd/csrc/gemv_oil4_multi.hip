@@ -46,6 +46,7 @@ __device__ __forceinline__ uint32_t split_level(float L) {
     return (uint32_t)__half_as_ushort(h) | ((uint32_t)__half_as_ushort(l) << 16);
 }
 
+constexpr size_t kBatchCounterBytes = 16u * 4096u;   // a page of slab counters for each of up to 16 jobs of a grouped launch
 constexpr int kGroups = 4;                // 16 x 16 partial-sum tiles per wavefront and row tile (groups of 16 rows x token tiles)
 constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
 // partial sums of a 16 x 16 tile, accumulator lane 16 q + j, element v at float q*68 + 4 j + v of 272: for one token j the
@@ -79,6 +80,7 @@ __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* __restrict__ 
 // xp + xp_off[j] (exponents at xp_exp + exp_off[j]); its rows are list[row0[j] + m] when use_list is set, else
 // row0[j] + m.  The list travels by value with the launch, so the host needs no copy and no synchronisation.
 constexpr int kMaxJobs = 16, kMaxListed = 448;
+static_assert(kBatchCounterBytes == (size_t)kMaxJobs * 4096u, "one page of counters per job");
 struct PackJobs {
     uint32_t n, wgs_per_job;
     int M[kMaxJobs], row0[kMaxJobs];
@@ -547,14 +549,23 @@ size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t c
     const uint32_t bpr = (uint32_t)(cols >> 8), NT = kind == 2 ? 2u : 1u, tokens = kind == 0 ? 8u : kind == 1 ? 16u : 32u;
     const uint32_t pb = kind == 2 ? 8u : 16u, ks = (bpr + pb - 1u) / pb;
     size_t per_batch = (size_t)NT * bpr * 16384u + (size_t)NT * bpr * 64u;
-    size_t per_job = 4096u + (ks > 2u ? (size_t)ks * tokens * rows * 4u : 0u);
-    return (size_t)nb * per_batch + (size_t)2 * nb * per_job + 256u;
+    size_t per_job = ks > 2u ? (size_t)ks * tokens * rows * 4u : 0u;
+    return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)2 * nb * per_job + 256u;
+}
+
+// The slab counters of the ordered K-split sums sit at the start of a batch workspace, one 4 KB page per job.  Every
+// launch leaves them at zero, so a caller that runs several launches over one workspace clears them once.
+int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s) {
+    hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)(kBatchCounterBytes / 1024u)), dim3(256), 0, s, static_cast<uint32_t*>(d_ws),
+                       (uint32_t)(kBatchCounterBytes / 4u));
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
 }
 
 int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
-                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s) {
+                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean) {
     if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || kind < 0 || kind > 2 || nlist > kMaxListed) return 1;
     const oilhip_weights& w0 = *wa[0];
     if (w0.rows == 0 || w0.rows > 0x7FFFFFFFull || w0.cols > kMaxPackCols || (w0.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
@@ -569,14 +580,14 @@ int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const
     uint32_t ks = (bpr + pb - 1u) / pb;
     if (ks < 2u || ks > (uint32_t)device_cu_count()) ks = 1u;
     const size_t xp_dwords = (size_t)NT * bpr * 4096u, exp_ints = (size_t)NT * bpr * 16u;
-    uint8_t* base = static_cast<uint8_t*>(d_ws);
+    uint32_t* counter = static_cast<uint32_t*>(d_ws);
+    uint8_t* base = static_cast<uint8_t*>(d_ws) + kBatchCounterBytes;
     uint32_t* xp = reinterpret_cast<uint32_t*>(base);
     int* xp_exp = reinterpret_cast<int*>(base + (size_t)nb * xp_dwords * 4u);
     const int njobs = wb ? 2 * nb : nb;
     uint8_t* jobs_base = base + (size_t)nb * (xp_dwords * 4u + exp_ints * 4u);
     const size_t part_floats = ks > 2u ? (size_t)ks * tokens * w0.rows : 0u;
-    uint32_t* counter = reinterpret_cast<uint32_t*>(jobs_base);
-    float* partial = reinterpret_cast<float*>(jobs_base + (size_t)njobs * 4096u);
+    float* partial = reinterpret_cast<float*>(jobs_base);
     if (xp_dwords * (size_t)nb > 0xFFFFFFFFull || part_floats * (size_t)njobs > 0xFFFFFFFFull) return 1;
 
     PackJobs pj{};
@@ -606,7 +617,7 @@ int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const
             mj.partial_off[j] = (uint32_t)(j * part_floats); mj.counter_off[j] = (uint32_t)(j * 1024);
         }
     }
-    if (ks > 2u && ordered)                                               // the caller's workspace is not known to be zero
+    if (ks > 2u && ordered && !counters_clean)                            // the caller's workspace is not known to be zero
         hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
     hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
                        (uint32_t)w0.cols, 0, 0, ldx, xrows, kind == 0 ? 1 : 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);

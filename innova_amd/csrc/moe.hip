@@ -17,6 +17,16 @@ __global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ p, s
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) p[i] = 0.0f;
 }
 
+// three ranges in one launch (what a grouped step needs cleared before its first kernel)
+__global__ void __launch_bounds__(256) fill_zero3_kernel(float* __restrict__ a, size_t na, float* __restrict__ b, size_t nb,
+                                                         float* __restrict__ c, size_t nc) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < na + nb + nc; i += (size_t)gridDim.x * 256) {
+        if (i < na) a[i] = 0.0f;
+        else if (i < na + nb) b[i - na] = 0.0f;
+        else c[i - na - nb] = 0.0f;
+    }
+}
+
 // h = silu(g) * u, silu(v) = v / (1 + exp(-v))  (src/math.cpp:117-126)
 __global__ void __launch_bounds__(256) swiglu_kernel(float* __restrict__ g, const float* __restrict__ u, size_t n) {
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (size_t)gridDim.x * 256) {
@@ -85,6 +95,7 @@ struct CombineLists {
     float wgt[kMaxPairs];       // its weight (<= 0: dropped)
 };
 
+// zacc == nullptr: the caller does not want the z-loss, and the workgroups skip their atomic on its one address
 __global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __restrict__ o, uint32_t D, float* __restrict__ out,
                                                               double* __restrict__ zacc, const CombineLists L) {
     __shared__ double part[4];
@@ -102,6 +113,7 @@ __global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __res
         }
         out[(size_t)t * D + d] = sum;
     }
+    if (!zacc) return;                                     // uniform over the grid
     for (int off = 32; off > 0; off >>= 1) z += __shfl_xor(z, off, 64);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = z;
     __syncthreads();
@@ -248,9 +260,10 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
     for (int e = 0; e < E && grouped; ++e) grouped = plain_oil4(*gate[e]) && plain_oil4(*up[e]) && plain_oil4(*down[e]);
     if (grouped) {
         const int64_t pairs = (int64_t)tok.size();
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(1), dim3(256), 0, s, (float*)ws.z, (size_t)2);
-        // outputs of row parts that meet through atomics start at zero
-        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, s, ws.g, (size_t)(pairs * (2 * F + D)));
+        // outputs of row parts that meet through atomics start at zero; so do the z-loss accumulator and the slab
+        // counters at the start of the batch workspace (every launch leaves them at zero again)
+        hipLaunchKernelGGL(fill_zero3_kernel, dim3(1024), dim3(256), 0, s, ws.g, (size_t)(pairs * (2 * F + D)), (float*)ws.z, (size_t)2,
+                           (float*)ws.batch, (size_t)(16 * 4096 / 4));
         OILHIP_HIP(hipGetLastError());
         struct Batch { int e, pair0, m; };
         std::vector<Batch> byKind[3];
@@ -275,10 +288,10 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                     Mb[b] = B.m; r0[b] = B.pair0;
                 }
                 int rc = launch_gemv_oil4_multi_batches(kind, nb, wg, yg, wu, yu, Mb, r0, tok.data(), (int)tok.size(), d_x, nullptr,
-                                                        (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s);
+                                                        (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s, true);
                 if (rc == 0)
                     rc = launch_gemv_oil4_multi_batches(kind, nb, wd, yo, nullptr, nullptr, Mb, r0, nullptr, 0, ws.g, ws.u,
-                                                        (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s);
+                                                        (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s, true);
                 if (rc < 0) return rc;
                 if (rc == 1) return fail(OILHIP_E_ARG, "moe_forward: the grouped launch refused a shape it was planned for");
             }
@@ -294,7 +307,7 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                 filled[(size_t)t]++;
             }
         hipLaunchKernelGGL(combine_grouped_kernel, dim3((uint32_t)((D + 255) / 256), (uint32_t)T), dim3(256), 0, s, ws.o, (uint32_t)D,
-                           d_out, ws.z, L);
+                           d_out, z_loss ? ws.z : (double*)nullptr, L);
         OILHIP_HIP(hipGetLastError());
         if (z_loss) {
             double z = 0.0;
