@@ -65,3 +65,37 @@ def test_host_quantizer_rejects_bad_arguments():
         ia.block_codec.quantize_block_all(99, np.zeros(4, np.float32))
     with pytest.raises(ia.OilHipError):
         ia.block_codec.quantize_tensor(np.zeros(512, np.float32), np.zeros(3, np.uint8))
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_device():
+    """Argument checks come first in every entry point: these calls fail with OILHIP_E_ARG on a machine without a GPU
+    (nothing is launched) and the thread-local message says why."""
+    import ctypes as C
+
+    from innova_amd import _lib
+    L = _lib.lib()
+    one = C.c_float(0.0)
+    p = C.addressof(one)
+
+    def refused(rc, needle):
+        assert rc != 0
+        assert needle in L.oilhip_last_error().decode()
+
+    refused(L.oilhip_tl_gemm(3, p, p, p, 1, 1, 3, None), "kind")
+    refused(L.oilhip_tl_gemm(2, p, p, p, 1, 1, 16, None), "multiple of 3")
+    refused(L.oilhip_tl_gemm(1, None, p, p, 1, 1, 4, None), "null")
+    refused(L.oilhip_dense_map_f32(9, p, p, 0.0, p, 4, None), "operation")
+    refused(L.oilhip_dense_map_f32(3, p, None, 0.0, p, 4, None), "null")
+    refused(L.oilhip_dense_norm_f32(2, p, p, p, 1e-5, p, 1, 4, None), "kind")
+    refused(L.oilhip_dense_gemm_f32(1.0, p, p, 0.0, p, -1, 1, 1, None), "negative")
+    refused(L.oilhip_dense_gemv_f32(1.0, None, p, 0.0, p, 2, 2, None), "null")
+    refused(L.oilhip_dense_softmax_f32(None, p, 1, 4, 1, None), "null")
+    refused(L.oilhip_read_probe(p, 4096, 3, 0, 0, 256, 512, p, None), "in flight")
+    refused(L.oilhip_read_probe(p, 4096, 4, 0, 0, 256, 100, p, None), "threads")
+    refused(L.oilhip_profile_gemv(4, p, p, 1.0, p, p, 4, 16, 10, None, None), "null result")
+    perf = (C.c_uint64 * 4)()
+    refused(L.oilhip_profile_gemv(5, p, p, 1.0, p, p, 4, 16, 10, C.addressof(perf), None), "kind")
+    # empty problems are not errors and launch nothing
+    assert L.oilhip_tl_gemm(1, p, p, p, 0, 4, 8, None) == 0
+    assert L.oilhip_dense_map_f32(0, p, None, 0.0, p, 0, None) == 0
+    assert L.oilhip_dense_gemm_f32(1.0, p, p, 0.0, p, 0, 5, 5, None) == 0
