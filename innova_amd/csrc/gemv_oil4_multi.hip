@@ -283,13 +283,17 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
 #pragma unroll
         for (int a = 0; a < kGroups; ++a) acc[a] = v4f{0.f, 0.f, 0.f, 0.f};
         for (uint32_t pass = 0; pass < npass; ++pass) {
-            if (tile > 0 || pass > 0) issue_group(0, tg0, pass);
             if (npass > 1 || tile == 0) load_b(pass);
             if (!table_synced) { __syncthreads(); table_synced = true; }   // the level table is complete
+            // the (tile, pass) that follows this one: groups past the slab's last one load nothing
+            const bool last_pass = pass + 1u == npass;
+            const uint32_t next_tg0 = last_pass ? tg0 + KG : tg0, next_pass = last_pass ? 0u : pass + 1u;
             // ---- main loop: groups of the tile, two blocks each -------------------------------------------
 #pragma unroll
             for (int g = 0; g < KG; ++g) {
+                static_assert(KG % 2 == 0, "the first group of a tile lands in buffer 0");
                 if (g + 1 < KG) issue_group((g + 1) & 1, tg0 + g + 1, pass);
+                else issue_group(0, next_tg0, next_pass);                  // flies during the tile's sums
                 const bool g_on = tg0 + g < g1;                            // wave-uniform
 #pragma unroll
                 for (int b2 = 0; b2 < BPW; ++b2) {

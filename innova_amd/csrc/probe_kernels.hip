@@ -9,7 +9,10 @@ namespace {
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
 // U loads in flight per wavefront.  PAT 0: each wavefront streams its own contiguous share (as the GEMVs' row groups
-// do); PAT 1: wavefronts interleaved KB by KB.  NT: loads marked non-temporal (streaming, no reuse expected).
+// do); PAT 1: wavefronts interleaved KB by KB; PAT 2: the multi-token GEMV's pattern over rows of 2 KB: a workgroup of
+// 8 wavefronts walks groups of 16 rows, wavefront w reads blocks 2w and 2w+1 of each row with four loads whose lane
+// 16*kq + i fetches 16 bytes of row i (64 contiguous bytes per row and load).  NT: loads marked non-temporal
+// (streaming, no reuse expected).
 template <int U, bool NT, int PAT>
 __global__ void __launch_bounds__(1024)
 read_probe_kernel(const uint8_t* __restrict__ base, uint64_t bytes, uint32_t* __restrict__ sink) {
@@ -20,6 +23,24 @@ read_probe_kernel(const uint8_t* __restrict__ base, uint64_t bytes, uint32_t* __
     if (PAT == 0) { k0 = kbs * gw / nw; k1 = kbs * (gw + 1) / nw; step = 1; }
     else { k0 = gw; k1 = kbs; step = nw; }
     uint32_t acc = 0;
+    if (PAT == 2) {
+        constexpr int UG = U >= 4 ? U / 4 : 1;                     // groups of 16 rows in flight
+        const uint64_t ng = bytes >> 15, g0 = ng * blockIdx.x / gridDim.x, g1 = ng * (blockIdx.x + 1) / gridDim.x;
+        for (uint64_t g = g0; g < g1; g += UG) {
+            u32x4 v[UG * 4];
+#pragma unroll
+            for (int u = 0; u < UG * 4; ++u) {
+                const uint64_t gg = g + u / 4 < g1 ? g + u / 4 : g0;
+                const u32x4* p = reinterpret_cast<const u32x4*>(base + gg * 32768ull + (lane & 15u) * 2048u +
+                                                                (2u * (wave & 7u) + ((u >> 1) & 1)) * 128u + (u & 1) * 64u + (lane >> 4) * 16u);
+                v[u] = NT ? __builtin_nontemporal_load(p) : *p;
+            }
+#pragma unroll
+            for (int u = 0; u < UG * 4; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+        }
+        if (acc == 0x9e3779b9u) sink[gw] = acc;
+        return;
+    }
     for (uint64_t k = k0; k < k1; k += step * U) {
         u32x4 v[U];
 #pragma unroll
@@ -37,6 +58,7 @@ read_probe_kernel(const uint8_t* __restrict__ base, uint64_t bytes, uint32_t* __
 template <int U, bool NT>
 void launch_pat(int pattern, dim3 g, dim3 b, hipStream_t s, const uint8_t* p, uint64_t bytes, uint32_t* sink) {
     if (pattern == 0) hipLaunchKernelGGL((read_probe_kernel<U, NT, 0>), g, b, 0, s, p, bytes, sink);
+    else if (pattern == 2) hipLaunchKernelGGL((read_probe_kernel<U, NT, 2>), g, b, 0, s, p, bytes, sink);
     else hipLaunchKernelGGL((read_probe_kernel<U, NT, 1>), g, b, 0, s, p, bytes, sink);
 }
 template <int U>
@@ -58,7 +80,9 @@ extern "C" int oilhip_read_probe(const void* d_buf, uint64_t bytes, int in_fligh
         return fail(OILHIP_E_ARG, "read_probe: loads in flight must be 1, 2, 4 or 8");
     if (threads < 64 || threads > 1024 || threads % 64 != 0 || workgroups < 1 || workgroups > 65536)
         return fail(OILHIP_E_ARG, "read_probe: threads must be a multiple of 64 up to 1024, workgroups 1..65536");
-    if (pattern != 0 && pattern != 1) return fail(OILHIP_E_ARG, "read_probe: pattern must be 0 (contiguous shares) or 1 (interleaved)");
+    if (pattern < 0 || pattern > 2) return fail(OILHIP_E_ARG, "read_probe: pattern must be 0 (contiguous shares), 1 (interleaved) or 2 (16 rows of 2 KB per load)");
+    if (pattern == 2 && (threads != 512 || in_flight < 4 || bytes < 32768 * (uint64_t)workgroups))
+        return fail(OILHIP_E_ARG, "read_probe: pattern 2 needs 512 threads, 4 or 8 loads in flight and at least 32 KB per workgroup");
     auto s = static_cast<hipStream_t>(stream);
     const dim3 g((unsigned)workgroups), b((unsigned)threads);
     const uint8_t* p = static_cast<const uint8_t*>(d_buf);
