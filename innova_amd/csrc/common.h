@@ -127,6 +127,7 @@ int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
                                    uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean = false);
 // clears the slab counters at the start of a batch workspace; launches over it may then be told that they are clean
+constexpr size_t kGemvBatchCounterBytes = 32u * 4096u;   // slab counters at the start of a batch workspace: a 4 KB page per job
 int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s);
 // widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
 constexpr uint32_t kGemvPackMaxCols = 32768;

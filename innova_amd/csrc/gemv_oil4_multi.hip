@@ -46,7 +46,7 @@ __device__ __forceinline__ uint32_t split_level(float L) {
     return (uint32_t)__half_as_ushort(h) | ((uint32_t)__half_as_ushort(l) << 16);
 }
 
-constexpr size_t kBatchCounterBytes = 16u * 4096u;   // a page of slab counters for each of up to 16 jobs of a grouped launch
+constexpr size_t kBatchCounterBytes = kGemvBatchCounterBytes;   // a page of slab counters for each of up to 32 jobs of a grouped launch
 constexpr int kGroups = 4;                // 16 x 16 partial-sum tiles per wavefront and row tile (groups of 16 rows x token tiles)
 constexpr int kRedBase = kTabBytes;       // partial sums follow the level table
 // partial sums of a 16 x 16 tile, accumulator lane 16 q + j, element v at float q*68 + 4 j + v of 272: for one token j the
@@ -79,7 +79,7 @@ __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* __restrict__ 
 // Several batches in one launch (the experts of a mixture-of-experts step): batch j packs M[j] rows of x into
 // xp + xp_off[j] (exponents at xp_exp + exp_off[j]); its rows are list[row0[j] + m] when use_list is set, else
 // row0[j] + m.  The list travels by value with the launch, so the host needs no copy and no synchronisation.
-constexpr int kMaxJobs = 16, kMaxListed = 448;
+constexpr int kMaxJobs = 32, kMaxListed = 448;
 static_assert(kBatchCounterBytes == (size_t)kMaxJobs * 4096u, "one page of counters per job");
 struct PackJobs {
     uint32_t n, wgs_per_job;

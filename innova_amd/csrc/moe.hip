@@ -127,12 +127,12 @@ struct Workspace {
     size_t bytes, batch_bytes;
 };
 
-constexpr int kChunk = 8;       // expert batches per grouped launch (gate and up together are 16 tensors)
+constexpr int kChunk = 16;      // expert batches per grouped launch (gate and up together are 32 tensors)
 
 // scratch of one grouped launch: the larger of the gate/up side (rows F, cols D) and the down side (rows D, cols F)
 size_t batch_scratch_bytes(int64_t D, int64_t F) {
     size_t m = 0;
-    for (int kind = 0; kind < 3; ++kind) {
+    for (int kind = 0; kind < 2; ++kind) {         // passes of 8 and of 16 tokens
         m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)F, (uint64_t)D));
         m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)D, (uint64_t)F));
     }
@@ -253,7 +253,7 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
             if (tok[(size_t)i] == tok[(size_t)i - 1]) distinct[(size_t)e] = 0;
     if (dropped) *dropped = drop;
     // ---- grouped path: uniform OIL4 experts, lists small enough to travel with the launches ---------------------
-    // Per pass size (32, 16 or 8 tokens) and chunk of experts: one launch that splits the gathered activations, one
+    // Per pass size (16 or 8 tokens) and chunk of experts: one launch that splits the gathered activations, one
     // launch over the gate and up projections of all those experts, one that forms silu(gate) * up while splitting it,
     // one over their down projections; then one combine.  No copy, no synchronisation: the step can be captured.
     bool grouped = ws.batch_bytes > 0 && (int64_t)tok.size() <= kMaxPairs && T * K <= kMaxPairs && !tok.empty();
@@ -263,19 +263,19 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         // outputs of row parts that meet through atomics start at zero; so do the z-loss accumulator and the slab
         // counters at the start of the batch workspace (every launch leaves them at zero again)
         hipLaunchKernelGGL(fill_zero3_kernel, dim3(1024), dim3(256), 0, s, ws.g, (size_t)(pairs * (2 * F + D)), (float*)ws.z, (size_t)2,
-                           (float*)ws.batch, (size_t)(16 * 4096 / 4));
+                           (float*)ws.batch, kGemvBatchCounterBytes / 4);
         OILHIP_HIP(hipGetLastError());
         struct Batch { int e, pair0, m; };
-        std::vector<Batch> byKind[3];
+        std::vector<Batch> byKind[2];
         for (int e = 0; e < E; ++e) {
             int n = begin[(size_t)e + 1] - begin[(size_t)e], pos = begin[(size_t)e];
             while (n > 0) {
-                const int take = n > 32 ? 32 : n;
-                byKind[take <= 8 ? 0 : take <= 16 ? 1 : 2].push_back(Batch{e, pos, take});
+                const int take = n > 16 ? 16 : n;                 // passes of 16: two of them beat one pass of 32 (twice the products per table read)
+                byKind[take <= 8 ? 0 : 1].push_back(Batch{e, pos, take});
                 pos += take; n -= take;
             }
         }
-        for (int kind = 2; kind >= 0; --kind)
+        for (int kind = 1; kind >= 0; --kind)
             for (size_t c0 = 0; c0 < byKind[kind].size(); c0 += kChunk) {
                 const int nb = (int)std::min<size_t>(kChunk, byKind[kind].size() - c0);
                 const oilhip_weights *wg[kChunk], *wu[kChunk], *wd[kChunk];
