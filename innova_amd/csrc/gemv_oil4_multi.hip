@@ -18,7 +18,7 @@
 // activations are split and laid out in this operand order once per launch by pack_x_kernel (every workgroup needs
 // all of them), so the main kernel fetches its 128 operand dwords with plain 16-byte loads.  Partial sums of the
 // wavefronts are added through LDS once per tile of 64 rows.
-// Batches of more than 16 tokens run passes of 32: a wavefront then owns one block per K-pass and multiplies each
+// Single tensors with more than 16 tokens run passes of 32: a wavefront then owns one block per K-pass and multiplies each
 // decoded weight operand with the activations of two token tiles (the table look-ups, which bound the main loop, are
 // shared), a row tile is 32 rows.
 #include <hip/hip_fp16.h>
