@@ -54,6 +54,8 @@ def test_dispatch_matches_reference_fixture():
 
 @pytest.mark.parametrize("T,E,K,D,F,fmts", [(24, 4, 2, 512, 768, (3, 3, 3)),        # OIL4 experts: fast kernel, 1..many tokens each
                                              (40, 2, 2, 256, 512, (3, 3, 3)),        # > 16 tokens per expert: several passes
+                                             (12, 8, 2, 256, 512, (3, 3, 3)),        # a few tokens per expert: passes of 8 only
+                                             (50, 6, 2, 256, 512, (3, 3, 3)),        # passes of 16 and six remainders, which get launches of their own
                                              (9, 3, 1, 256, 512, (4, 10, 1))])       # OIL8 / OIL4_GRP / SPARK_Q0: general kernel
 def test_dispatch_against_oracle(T, E, K, D, F, fmts):
     packs, dense = MF.moe_experts(5 + T, E, D, F, fmts)
