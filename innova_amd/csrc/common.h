@@ -129,6 +129,7 @@ int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const
 // clears the slab counters at the start of a batch workspace; launches over it may then be told that they are clean
 constexpr size_t kGemvBatchCounterBytes = 32u * 4096u;   // slab counters at the start of a batch workspace: a 4 KB page per job
 int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s);
+bool gemv_oil4_multi_batches_accumulate(int kind, uint64_t cols);
 // widest row that kernel takes and the bytes of packed activations one pass of it needs (d_pack, or stream scratch)
 constexpr uint32_t kGemvPackMaxCols = 32768;
 constexpr size_t kGemvPackExpBytes = (size_t)(kGemvPackMaxCols >> 8) * 2u * 16u * 4u;    // one scale exponent per (token tile, block, column)

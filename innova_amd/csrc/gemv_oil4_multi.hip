@@ -557,6 +557,15 @@ size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t c
     return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)2 * nb * per_job + 256u;
 }
 
+// Whether a grouped launch over tensors with rows of `cols` weights adds partial sums into its outputs with atomics
+// (two K parts, or more with the ordered sums switched off): the outputs must then start at zero.
+bool gemv_oil4_multi_batches_accumulate(int kind, uint64_t cols) {
+    const uint32_t bpr = (uint32_t)(cols >> 8), pb = kind == 2 ? 8u : 16u;
+    uint32_t ks = (bpr + pb - 1u) / pb;
+    if (ks < 2u || ks > (uint32_t)device_cu_count()) ks = 1u;
+    return ks == 2u || (ks > 2u && g_ordered_sums.load(std::memory_order_relaxed) == 0);
+}
+
 // The slab counters of the ordered K-split sums sit at the start of a batch workspace, one 4 KB page per job.  Every
 // launch leaves them at zero, so a caller that runs several launches over one workspace clears them once.
 int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s) {

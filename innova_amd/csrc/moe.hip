@@ -263,8 +263,11 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         const int64_t pairs = (int64_t)tok.size();
         // outputs of row parts that meet through atomics start at zero; so do the z-loss accumulator and the slab
         // counters at the start of the batch workspace (every launch leaves them at zero again)
-        hipLaunchKernelGGL(fill_zero3_kernel, dim3(1024), dim3(256), 0, s, ws.g, (size_t)(pairs * (2 * F + D)), (float*)ws.z, (size_t)2,
-                           (float*)ws.batch, kGemvBatchCounterBytes / 4);
+        bool adds = false;                                       // the expert buffers only where a launch adds into them
+        for (int kind = 0; kind < 2; ++kind)
+            adds = adds || gemv_oil4_multi_batches_accumulate(kind, (uint64_t)D) || gemv_oil4_multi_batches_accumulate(kind, (uint64_t)F);
+        hipLaunchKernelGGL(fill_zero3_kernel, dim3(adds ? 1024 : 64), dim3(256), 0, s, ws.g, adds ? (size_t)(pairs * (2 * F + D)) : (size_t)0,
+                           (float*)ws.z, (size_t)2, (float*)ws.batch, kGemvBatchCounterBytes / 4);
         OILHIP_HIP(hipGetLastError());
         struct Batch { int e, pair0, m; };
         std::vector<Batch> byKind[2];
