@@ -11,7 +11,7 @@
 // kq+4 (64 nibbles), one dword (8 nibbles) per matrix instruction.  Lane 16*kq + j supplies token j at the same
 // nibble positions, and accumulator register v of that lane collects row 4*kq + v x token j.
 //
-// A wavefront owns two blocks of the row per K-pass (8 wavefronts = 16 blocks = 4096 columns) and keeps the split
+// A wavefront owns two blocks of the row per K-pass (blocks w and w + 8 of the pass; 8 wavefronts = 16 blocks = 4096 columns) and keeps the split
 // activations of those blocks in registers (2 x 64 FP16 pairs per lane), so the main loop is: two 16-byte loads per
 // lane and unit (16 rows x 1 block), 32 byte-pair table lookups (each returns the two high and the two low halves
 // of a byte's levels, already packed as matrix operands), 24 matrix instructions, 4 scale multiplies.  The
@@ -207,7 +207,12 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     constexpr int BPW = NT == 2 ? 1 : 2;                                   // blocks of the row per wavefront and pass
     constexpr uint32_t PB = 8u * BPW;                                      // blocks per pass
     constexpr int KG = kGroups / NT;                                       // groups of 16 rows per tile
-    const uint32_t blk_lo = bpr * part / ksplit, blk_hi = bpr * (part + 1u) / ksplit;
+    // Parts of near-equal length, unless full passes leave a last part of at most half a pass: block b2 of a wavefront
+    // is block 8 b2 + wave of the pass, so such a part keeps every wavefront busy with one block and takes half the
+    // time (56 blocks: 16 + 16 + 16 + 8 is three and a half units of work, four parts of 14 are four).
+    const bool full_parts = ksplit > 1u && bpr - (ksplit - 1u) * PB <= PB / 2u;
+    const uint32_t blk_lo = full_parts ? part * PB : bpr * part / ksplit;
+    const uint32_t blk_hi = full_parts ? (blk_lo + PB < bpr ? blk_lo + PB : bpr) : bpr * (part + 1u) / ksplit;
     const uint32_t npass = (blk_hi - blk_lo + PB - 1u) / PB;
 
     // groups of 16 rows [g0, g1) of this workgroup
@@ -230,7 +235,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         const uint32_t r = g * 16u + li;
 #pragma unroll
         for (int b2 = 0; b2 < BPW; ++b2) {
-            const uint32_t blk = blk_lo + pass * PB + wave * BPW + b2;
+            const uint32_t blk = blk_lo + pass * PB + (uint32_t)b2 * 8u + wave;
             const bool ok = g < g1 && r < rows && blk < blk_hi;
             const uint32_t off = (r - g0 * 16u) * row_bytes + blk * 128u + kq * 16u;
             wv[buf][b2][0] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, ok ? off : kOobOffset, 0, 2);
@@ -243,7 +248,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     auto load_b = [&](uint32_t pass) {
 #pragma unroll
         for (int b2 = 0; b2 < 2; ++b2) {   // NT = 2: b2 is the token tile, whose activations follow those of tile 0
-            const uint32_t blk = blk_lo + pass * PB + wave * BPW + (NT == 2 ? 0 : b2);
+            const uint32_t blk = blk_lo + pass * PB + (NT == 2 ? 0u : (uint32_t)b2 * 8u) + wave;
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const uint32_t off = blk < blk_hi ? (blk * 2u + h) * 8192u + lane * 16u + (NT == 2 ? b2 * bpr * 16384u : 0u) : kOobOffset;
@@ -297,7 +302,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                 const bool g_on = tg0 + g < g1;                            // wave-uniform
 #pragma unroll
                 for (int b2 = 0; b2 < BPW; ++b2) {
-                    const bool on = g_on && blk_lo + pass * PB + wave * BPW + b2 < blk_hi;     // wave-uniform
+                    const bool on = g_on && blk_lo + pass * PB + (uint32_t)b2 * 8u + wave < blk_hi;     // wave-uniform
                     if (!on) continue;
                     const u32x4 w0 = wv[g & 1][b2][0], w1 = wv[g & 1][b2][1];
                     v4f t0[NT], t1[NT];                                    // this block: Lh xh, and Lh xl + Ll xh, per token tile
@@ -345,7 +350,7 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
                     float unscale[NT];
 #pragma unroll
                     for (int t = 0; t < NT; ++t)
-                        unscale[t] = undo[((uint32_t)t * (blk_hi - blk_lo) + pass * PB + wave * BPW + b2) * 16u + li];
+                        unscale[t] = undo[((uint32_t)t * (blk_hi - blk_lo) + pass * PB + (uint32_t)b2 * 8u + wave) * 16u + li];
                     // the block's FP16 scale of row r sits in the low half of the first dword of lane r (kq = 0)
 #pragma unroll
                     for (int v = 0; v < 4; ++v) {
