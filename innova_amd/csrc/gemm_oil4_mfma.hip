@@ -51,18 +51,38 @@ __device__ __forceinline__ float level_literal(uint32_t i) {      // kOIL4Levels
     return __uint_as_float(bits | (i < 8u ? 0x80000000u : 0u));
 }
 
-// X (bf16 bit patterns, [M][K]) -> X' ([Mpad][K], rows >= M zero), columns in nibble order.
+// X (bf16 bit patterns, [M][K]) -> X' ([Mpad][K], rows >= M zero), columns in nibble order: a thread forms eight
+// consecutive columns of X' (one 16-byte store).  The same launch clears Y (zn floats per row, ldy apart) for the
+// launches whose two K halves add into it.
 __global__ void __launch_bounds__(256)
-permute_x_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ xp, uint32_t M, uint32_t K, uint32_t Mpad) {
+permute_x_kernel(const uint16_t* __restrict__ x, uint16_t* __restrict__ xp, uint32_t M, uint32_t K, uint32_t Mpad,
+                 float* __restrict__ y, uint32_t zn, uint32_t ldy) {
     const uint32_t row = blockIdx.y;
-    for (uint32_t c = blockIdx.x * 256 + threadIdx.x; c < K; c += gridDim.x * 256) {
-        const uint32_t p = c & 255u;
-        uint16_t v = 0;
-        if (p >= 4 && row < M) {
-            const uint32_t q = p - 4;
-            v = x[(size_t)row * K + (c - p) + q + (q >= 63) + (q >= 126) + (q >= 189)];
+    for (uint32_t c8 = blockIdx.x * 256 + threadIdx.x; c8 * 8u < K; c8 += gridDim.x * 256) {
+        const uint32_t c = c8 * 8u, p0 = c & 255u;
+        uint16_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t p = p0 + k;
+            v[k] = 0;
+            if (p >= 4 && row < M) {
+                const uint32_t q = p - 4;
+                v[k] = x[(size_t)row * K + (c - p0) + q + (q >= 63) + (q >= 126) + (q >= 189)];
+            }
         }
-        xp[(size_t)row * K + c] = v;
+        uint4 o;
+        o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+        o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+        *reinterpret_cast<uint4*>(xp + (size_t)row * K + c) = o;
+    }
+    if (y && row < M) {
+        float* yr = y + (size_t)row * ldy;
+        if (((ldy | zn) & 3u) == 0u && (reinterpret_cast<uintptr_t>(y) & 15u) == 0u) {
+            for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i * 4u < zn; i += gridDim.x * 256)
+                reinterpret_cast<float4*>(yr)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+        } else {
+            for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < zn; i += gridDim.x * 256) yr[i] = 0.0f;
+        }
     }
 }
 
@@ -437,17 +457,30 @@ int launch(const oilhip_weights& w, const uint16_t* xp, float* d_y, uint32_t M, 
     return OILHIP_OK;
 }
 
+// Tiling of the pipelined kernel for M tokens and Nc weight rows
+struct PipePlan { bool wide; uint32_t ntn, tbm, mt, ksplit; };
+PipePlan pipe_plan(uint32_t M, uint32_t Nc, uint32_t K) {
+    PipePlan p;
+    const uint32_t cus = (uint32_t)device_cu_count();
+    p.ntn = (Nc + PBN - 1) / PBN;
+    p.wide = M > 256u && p.ntn * ((M + 255u) / 256u) * 2u > cus;
+    p.tbm = p.wide ? 256u : 128u;
+    p.mt = (M + p.tbm - 1) / p.tbm;
+    p.ksplit = p.ntn * p.mt * 2u <= cus && (K / PK) % 8u == 0u ? 2u : 1u;
+    return p;
+}
+
 // The pipelined kernel over Nc weight rows (OIL4 blocks, or DENSE: bf16 [Nc][K]); Y + column offset already applied,
 // ldy floats per output row.  A grid that leaves half of the compute units idle is cut in two along K (two partial
 // sums into a zeroed Y: the order of two addends does not matter).
 template <bool DENSE>
-int launch_pipe(const uint8_t* wmat, const uint16_t* x, float* d_y, uint32_t M, uint32_t Nc, uint32_t K, uint32_t ldy, hipStream_t s) {
+int launch_pipe(const uint8_t* wmat, const uint16_t* x, float* d_y, uint32_t M, uint32_t Nc, uint32_t K, uint32_t ldy, hipStream_t s,
+                bool y_is_zero = false) {
     static std::atomic<uint64_t> attr_done[2];
-    const uint32_t ntn = (Nc + PBN - 1) / PBN, cus = (uint32_t)device_cu_count();
-    const bool wide = M > 256u && ntn * ((M + 255u) / 256u) * 2u > cus;
-    const uint32_t tbm = wide ? 256u : 128u, mt = (M + tbm - 1) / tbm;
-    const uint32_t ksplit = ntn * mt * 2u <= cus && (K / PK) % 8u == 0u ? 2u : 1u;
-    if (ksplit > 1u) {
+    const PipePlan pl = pipe_plan(M, Nc, K);
+    const bool wide = pl.wide;
+    const uint32_t ntn = pl.ntn, tbm = pl.tbm, mt = pl.mt, ksplit = pl.ksplit;
+    if (ksplit > 1u && !y_is_zero) {
         if (ldy == Nc) {
             hipLaunchKernelGGL(zero_y_kernel, dim3((uint32_t)std::min<size_t>(((size_t)M * Nc + 255) / 256, 4096)), dim3(256), 0, s, d_y, (size_t)M * Nc);
         } else {
@@ -502,11 +535,13 @@ int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d
     const uint32_t Mpad = ((uint32_t)M + BM - 1) / BM * BM;
     uint16_t* xp = nullptr;
     if (int rc = stream_scratch(s, kScratchGemmX, (size_t)Mpad * K * 2, reinterpret_cast<void**>(&xp))) return rc;
-    uint32_t gx = (K + 255) / 256;
+    // the launch that follows adds two K halves into Y: cleared here, in the same launch
+    const bool clear_y = big && pipe_plan((uint32_t)M, N, K).ksplit > 1u;
+    uint32_t gx = std::max<uint32_t>((K / 8u + 255u) / 256u, clear_y ? (N / 4u + 255u) / 256u : 1u);
     if (gx > 64) gx = 64;
-    hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad);
+    hipLaunchKernelGGL(permute_x_kernel, dim3(gx, Mpad), dim3(256), 0, s, d_x, xp, (uint32_t)M, K, Mpad, clear_y ? d_y : (float*)nullptr, N, N);
     OILHIP_HIP(hipGetLastError());
-    if (big) return launch_pipe<false>(w.d_payload, xp, d_y, (uint32_t)M, N, K, N, s);
+    if (big) return launch_pipe<false>(w.d_payload, xp, d_y, (uint32_t)M, N, K, N, s, clear_y);
     return launch<2, 2>(w, xp, d_y, (uint32_t)M, Mpad, s);
 }
 
