@@ -202,7 +202,8 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     // activations are loaded once and stay in registers) for row slab blockIdx.x / ksplit.  Two parts add into a zeroed
     // y with float atomics (two addends: the sum does not depend on their order); three or more parts write their sums
     // to `partial` and the workgroup that arrives last at the slab's counter adds them in ascending order
-    const uint32_t slab = ksplit > 1u ? bid / ksplit : bid, part = ksplit > 1u ? bid % ksplit : 0u;
+    uint32_t slab = bid, part = 0u;
+    if (ksplit > 1u) { slab = bid / ksplit; part = bid - slab * ksplit; }   // (a uniform branch: no division otherwise)
     static_assert(NT == 1 || !HALF, "passes of 8 tokens have one token tile");
     constexpr int BPW = NT == 2 ? 1 : 2;                                   // blocks of the row per wavefront and pass
     constexpr uint32_t PB = 8u * BPW;                                      // blocks per pass
@@ -211,8 +212,9 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     // is block 8 b2 + wave of the pass, so such a part keeps every wavefront busy with one block and takes half the
     // time (56 blocks: 16 + 16 + 16 + 8 is three and a half units of work, four parts of 14 are four).
     const bool full_parts = ksplit > 1u && bpr - (ksplit - 1u) * PB <= PB / 2u;
-    const uint32_t blk_lo = full_parts ? part * PB : bpr * part / ksplit;
-    const uint32_t blk_hi = full_parts ? (blk_lo + PB < bpr ? blk_lo + PB : bpr) : bpr * (part + 1u) / ksplit;
+    uint32_t blk_lo = 0u, blk_hi = bpr;
+    if (full_parts) { blk_lo = part * PB; blk_hi = blk_lo + PB < bpr ? blk_lo + PB : bpr; }
+    else if (ksplit > 1u) { blk_lo = bpr * part / ksplit; blk_hi = bpr * (part + 1u) / ksplit; }
     const uint32_t npass = (blk_hi - blk_lo + PB - 1u) / PB;
 
     // groups of 16 rows [g0, g1) of this workgroup
@@ -277,9 +279,14 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
             reinterpret_cast<uint4*>(tab)[tid + 512u * k] = make_uint4(e_hi, e_lo, e_hi, e_lo);
         }
     }
-    for (uint32_t i = tid; i < (uint32_t)NT * (blk_hi - blk_lo) * 16u; i += 512u) {
-        const uint32_t t = i / ((blk_hi - blk_lo) * 16u), rem = i % ((blk_hi - blk_lo) * 16u);
-        undo[i] = ldexpf(1.0f, -xp_exp[(t * bpr + blk_lo) * 16u + rem]);
+    {
+        const uint32_t per_tile = (blk_hi - blk_lo) * 16u;
+        for (uint32_t i = tid; i < (uint32_t)NT * per_tile; i += 512u) {
+            const uint32_t t = NT == 2 && i >= per_tile ? 1u : 0u, rem = i - t * per_tile;
+            // 2^-e: a bit pattern where it is a normal number, else (activations below 2^-113) the library call
+            const int e = xp_exp[(t * bpr + blk_lo) * 16u + rem], be = 127 - e;
+            undo[i] = be > 0 && be < 255 ? __uint_as_float((uint32_t)be << 23) : ldexpf(1.0f, -e);
+        }
     }
     bool table_synced = false;
 
