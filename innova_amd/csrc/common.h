@@ -140,4 +140,6 @@ int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M
 int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_any_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
+// plain uniform OIL4, more than 256 tokens: activations in fragment order straight from memory (gemm_oil4_frag.hip)
+int launch_gemm_oil4_frag(const oilhip_weights& w, const void* d_x, bool x_is_f32, float* d_y, int M, hipStream_t s);
 }  // namespace oilhip

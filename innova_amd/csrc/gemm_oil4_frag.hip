@@ -1,0 +1,457 @@
+// gemm_oil4_frag.hip -- prefill GEMM over uniform OIL4 tensors for batches of more than 256 tokens:
+// Y[M][N] = X[M][K] . W^T, X in bf16 (or FP32, rounded once to bf16), W dequantized to bf16 on the fly,
+// v_mfma_f32_32x32x16_bf16 with FP32 accumulation, FP32 output.  Same contraction as the reference's FP32
+// prefill (Qwen35Engine::gemm with B up to 512, src/adapters/tools/qwen35_engine.cpp:47-85,630-753) over
+// dequant_lattice blocks (src/block_codec.cpp:173-182).
+//
+// Shape of the kernel.  A workgroup is four wavefronts, one per SIMD, as 2 x 2; a wavefront owns FM x FN
+// blocks of 32 x 32 outputs (4 x 4: a 256 x 256 workgroup tile, 256 accumulator registers per lane), so one
+// 16-byte operand fragment feeds four matrix instructions.
+//  * Activations never pass through LDS.  A pre-pass writes X' in the order the matrix instruction wants its
+//    A operand: [32-token block][16-column group][lane][8 bf16], columns in nibble order (the 4-bit index of
+//    weight i of a 256-weight block sits at nibble 4 + i - i/64; nibbles 0..3 are the FP16 scale and meet
+//    zeros in X').  A fragment is then one coalesced 1 KB load straight into registers, issued one 64-column
+//    step ahead.
+//  * Weights: a lane loads 16 bytes (32 nibbles) of one weight row per step, turns every packed byte into two
+//    FP32 levels through the byte -> (level, level) pair table in LDS (the table of the decode GEMV), multiplies
+//    by the block's FP16 scale, rounds once to bf16 and stores the result in B-operand fragment order.  Each
+//    weight is decoded once per workgroup; the four wavefronts read the fragments back with conflict-free
+//    16-byte LDS reads.  Two tile buffers, one workgroup barrier per step: the fragments of step s are read
+//    and the tile of step s + 1 is written between the same two barriers, and the decode is cut into four
+//    quarters that ride behind the four groups of matrix instructions of a step.
+//  * Tiles that do not fill a whole round of compute units are cut in two along K (two addends into a zeroed Y:
+//    the sum does not depend on their order); tile order keeps the workgroups of one XCD on few token blocks and
+//    neighbouring weight rows so that its L2 serves most of their reads.
+#include <hip/hip_fp16.h>
+
+#include <algorithm>
+#include <type_traits>
+
+#include "common.h"
+#include "oil4_lds.h"
+
+namespace oilhip {
+namespace {
+
+using oil4::kTabBytes;
+using oil4::level_literal;
+using oil4::LevelPair;
+using oil4::lookup;
+using oil4::u32x4;
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// Tile order: token blocks in groups of four; inside a group weight-row blocks ascending, the group's token blocks
+// innermost.  A run of consecutive tiles therefore covers few token blocks and neighbouring weight rows.
+__host__ __device__ inline void frag_tile_of(uint32_t T, uint32_t MT, uint32_t NT, uint32_t& mt, uint32_t& nt) {
+    const uint32_t per = 4u * NT, lastg = (MT - 1u) / 4u;
+    uint32_t mg = T / per;
+    if (mg > lastg) mg = lastg;
+    const uint32_t rem = T - mg * per, left = MT - 4u * mg, gm = left < 4u ? left : 4u;
+    nt = rem / gm;
+    mt = 4u * mg + rem % gm;
+}
+
+// Workgroups are dealt to the eight XCDs in turn; XCD x takes the x-th run of n / 8 consecutive items.
+__device__ inline uint32_t xcd_chunk(uint32_t b, uint32_t n) {
+    const uint32_t x = b & 7u, q = b >> 3, c = n >> 3, r = n & 7u;
+    return (x < r ? x * (c + 1u) : r * (c + 1u) + (x - r) * c) + q;
+}
+
+struct FragGrid {
+    uint32_t MT, NT;        // tiles along tokens and weight rows
+    uint32_t nfull;         // the first nfull tiles (in tile order) run all of K in one workgroup
+    uint32_t ksplit;        // the others are cut into this many parts along K (1 or 2) ...
+    uint32_t halves;        // ... or into two halves along the weight rows (2; 256-row tiles only), each with all of K
+};
+
+// X ([M][K], bf16 bit patterns or FP32) -> X' in A-fragment order, rows >= M zero.  One wavefront writes one 1 KB
+// fragment: lane = 32 * (column half) + token % 32 holds columns 16 g + 8 half .. + 7 of X' (nibble order).
+// Workgroups past the packing ones clear the Y tiles whose K parts are added: tile nfull + (index).
+template <bool F32, int TM, int TN>
+__global__ void __launch_bounds__(256)
+pack_x_frag_kernel(const void* __restrict__ xin, uint16_t* __restrict__ xf, uint32_t M, uint32_t K, uint32_t npack,
+                   float* __restrict__ y, uint32_t N, uint32_t ldy, FragGrid gr) {
+    const uint32_t tid = threadIdx.x;
+    if (blockIdx.x >= npack) {
+        uint32_t mt, nt;
+        frag_tile_of(gr.nfull + (blockIdx.x - npack), gr.MT, gr.NT, mt, nt);
+        const uint32_t m0 = mt * TM, n0 = nt * TN;
+        const uint32_t nc = N - n0 < (uint32_t)TN ? N - n0 : (uint32_t)TN;
+        for (uint32_t r = tid >> 6; r < (uint32_t)TM && m0 + r < M; r += 4u) {
+            float* yr = y + (size_t)(m0 + r) * ldy + n0;
+            for (uint32_t c = tid & 63u; c < nc; c += 64u) yr[c] = 0.0f;
+        }
+        return;
+    }
+    const uint32_t G = K >> 4, gq = G >> 2;
+    const uint32_t mb = blockIdx.x / gq, g = (blockIdx.x % gq) * 4u + (tid >> 6);
+    const uint32_t lane = tid & 63u, m = mb * 32u + (lane & 31u);
+    const uint32_t c = g * 16u + (lane >> 5) * 8u, p0 = c & 255u;
+    // X' column p of a block (p >= 4) is X column p - 4 + (slots before it): the eight columns of this lane come
+    // from the 16 aligned X columns [c - 8, c + 8), window index k + 4 + slots
+    uint16_t e[16];
+#pragma unroll
+    for (int k = 0; k < 16; ++k) e[k] = 0;
+    if (m < M) {
+        if constexpr (F32) {
+            const float* xr = reinterpret_cast<const float*>(xin) + (size_t)m * K + c;
+#pragma unroll
+            for (int h = 0; h < 4; ++h) {
+                if (h < 2 && p0 == 0u) continue;
+                const float4 f = *reinterpret_cast<const float4*>(xr - 8 + 4 * h);
+                const __bf16 b0 = (__bf16)f.x, b1 = (__bf16)f.y, b2 = (__bf16)f.z, b3 = (__bf16)f.w;
+                e[4 * h] = *reinterpret_cast<const uint16_t*>(&b0); e[4 * h + 1] = *reinterpret_cast<const uint16_t*>(&b1);
+                e[4 * h + 2] = *reinterpret_cast<const uint16_t*>(&b2); e[4 * h + 3] = *reinterpret_cast<const uint16_t*>(&b3);
+            }
+        } else {
+            const uint16_t* xr = reinterpret_cast<const uint16_t*>(xin) + (size_t)m * K + c;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                if (h == 0 && p0 == 0u) continue;
+                const uint4 q = *reinterpret_cast<const uint4*>(xr - 8 + 8 * h);
+                e[8 * h] = (uint16_t)q.x; e[8 * h + 1] = (uint16_t)(q.x >> 16); e[8 * h + 2] = (uint16_t)q.y; e[8 * h + 3] = (uint16_t)(q.y >> 16);
+                e[8 * h + 4] = (uint16_t)q.z; e[8 * h + 5] = (uint16_t)(q.z >> 16); e[8 * h + 6] = (uint16_t)q.w; e[8 * h + 7] = (uint16_t)(q.w >> 16);
+            }
+        }
+    }
+    uint16_t v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t p = p0 + k, sl = (p >= 67u) + (p >= 130u) + (p >= 193u);
+        const uint16_t t = sl == 0u ? e[k + 4] : sl == 1u ? e[k + 5] : sl == 2u ? e[k + 6] : e[k + 7];
+        v[k] = p >= 4u ? t : (uint16_t)0;
+    }
+    uint4 o;
+    o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+    o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+    *reinterpret_cast<uint4*>(xf + (((size_t)mb * G + g) * 64u + lane) * 8u) = o;
+}
+
+template <int V> using IC = std::integral_constant<int, V>;
+
+// One workgroup's tile: tokens [m0, m0 + 64 FM), weight rows [n0, n0 + 64 FN), part kpart of `parts` along K.
+template <int FM, int FN>
+__device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xf, float* __restrict__ Y,
+                                          uint32_t M, uint32_t N, uint32_t K, uint32_t ldy, uint32_t m0, uint32_t n0,
+                                          uint32_t kpart, uint32_t parts) {
+    static_assert((FN == 2 || FN == 4) && (FM == 2 || FM == 4), "wavefront tiles of 64 or 128 tokens and weight rows");
+    constexpr int TN = 64 * FN;                     // weight rows of the workgroup tile
+    constexpr int NB = TN / 32;                     // 32-row blocks of weight rows in the tile
+    constexpr int NBW = NB / 4;                     // ... that one wavefront decodes
+    constexpr int BUF = NB * 4096;                  // bytes of one tile buffer: [NB][4 column groups][64 lanes][16 B]
+    extern __shared__ __align__(16) uint8_t lds[];
+    float* tab = reinterpret_cast<float*>(lds);     // pair table at LDS offset 0 (the look-up builds absolute addresses)
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));    // scalar: buffer resources and LDS bases depend on it
+    const uint32_t wm = wave >> 1, wn = wave & 1u;
+    const uint32_t bpr = K >> 8, G = K >> 4;
+    // steps of 64 columns [kbeg, kend): whole blocks, so that both are multiples of 4
+    const uint32_t bsplit = (bpr + parts - 1u) / parts;
+    const uint32_t kbeg = kpart * bsplit * 4u, kend = (kpart + 1u == parts ? bpr : (kpart + 1u) * bsplit) * 4u;
+
+    {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 256 * k
+        const float lv_lane = level_literal(lane & 15u);
+        const float lo = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+#pragma unroll
+        for (int k = 0; k < 16; ++k) {
+            const float hi = level_literal(k);
+            reinterpret_cast<float4*>(tab)[tid + 256u * k] = make_float4(lo, hi, lo, hi);
+        }
+    }
+
+    const uint32_t nrows = N - n0 < (uint32_t)TN ? N - n0 : (uint32_t)TN;
+    const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(W + (size_t)n0 * bpr * 128u), 0, (int)((uint64_t)nrows * bpr * 128u), 0x00020000);
+    const uint32_t r32 = lane & 31u, hh = lane >> 5;
+    const uint32_t lanebase = r32 * 8u;
+    // weight bytes of this lane: row (wave * NBW + j) * 32 + r32 of the tile, 16 bytes at step * 32 + hh * 16
+    uint32_t woff[NBW];
+#pragma unroll
+    for (int j = 0; j < NBW; ++j) woff[j] = ((wave * NBW + j) * 32u + r32) * bpr * 128u;
+    // A fragments through a buffer resource over this wavefront's FM token blocks: lane part in the vector offset,
+    // the 16-column group in the scalar offset, no address arithmetic per load
+    const __amdgpu_buffer_rsrc_t xrs = __builtin_amdgcn_make_buffer_rsrc(
+        (void*)(Xf + ((size_t)(m0 / 32u + wm * FM) * G) * 512u), 0, (int)((uint32_t)FM * G * 1024u), 0x00020000);
+    uint32_t xoff[FM];
+#pragma unroll
+    for (int i = 0; i < FM; ++i) xoff[i] = (uint32_t)i * G * 1024u + lane * 16u;
+
+    u32x4 fa[4][FM];            // A fragments of one step, slot = column group of the step
+    u32x4 fb[2][FN];            // B fragments, set = column group & 1
+    u32x4 wr[4][NBW];           // packed weights of four steps in flight, slot = step & 3
+    float scA[NBW], scB[NBW];   // block scales of the current and the next 256-column block
+    uint32_t scraw[NBW];
+    uint32_t tadr[NBW][4];      // table addresses of the quarter that is decoded next
+    oil4::f32x2 tv[NBW][4];     // its table entries
+
+    const uint32_t glast = kend * 4u - 1u;
+    auto load_a1 = [&](int slot, int i, uint32_t g) {
+        g = g < glast ? g : glast;
+        fa[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, xoff[i], g * 1024u, 0);
+    };
+    auto load_w = [&](int slot, uint32_t step) {
+#pragma unroll
+        for (int j = 0; j < NBW; ++j) wr[slot][j] = __builtin_amdgcn_raw_buffer_load_b128(wrs, woff[j] + hh * 16u, step * 32u, 0);
+    };
+    auto load_scale = [&](uint32_t blk) {
+#pragma unroll
+        for (int j = 0; j < NBW; ++j) scraw[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], blk * 128u, 0);
+    };
+    auto cvt_scale = [&](float (&dst)[NBW]) {
+#pragma unroll
+        for (int j = 0; j < NBW; ++j) dst[j] = __half2float(__ushort_as_half((unsigned short)scraw[j]));
+    };
+    // A quarter of a step's decode is NBW dwords (8 nibbles each) per lane -> NBW 16-byte pieces in fragment order.
+    // Quarter q, piece t is dword (q * NBW + t) % 4 of the lane's 16 bytes of weight-row block (q * NBW + t) / 4.
+    // Three phases that the main loop places apart: table addresses (one v_perm_b32 per byte), table reads,
+    // scale + round + store.
+    auto q_addr = [&](auto qc, int slot, int t, int b) {
+        constexpr int q = decltype(qc)::value;
+        const int e = q * NBW + t, j = e >> 2, d = e & 3;
+        const uint32_t word = d == 0 ? wr[slot][j].x : d == 1 ? wr[slot][j].y : d == 2 ? wr[slot][j].z : wr[slot][j].w;
+        tadr[t][b] = __builtin_amdgcn_perm(word, lanebase, 0x0C0C0000u | ((4u + (uint32_t)b) << 8));
+    };
+    auto q_read = [&](int t, int b) { tv[t][b] = *(oil4::lds_cfloat2*)(uintptr_t)tadr[t][b]; };
+    uint32_t tout[NBW][4];
+    auto q_math = [&](int t, int b, float s) {
+        const bf16x2 o = bf16x2{(__bf16)(tv[t][b].x * s), (__bf16)(tv[t][b].y * s)};
+        tout[t][b] = *reinterpret_cast<const uint32_t*>(&o);
+    };
+    const uint32_t wbase = kTabBytes + wave * (NBW * 4096u) + hh * 2048u + r32 * 16u;
+    auto q_store = [&](auto qc, int t, int buf) {
+        constexpr int q = decltype(qc)::value;
+        const int e = q * NBW + t, j = e >> 2, d = e & 3;
+        *reinterpret_cast<u32x4*>(lds + wbase + buf * BUF + j * 4096 + (d >> 1) * 1024 + (d & 1) * 512) =
+            u32x4{tout[t][0], tout[t][1], tout[t][2], tout[t][3]};
+    };
+    const uint32_t rbase = kTabBytes + wn * (FN * 4096u) + lane * 16u;
+    auto read_frags = [&](int kk, int buf, int set) {
+#pragma unroll
+        for (int j = 0; j < FN; ++j) fb[set][j] = *reinterpret_cast<const u32x4*>(lds + rbase + buf * BUF + j * 4096 + kk * 1024);
+    };
+    f32x16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
+    auto mfma1 = [&](int kk, int i, int j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&fa[kk][i]),
+                                                            *reinterpret_cast<const bf16x8*>(&fb[kk & 1][j]), acc[i][j], 0, 0, 0);
+    };
+
+    // One group: the FM * FN matrix instructions of column group kk of step s, and behind them, in fixed places
+    // (nothing moves across a matrix instruction): at the start the table reads of quarter QC (addresses formed in
+    // the group before) and the fragment reads RK of buffer rbuf into set RK & 1; behind the last use of each A
+    // fragment its reload for the next step; the table addresses of the next quarter (QN, weights in slot nslot);
+    // scale, round and store of quarter QC into buffer wbuf.
+    auto group = [&](auto kkc, auto qc, auto qn, int rk, int rbuf, int wbuf, int nslot, const float (&sc)[NBW], uint32_t gnext) {
+        constexpr int kk = decltype(kkc)::value;
+        constexpr int NM = FM * FN, NU = NBW * 4;            // matrix instructions, decode units (bytes per lane) of the group
+        // places: addresses behind instructions A0 .. A0 + NU/PA - 1, math from M0 on
+        constexpr int PA = NM >= 16 ? 2 : 4;                 // addresses per place
+        constexpr int A0 = NM >= 16 ? 1 : 0;
+        constexpr int M0 = NM >= 16 ? 6 : 1;
+        constexpr int PM = NM >= 16 ? 1 : 2;                 // math units per place
+#pragma unroll
+        for (int t = 0; t < NBW; ++t)
+#pragma unroll
+            for (int b = 0; b < 4; ++b) q_read(t, b);
+        read_frags(rk, rbuf, rk & 1);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int n = 0; n < NM; ++n) {
+            const int i = n / FN, j = n % FN;
+            mfma1(kk, i, j);
+            if (j == FN - 1) load_a1(kk, i, gnext);
+            if (n >= A0 && (n - A0) * PA < NU) {
+#pragma unroll
+                for (int a = 0; a < PA; ++a) { const int un = (n - A0) * PA + a; q_addr(qn, nslot, un >> 2, un & 3); }
+            }
+            if (n >= M0 && (n - M0) * PM < NU) {
+#pragma unroll
+                for (int a = 0; a < PM; ++a) {
+                    const int un = (n - M0) * PM + a;
+                    q_math(un >> 2, un & 3, sc[(decltype(qc)::value * NBW + (un >> 2)) >> 2]);
+                    if ((un & 3) == 3) q_store(qc, un >> 2, wbuf);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // ---- prologue: loads of the first steps, tile kbeg whole and the table addresses of the first quarter of tile kbeg + 1
+    load_w(1, kbeg + 1u);
+    load_w(2, kbeg + 2u);
+    load_w(3, kbeg + 3u);
+    load_w(0, kbeg);
+    // both scales ahead of the A loads: every wait on them then leaves a whole step of loads in flight
+    uint32_t scraw0[NBW], scraw1[NBW];
+#pragma unroll
+    for (int j = 0; j < NBW; ++j) {
+        scraw0[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], (kbeg >> 2) * 128u, 0);
+        scraw1[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], ((kbeg >> 2) + 1u) * 128u, 0);
+    }
+#pragma unroll
+    for (int kk = 0; kk < 3; ++kk)
+#pragma unroll
+        for (int i = 0; i < FM; ++i) load_a1(kk, i, kbeg * 4u + (uint32_t)kk);
+#pragma unroll
+    for (int j = 0; j < NBW; ++j) {
+        scA[j] = __half2float(__ushort_as_half((unsigned short)scraw0[j]));
+        scB[j] = __half2float(__ushort_as_half((unsigned short)scraw1[j]));
+    }
+    __syncthreads();                                   // table complete
+    {
+        auto whole = [&](auto qc) {
+#pragma unroll
+            for (int t = 0; t < NBW; ++t) {
+#pragma unroll
+                for (int b = 0; b < 4; ++b) { q_addr(qc, 0, t, b); q_read(t, b); }
+#pragma unroll
+                for (int b = 0; b < 4; ++b) q_math(t, b, scA[(decltype(qc)::value * NBW + t) >> 2]);
+                q_store(qc, t, 0);
+            }
+        };
+        whole(IC<0>{}); whole(IC<1>{}); whole(IC<2>{}); whole(IC<3>{});
+    }
+#pragma unroll
+    for (int t = 0; t < NBW; ++t)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) q_addr(IC<0>{}, 1, t, b);
+    load_w(0, kbeg + 4u);
+#pragma unroll
+    for (int i = 0; i < FM; ++i) load_a1(3, i, kbeg * 4u + 3u);
+    __syncthreads();
+    read_frags(0, 0, 0);
+    // the first quarter of tile kbeg + 1 goes to buffer 1 ahead of the loop (nobody reads that buffer yet)
+#pragma unroll
+    for (int t = 0; t < NBW; ++t) {
+#pragma unroll
+        for (int b = 0; b < 4; ++b) q_read(t, b);
+#pragma unroll
+        for (int b = 0; b < 4; ++b) q_math(t, b, scA[t >> 2]);
+        q_store(IC<0>{}, t, 1);
+    }
+#pragma unroll
+    for (int t = 0; t < NBW; ++t)
+#pragma unroll
+        for (int b = 0; b < 4; ++b) q_addr(IC<1>{}, 1, t, b);
+
+    // ---- main loop: one 256-column block (four steps) per trip.  In step s (u = s & 3, tile s in buffer u & 1) the
+    // groups 0..2 read the fragments of column groups 1..3 and decode the quarters 1..3 of tile s + 1 into the other
+    // buffer; after the barrier group 3 reads the first fragments of tile s + 1 and decodes the first quarter of
+    // tile s + 2 into the buffer that tile s has just left.  Tile s + 1 belongs to the next block from u = 3 on,
+    // tile s + 2 from u = 2 on.  The weights of tile s + 5 replace those of tile s + 1 when its last quarter is read.
+    auto step = [&](auto uc, uint32_t s) {
+        constexpr int u = decltype(uc)::value, cur = u & 1, nxt = cur ^ 1;
+        const float (&sc1)[NBW] = u == 3 ? scB : scA;
+        const float (&sc2)[NBW] = u >= 2 ? scB : scA;
+        group(IC<0>{}, IC<1>{}, IC<2>{}, 1, cur, nxt, (u + 1) & 3, sc1, s * 4u + 4u);
+        group(IC<1>{}, IC<2>{}, IC<3>{}, 2, cur, nxt, (u + 1) & 3, sc1, s * 4u + 5u);
+        group(IC<2>{}, IC<3>{}, IC<0>{}, 3, cur, nxt, (u + 2) & 3, sc1, s * 4u + 6u);
+        load_w((u + 1) & 3, s + 5u);
+        if constexpr (u == 0) load_scale((s >> 2) + 2u);
+        __syncthreads();
+        group(IC<3>{}, IC<0>{}, IC<1>{}, 0, nxt, cur, (u + 2) & 3, sc2, s * 4u + 7u);
+    };
+    for (uint32_t s = kbeg; s < kend; s += 4u) {
+        step(IC<0>{}, s);
+        step(IC<1>{}, s + 1u);
+        step(IC<2>{}, s + 2u);
+        step(IC<3>{}, s + 3u);
+#pragma unroll
+        for (int j = 0; j < NBW; ++j) scA[j] = scB[j];
+        cvt_scale(scB);
+    }
+
+    // C layout of the 32x32 matrix instruction: lane l holds column l % 32; register v holds row 8 * (v / 4) + 4 * (l / 32) + v % 4
+#pragma unroll
+    for (int i = 0; i < FM; ++i)
+#pragma unroll
+        for (int j = 0; j < FN; ++j) {
+            const uint32_t col = n0 + (wn * FN + j) * 32u + r32;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t row = m0 + (wm * FM + i) * 32u + 8u * (v >> 2) + 4u * hh + (v & 3u);
+                if (row < M && col < N) {
+                    if (parts > 1u) unsafeAtomicAdd(Y + (size_t)row * ldy + col, acc[i][j][v]);
+                    else Y[(size_t)row * ldy + col] = acc[i][j][v];
+                }
+            }
+        }
+}
+
+template <int FM, int FN>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+gemm_oil4_frag_kernel(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xf, float* __restrict__ Y,
+                      uint32_t M, uint32_t N, uint32_t K, uint32_t ldy, FragGrid gr) {
+    constexpr int TM = 64 * FM, TN = 64 * FN;
+    const uint32_t b = blockIdx.x;
+    uint32_t mt, nt;
+    if (b < gr.nfull) {
+        frag_tile_of(xcd_chunk(b, gr.nfull), gr.MT, gr.NT, mt, nt);
+        frag_tile<FM, FN>(W, Xf, Y, M, N, K, ldy, mt * TM, nt * TN, 0u, 1u);
+        return;
+    }
+    // the tiles of the last round, in two pieces each: 256-row tiles as halves of 128 weight rows, others as halves of K
+    const uint32_t u = xcd_chunk(b - gr.nfull, (gr.MT * gr.NT - gr.nfull) * 2u);
+    frag_tile_of(gr.nfull + u / 2u, gr.MT, gr.NT, mt, nt);
+    if constexpr (FN == 4) {
+        const uint32_t n0 = nt * TN + (u & 1u) * (TN / 2);
+        if (n0 < N) frag_tile<FM, 2>(W, Xf, Y, M, N, K, ldy, mt * TM, n0, 0u, 1u);
+    } else {
+        frag_tile<FM, FN>(W, Xf, Y, M, N, K, ldy, mt * TM, nt * TN, u & 1u, 2u);
+    }
+}
+
+template <int FM, int FN, bool F32>
+int launch_frag(const oilhip_weights& w, const void* d_x, float* d_y, uint32_t M, hipStream_t s) {
+    constexpr int TM = 64 * FM, TN = 64 * FN;
+    const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols, cus = (uint32_t)device_cu_count();
+    FragGrid gr;
+    gr.MT = (M + TM - 1) / TM;
+    gr.NT = (N + TN - 1) / TN;
+    const uint32_t tiles = gr.MT * gr.NT, tail = tiles % cus;
+    // A last round that fills at most half of the compute units is cut in two: 256-row tiles into halves of 128 weight
+    // rows (each with all of K: no partial sums), smaller tiles along K (two addends into a cleared Y; a row of one
+    // block cannot be cut).
+    const bool split = tail != 0u && tail * 2u <= cus && (FN == 4 || K >= 512u);
+    gr.nfull = split ? tiles - tail : tiles;
+    gr.halves = split && FN == 4 ? 2u : 1u;
+    gr.ksplit = split && FN != 4 ? 2u : 1u;
+    const uint32_t Mpad = gr.MT * TM;
+    uint16_t* xf = nullptr;
+    if (int rc = stream_scratch(s, kScratchGemmX, (size_t)Mpad * K * 2, reinterpret_cast<void**>(&xf))) return rc;
+    const uint32_t npack = (Mpad / 32u) * (K >> 6), nzero = gr.ksplit > 1u ? tiles - gr.nfull : 0u;
+    hipLaunchKernelGGL((pack_x_frag_kernel<F32, TM, TN>), dim3(npack + nzero), dim3(256), 0, s, d_x, xf, M, K, npack, d_y, N, N, gr);
+    OILHIP_HIP(hipGetLastError());
+    static std::atomic<uint64_t> attr_done{0};
+    auto kern = gemm_oil4_frag_kernel<FM, FN>;
+    if (int rc = ensure_max_lds(attr_done, reinterpret_cast<const void*>(kern), 160 * 1024)) return rc;
+    const size_t lds_bytes = (size_t)kTabBytes + 2ull * (TN / 32) * 4096;
+    hipLaunchKernelGGL(kern, dim3(gr.nfull + (tiles - gr.nfull) * (split ? 2u : 1u)), dim3(256), lds_bytes, s, w.d_payload, xf, d_y, M, N, K, N, gr);
+    OILHIP_HIP(hipGetLastError());
+    return OILHIP_OK;
+}
+
+}  // namespace
+
+// Prefill over a plain uniform OIL4 tensor with the fragment-order kernel; x is bf16 bit patterns, or FP32 when x_is_f32.
+int launch_gemm_oil4_frag(const oilhip_weights& w, const void* d_x, bool x_is_f32, float* d_y, int M, hipStream_t s) {
+    if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
+    const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols, cus = (uint32_t)device_cu_count();
+    if ((uint64_t)256 * (K >> 8) * 128u >= 0x80000000ull) return fail(OILHIP_E_ARG, "rows too wide for the prefill kernel");
+    // 256 x 256 tiles unless they would leave three quarters of the compute units without work even when cut along K
+    const uint32_t big_tiles = (((uint32_t)M + 255u) / 256u) * ((N + 255u) / 256u);
+    const bool small = big_tiles * 4u <= cus;
+    if (small) return x_is_f32 ? launch_frag<2, 2, true>(w, d_x, d_y, (uint32_t)M, s) : launch_frag<2, 2, false>(w, d_x, d_y, (uint32_t)M, s);
+    return x_is_f32 ? launch_frag<4, 4, true>(w, d_x, d_y, (uint32_t)M, s) : launch_frag<4, 4, false>(w, d_x, d_y, (uint32_t)M, s);
+}
+
+}  // namespace oilhip
