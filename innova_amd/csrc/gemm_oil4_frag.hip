@@ -132,6 +132,11 @@ pack_x_frag_kernel(const void* __restrict__ xin, uint16_t* __restrict__ xf, uint
 
 template <int V> using IC = std::integral_constant<int, V>;
 
+#ifndef OILHIP_FRAG_AHEAD
+#define OILHIP_FRAG_AHEAD 2
+#endif
+constexpr int kFragAhead = OILHIP_FRAG_AHEAD;
+
 // One workgroup's tile: tokens [m0, m0 + 64 FM), weight rows [n0, n0 + 64 FN), part kpart of `parts` along K.
 template <int FM, int FN>
 __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const uint16_t* __restrict__ Xf, float* __restrict__ Y,
@@ -143,7 +148,7 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
     constexpr int NBW = NB / 4;                     // ... that one wavefront decodes
     constexpr int BUF = NB * 4096;                  // bytes of one tile buffer: [NB][4 column groups][64 lanes][16 B]
     extern __shared__ __align__(16) uint8_t lds[];
-    float* tab = reinterpret_cast<float*>(lds);     // pair table at LDS offset 0 (the look-up builds absolute addresses)
+    uint32_t* tab = reinterpret_cast<uint32_t*>(lds);   // pair table at LDS offset 0 (the look-up builds absolute addresses)
 
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));    // scalar: buffer resources and LDS bases depend on it
@@ -153,13 +158,14 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
     const uint32_t bsplit = (bpr + parts - 1u) / parts;
     const uint32_t kbeg = kpart * bsplit * 4u, kend = (kpart + 1u == parts ? bpr : (kpart + 1u) * bsplit) * 4u;
 
-    {   // pair table from literals: float4 e = (lo, hi, lo, hi) of byte value v = e >> 4; e = tid + 256 * k
-        const float lv_lane = level_literal(lane & 15u);
-        const float lo = __int_as_float(__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), __float_as_int(lv_lane)));
+    {   // pair table from literals: row v (256 bytes) = 64 copies of fp16(level[v & 15]) | fp16(level[v >> 4]) << 16;
+        // uint4 e = tid + 256 * k belongs to row e >> 4: low level (tid >> 4) & 15, high level k
+        const uint32_t lv_lane = (uint32_t)__half_as_ushort(__float2half_rn(level_literal(lane & 15u)));
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_ds_bpermute((int)(((tid >> 4) & 15u) * 4u), (int)lv_lane);
 #pragma unroll
         for (int k = 0; k < 16; ++k) {
-            const float hi = level_literal(k);
-            reinterpret_cast<float4*>(tab)[tid + 256u * k] = make_float4(lo, hi, lo, hi);
+            const uint32_t e = lo | ((uint32_t)__half_as_ushort(__float2half_rn(level_literal(k))) << 16);
+            reinterpret_cast<uint4*>(tab)[tid + 256u * k] = make_uint4(e, e, e, e);
         }
     }
 
@@ -167,7 +173,7 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
     const __amdgpu_buffer_rsrc_t wrs = __builtin_amdgcn_make_buffer_rsrc(
         (void*)(W + (size_t)n0 * bpr * 128u), 0, (int)((uint64_t)nrows * bpr * 128u), 0x00020000);
     const uint32_t r32 = lane & 31u, hh = lane >> 5;
-    const uint32_t lanebase = r32 * 8u;
+    const uint32_t lanebase = lane * 4u;                   // this lane's copy of a table row
     // weight bytes of this lane: row (wave * NBW + j) * 32 + r32 of the tile, 16 bytes at step * 32 + hh * 16
     uint32_t woff[NBW];
 #pragma unroll
@@ -180,18 +186,23 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
 #pragma unroll
     for (int i = 0; i < FM; ++i) xoff[i] = (uint32_t)i * G * 1024u + lane * 16u;
 
-    u32x4 fa[4][FM];            // A fragments of one step, slot = column group of the step
-    u32x4 fb[2][FN];            // B fragments, set = column group & 1
+    const uint32_t klast = bpr * 4u - 1u;                 // last 64-column step of a row
+    constexpr int AD = kFragAhead;  // steps of A fragments in flight
+    u32x4 fa[AD][4][FM];        // A fragments of AD steps: set = step % AD, slot = column group of the step
+    u32x4 fb[FN];               // B fragments of the column group in work; each is re-read for the next group after its last use
     u32x4 wr[4][NBW];           // packed weights of four steps in flight, slot = step & 3
     float scA[NBW], scB[NBW];   // block scales of the current and the next 256-column block
     uint32_t scraw[NBW];
-    uint32_t tadr[NBW][4];      // table addresses of the quarter that is decoded next
-    oil4::f32x2 tv[NBW][4];     // its table entries
+    // decode pipeline, one quarter of a step per group of matrix instructions and three quarters in flight: table
+    // addresses of quarter g + 2, table reads of quarter g + 1, scale + round + store of quarter g
+    uint32_t tadr[NBW][4];
+    uint32_t tv[2][NBW][4];
 
-    const uint32_t glast = kend * 4u - 1u;
-    auto load_a1 = [&](int slot, int i, uint32_t g) {
-        g = g < glast ? g : glast;
-        fa[slot][i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, xoff[i], g * 1024u, 0);
+    // set = step & 1, slot = column group of the step; sbase = byte offset of the step's first column group.  Loads
+    // run two steps ahead: with the matrix pipe and the LDS returns busy, a fragment that misses L2 needs more than
+    // one step to arrive.
+    auto load_a1 = [&](int set, int slot, int i, uint32_t sbase) {
+        fa[set][slot][i] = __builtin_amdgcn_raw_buffer_load_b128(xrs, xoff[i] + (uint32_t)slot * 1024u, sbase, 0);
     };
     auto load_w = [&](int slot, uint32_t step) {
 #pragma unroll
@@ -207,31 +218,37 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
     };
     // A quarter of a step's decode is NBW dwords (8 nibbles each) per lane -> NBW 16-byte pieces in fragment order.
     // Quarter q, piece t is dword (q * NBW + t) % 4 of the lane's 16 bytes of weight-row block (q * NBW + t) / 4.
-    // Three phases that the main loop places apart: table addresses (one v_perm_b32 per byte), table reads,
-    // scale + round + store.
-    auto q_addr = [&](auto qc, int slot, int t, int b) {
-        constexpr int q = decltype(qc)::value;
+    auto q_addr = [&](int q, int slot, int t, int b) {
         const int e = q * NBW + t, j = e >> 2, d = e & 3;
         const uint32_t word = d == 0 ? wr[slot][j].x : d == 1 ? wr[slot][j].y : d == 2 ? wr[slot][j].z : wr[slot][j].w;
         tadr[t][b] = __builtin_amdgcn_perm(word, lanebase, 0x0C0C0000u | ((4u + (uint32_t)b) << 8));
     };
-    auto q_read = [&](int t, int b) { tv[t][b] = *(oil4::lds_cfloat2*)(uintptr_t)tadr[t][b]; };
+    auto q_read = [&](int set, int t, int b) { tv[set][t][b] = *(oil4::lds_cuint*)(uintptr_t)tadr[t][b]; };
     uint32_t tout[NBW][4];
-    auto q_math = [&](int t, int b, float s) {
-        const bf16x2 o = bf16x2{(__bf16)(tv[t][b].x * s), (__bf16)(tv[t][b].y * s)};
+    // FP16 level x FP32 scale in one instruction each (v_fma_mix_f32; the product is exact in FP32), rounded once to
+    // bf16.  The rounding reads its operands one place after the products write them: placed right behind them it
+    // costs a wait state each time.
+    float tlo[NBW][4], thi[NBW][4];
+    auto q_mul = [&](int set, int t, int b, float s) {
+        typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
+        const f16x2 h = *reinterpret_cast<const f16x2*>(&tv[set][t][b]);
+        tlo[t][b] = __builtin_fmaf((float)h.x, s, 0.0f);
+        thi[t][b] = __builtin_fmaf((float)h.y, s, 0.0f);
+    };
+    auto q_round = [&](int t, int b) {
+        const bf16x2 o = bf16x2{(__bf16)tlo[t][b], (__bf16)thi[t][b]};
         tout[t][b] = *reinterpret_cast<const uint32_t*>(&o);
     };
+    auto q_math = [&](int set, int t, int b, float s) { q_mul(set, t, b, s); q_round(t, b); };
     const uint32_t wbase = kTabBytes + wave * (NBW * 4096u) + hh * 2048u + r32 * 16u;
-    auto q_store = [&](auto qc, int t, int buf) {
-        constexpr int q = decltype(qc)::value;
+    auto q_store = [&](int q, int t, int buf) {
         const int e = q * NBW + t, j = e >> 2, d = e & 3;
         *reinterpret_cast<u32x4*>(lds + wbase + buf * BUF + j * 4096 + (d >> 1) * 1024 + (d & 1) * 512) =
             u32x4{tout[t][0], tout[t][1], tout[t][2], tout[t][3]};
     };
     const uint32_t rbase = kTabBytes + wn * (FN * 4096u) + lane * 16u;
-    auto read_frags = [&](int kk, int buf, int set) {
-#pragma unroll
-        for (int j = 0; j < FN; ++j) fb[set][j] = *reinterpret_cast<const u32x4*>(lds + rbase + buf * BUF + j * 4096 + kk * 1024);
+    auto read_frag1 = [&](int kk, int buf, int j) {
+        fb[j] = *reinterpret_cast<const u32x4*>(lds + rbase + buf * BUF + j * 4096 + kk * 1024);
     };
     f32x16 acc[FM][FN];
 #pragma unroll
@@ -240,53 +257,61 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
         for (int j = 0; j < FN; ++j)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.0f;
-    auto mfma1 = [&](int kk, int i, int j) {
-        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&fa[kk][i]),
-                                                            *reinterpret_cast<const bf16x8*>(&fb[kk & 1][j]), acc[i][j], 0, 0, 0);
+    auto mfma1 = [&](int as, int kk, int i, int j) {
+        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(*reinterpret_cast<const bf16x8*>(&fa[as][kk][i]),
+                                                            *reinterpret_cast<const bf16x8*>(&fb[j]), acc[i][j], 0, 0, 0);
     };
 
-    // One group: the FM * FN matrix instructions of column group kk of step s, and behind them, in fixed places
-    // (nothing moves across a matrix instruction): at the start the table reads of quarter QC (addresses formed in
-    // the group before) and the fragment reads RK of buffer rbuf into set RK & 1; behind the last use of each A
-    // fragment its reload for the next step; the table addresses of the next quarter (QN, weights in slot nslot);
-    // scale, round and store of quarter QC into buffer wbuf.
-    auto group = [&](auto kkc, auto qc, auto qn, int rk, int rbuf, int wbuf, int nslot, const float (&sc)[NBW], uint32_t gnext) {
-        constexpr int kk = decltype(kkc)::value;
+    // One group: the FM * FN matrix instructions of column group kk of a step (B fragment outermost, so that a
+    // fragment's registers are free for the next group's after FM instructions) and, in fixed places between them
+    // (nothing moves across a matrix instruction): scale, round and store of quarter q0 (table entries of set
+    // kk & 1) into buffer wbuf; the table reads of the quarter after it; the table addresses of quarter q2 of the
+    // weights in slot s2 (each written after the read that used its register); the fragment reads of column group rk
+    // of buffer rbuf; after the last instruction the A fragments of the step after next.
+    // A wavefront alone on its SIMD issues one instruction per four clocks, and a 32x32x16 matrix instruction
+    // holds the issue port for 16 of its 32: four other instructions ride for free behind each, a fifth delays
+    // the next one.  The places below keep the gaps at four or fewer (five behind the last).  Table entries and A
+    // fragments are consumed youngest first, so that one wait covers all of them.
+    auto group = [&](auto kkc, int as, int q0, int wbuf, const float (&sc)[NBW], int q2, int s2, int rk, int rbuf, uint32_t abase) {
+        constexpr int kk = decltype(kkc)::value, cs = kk & 1, ns = cs ^ 1;
         constexpr int NM = FM * FN, NU = NBW * 4;            // matrix instructions, decode units (bytes per lane) of the group
-        // places: addresses behind instructions A0 .. A0 + NU/PA - 1, math from M0 on
-        constexpr int PA = NM >= 16 ? 2 : 4;                 // addresses per place
-        constexpr int A0 = NM >= 16 ? 1 : 0;
-        constexpr int M0 = NM >= 16 ? 6 : 1;
-        constexpr int PM = NM >= 16 ? 1 : 2;                 // math units per place
-#pragma unroll
-        for (int t = 0; t < NBW; ++t)
-#pragma unroll
-            for (int b = 0; b < 4; ++b) q_read(t, b);
-        read_frags(rk, rbuf, rk & 1);
-        __builtin_amdgcn_sched_barrier(0);
+        // place of math unit k (k-th in processing order) together with the table read of unit k
+        auto mslot = [](int k) { return NM == 16 ? k + k / 4 : NM == 8 ? k : k / 2; };
+        // place of the two (NM == 4: four) table addresses from u on: behind the read that used the register
+        auto pslot = [](int u) { return NM == 16 ? (u < 2 ? 4 : 8 + u / 2) : NM == 8 ? 4 + u / 2 : 3; };
 #pragma unroll
         for (int n = 0; n < NM; ++n) {
-            const int i = n / FN, j = n % FN;
-            mfma1(kk, i, j);
-            if (j == FN - 1) load_a1(kk, i, gnext);
-            if (n >= A0 && (n - A0) * PA < NU) {
+            const int j = n / FM, i = FM - 1 - n % FM;           // A fragment FM - 1 (the youngest load) first
+            mfma1(as, kk, i, j);
 #pragma unroll
-                for (int a = 0; a < PA; ++a) { const int un = (n - A0) * PA + a; q_addr(qn, nslot, un >> 2, un & 3); }
+            for (int k = 0; k < NU; ++k) {
+                if (mslot(k) != n) continue;
+                const int un = NU - 1 - k;                       // youngest table entry first
+                q_mul(cs, un >> 2, un & 3, sc[(q0 * NBW + (un >> 2)) >> 2]);
+                q_read(ns, k >> 2, k & 3);
             }
-            if (n >= M0 && (n - M0) * PM < NU) {
 #pragma unroll
-                for (int a = 0; a < PM; ++a) {
-                    const int un = (n - M0) * PM + a;
-                    q_math(un >> 2, un & 3, sc[(decltype(qc)::value * NBW + (un >> 2)) >> 2]);
-                    if ((un & 3) == 3) q_store(qc, un >> 2, wbuf);
-                }
+            for (int k = 0; k < NU; ++k)                         // rounding of the unit whose products sit one place back
+                if (mslot(k) + 1 == n) { const int un = NU - 1 - k; q_round(un >> 2, un & 3); }
+#pragma unroll
+            for (int t = 0; t < NBW; ++t)                        // piece t is complete behind the rounding of its unit 4 t
+                if (mslot(NU - 1 - 4 * t) + 1 == n) q_store(q0, t, wbuf);
+            if (n % FM == FM - 1 && (NM != 16 || n != 3 && n != 7)) read_frag1(rk, rbuf, j);
+            if (NM == 16 && (n == 4 || n == 9)) read_frag1(rk, rbuf, n == 4 ? 0 : 1);
+#pragma unroll
+            for (int u = 0; u < NU; ++u)
+                if (pslot(u) == n) q_addr(q2, s2, u >> 2, u & 3);
+            if (n == NM - 1) {
+#pragma unroll
+                for (int ii = 0; ii < FM; ++ii) load_a1(as, kk, ii, abase);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
     };
 
-    // ---- prologue: loads of the first steps, tile kbeg whole and the table addresses of the first quarter of tile kbeg + 1
-    load_w(1, kbeg + 1u);
+    // ---- prologue: loads of the first steps; tile kbeg whole and the first quarter of tile kbeg + 1 decoded, the
+    // second quarter's table entries read and the third's addresses formed
+    load_w(1, kbeg + 1u);                                 // (a part is at least one block: four steps)
     load_w(2, kbeg + 2u);
     load_w(3, kbeg + 3u);
     load_w(0, kbeg);
@@ -295,70 +320,64 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
 #pragma unroll
     for (int j = 0; j < NBW; ++j) {
         scraw0[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], (kbeg >> 2) * 128u, 0);
-        scraw1[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], ((kbeg >> 2) + 1u) * 128u, 0);
+        scraw1[j] = __builtin_amdgcn_raw_buffer_load_b16(wrs, woff[j], ((kbeg >> 2) + 1u < bpr ? (kbeg >> 2) + 1u : bpr - 1u) * 128u, 0);
     }
 #pragma unroll
-    for (int kk = 0; kk < 3; ++kk)
+    for (int d = 0; d < AD; ++d)
 #pragma unroll
-        for (int i = 0; i < FM; ++i) load_a1(kk, i, kbeg * 4u + (uint32_t)kk);
+        for (int kk = 0; kk < (d == AD - 1 ? 3 : 4); ++kk)
+#pragma unroll
+            for (int i = 0; i < FM; ++i) load_a1(d, kk, i, (kbeg + d < klast ? kbeg + d : klast) * 4096u);
 #pragma unroll
     for (int j = 0; j < NBW; ++j) {
         scA[j] = __half2float(__ushort_as_half((unsigned short)scraw0[j]));
         scB[j] = __half2float(__ushort_as_half((unsigned short)scraw1[j]));
     }
     __syncthreads();                                   // table complete
-    {
-        auto whole = [&](auto qc) {
+    auto whole = [&](int q, int slot, int buf) {
 #pragma unroll
-            for (int t = 0; t < NBW; ++t) {
+        for (int t = 0; t < NBW; ++t) {
 #pragma unroll
-                for (int b = 0; b < 4; ++b) { q_addr(qc, 0, t, b); q_read(t, b); }
+            for (int b = 0; b < 4; ++b) { q_addr(q, slot, t, b); q_read(0, t, b); }
 #pragma unroll
-                for (int b = 0; b < 4; ++b) q_math(t, b, scA[(decltype(qc)::value * NBW + t) >> 2]);
-                q_store(qc, t, 0);
-            }
-        };
-        whole(IC<0>{}); whole(IC<1>{}); whole(IC<2>{}); whole(IC<3>{});
-    }
+            for (int b = 0; b < 4; ++b) q_math(0, t, b, scA[(q * NBW + t) >> 2]);
+            q_store(q, t, buf);
+        }
+    };
+    whole(0, 0, 0); whole(1, 0, 0); whole(2, 0, 0); whole(3, 0, 0);
+    whole(0, 1, 1);                                    // nobody reads buffer 1 yet
 #pragma unroll
     for (int t = 0; t < NBW; ++t)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) q_addr(IC<0>{}, 1, t, b);
-    load_w(0, kbeg + 4u);
+        for (int b = 0; b < 4; ++b) { q_addr(1, 1, t, b); q_read(0, t, b); q_addr(2, 1, t, b); }
+    load_w(0, kbeg + 4u < klast ? kbeg + 4u : klast);
 #pragma unroll
-    for (int i = 0; i < FM; ++i) load_a1(3, i, kbeg * 4u + 3u);
+    for (int i = 0; i < FM; ++i) load_a1(AD - 1, 3, i, (kbeg + AD - 1u < klast ? kbeg + AD - 1u : klast) * 4096u);
     __syncthreads();
-    read_frags(0, 0, 0);
-    // the first quarter of tile kbeg + 1 goes to buffer 1 ahead of the loop (nobody reads that buffer yet)
 #pragma unroll
-    for (int t = 0; t < NBW; ++t) {
-#pragma unroll
-        for (int b = 0; b < 4; ++b) q_read(t, b);
-#pragma unroll
-        for (int b = 0; b < 4; ++b) q_math(t, b, scA[t >> 2]);
-        q_store(IC<0>{}, t, 1);
-    }
-#pragma unroll
-    for (int t = 0; t < NBW; ++t)
-#pragma unroll
-        for (int b = 0; b < 4; ++b) q_addr(IC<1>{}, 1, t, b);
+    for (int j = 0; j < FN; ++j) read_frag1(0, 0, j);
 
     // ---- main loop: one 256-column block (four steps) per trip.  In step s (u = s & 3, tile s in buffer u & 1) the
-    // groups 0..2 read the fragments of column groups 1..3 and decode the quarters 1..3 of tile s + 1 into the other
-    // buffer; after the barrier group 3 reads the first fragments of tile s + 1 and decodes the first quarter of
+    // groups 0..2 read the fragments of column groups 1..3 and finish the quarters 1..3 of tile s + 1 into the other
+    // buffer; after the barrier group 3 reads the first fragments of tile s + 1 and finishes the first quarter of
     // tile s + 2 into the buffer that tile s has just left.  Tile s + 1 belongs to the next block from u = 3 on,
-    // tile s + 2 from u = 2 on.  The weights of tile s + 5 replace those of tile s + 1 when its last quarter is read.
+    // tile s + 2 from u = 2 on.  The weights of tile s + 5 replace those of tile s + 1 once its last table addresses
+    // are formed (group 0).
     auto step = [&](auto uc, uint32_t s) {
-        constexpr int u = decltype(uc)::value, cur = u & 1, nxt = cur ^ 1;
+        constexpr int u = decltype(uc)::value, cur = u & 1, nxt = cur ^ 1, s1 = (u + 1) & 3, s2 = (u + 2) & 3;
         const float (&sc1)[NBW] = u == 3 ? scB : scA;
         const float (&sc2)[NBW] = u >= 2 ? scB : scA;
-        group(IC<0>{}, IC<1>{}, IC<2>{}, 1, cur, nxt, (u + 1) & 3, sc1, s * 4u + 4u);
-        group(IC<1>{}, IC<2>{}, IC<3>{}, 2, cur, nxt, (u + 1) & 3, sc1, s * 4u + 5u);
-        group(IC<2>{}, IC<3>{}, IC<0>{}, 3, cur, nxt, (u + 2) & 3, sc1, s * 4u + 6u);
-        load_w((u + 1) & 3, s + 5u);
-        if constexpr (u == 0) load_scale((s >> 2) + 2u);
+        // steps past the end of the row are loaded and never used; the scalar offsets are outside the buffer range
+        // check, so they are clamped to the row's last step / block
+        const uint32_t an = (s + AD < klast ? s + AD : klast) * 4096u;
+        constexpr int as = u % AD;
+        group(IC<0>{}, as, 1, nxt, sc1, 3, s1, 1, cur, an);
+        group(IC<1>{}, as, 2, nxt, sc1, 0, s2, 2, cur, an);
+        group(IC<2>{}, as, 3, nxt, sc1, 1, s2, 3, cur, an);
+        load_w(s1, s + 5u < klast ? s + 5u : klast);
+        if constexpr (u == 0) load_scale((s >> 2) + 2u < bpr - 1u ? (s >> 2) + 2u : bpr - 1u);
         __syncthreads();
-        group(IC<3>{}, IC<0>{}, IC<1>{}, 0, nxt, cur, (u + 2) & 3, sc2, s * 4u + 7u);
+        group(IC<3>{}, as, 0, cur, sc2, 2, s2, 0, nxt, an);
     };
     for (uint32_t s = kbeg; s < kend; s += 4u) {
         step(IC<0>{}, s);

@@ -65,6 +65,7 @@ __device__ __forceinline__ float level_literal(uint32_t i) {
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef __attribute__((address_space(3))) const f32x2 lds_cfloat2;
 typedef __attribute__((address_space(3))) const float lds_cfloat;
+typedef __attribute__((address_space(3))) const uint32_t lds_cuint;
 
 // Pair table, 64 KB at LDS offset 0: entry of byte value v and lane copy c at
 // byte v*256 + c*8 = (level[v & 15], level[v >> 4]).  32 lane-private copies:
