@@ -196,6 +196,19 @@ int oilhip_set_ordered_sums(int ordered);
  * the channel sizes the quantizer writes (OILHIP_E_ARG otherwise). */
 int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x_bf16, float* d_y, int M, void* stream);
 
+/* The same prefill GEMM for the reference's own call: FP32 activations X[M][cols], as Qwen35Engine::prefill hands
+ * them to gemm() in chunks of up to 512 tokens (src/adapters/tools/qwen35_engine.cpp:47-85,630-753).  X is rounded
+ * once to bf16 on its way into the kernel's operand order (no extra pass for plain OIL4 and M > 256; otherwise
+ * one conversion launch into a scratch buffer of the stream), so the result carries the bf16 tolerance (relative L2
+ * <= 2e-3 against the FP32 contraction) instead of oilhip_gemv_f32's 1e-5: a caller chooses it per call. */
+int oilhip_gemm_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream);
+
+/* Frees the scratch buffers the library holds for `stream` on the current device (packed activations of the
+ * multi-token GEMV, X' and decoded slabs of the prefill GEMM, the lookup kernels' codes): after a stream is destroyed, or
+ * to trim after a large batch.  Synchronizes the stream first; no captured graph may still replay launches that were
+ * recorded on it.  (No counterpart in the reference, which owns no device memory.) */
+int oilhip_release_stream_scratch(void* stream);
+
 /* ---------------------------------------------------- flat-codebook kernels
  * oil::kernel::oil8_gemm (include/oil/kernel.h:24-26, src/kernel_oil8.cpp:71-79):
  *   out[m*N+n] = sum_k cb[idx[n*K+k]] * act[m*K+k]

@@ -105,6 +105,14 @@ struct BlockRef {
 // A tensor of .oil blocks resident in HBM: what Qwen35Engine::Th + OILReader give the
 // reference's gemm (include/oil/qwen35_engine.h:29,38).  gemm() is that function:
 // Y[b*rows + r] = sum_c W[r][c] * X[b*cols + c], host pointers, FP32, any B >= 1.
+// Batches of at least `min_batch` activation rows go through the bf16 matrix-core prefill kernel (oilhip_gemm_f32:
+// X rounded once to bf16, relative L2 error <= 2e-3 against the FP32 contraction) instead of the FP32 decode kernels
+// (<= 1e-5).  0 (the default) keeps every batch on the FP32 path, as the reference computes it; 32 or more is where
+// the prefill kernel is faster.  Process-wide; Qwen35Engine::prefill calls gemm with up to 512 rows
+// (src/adapters/tools/qwen35_engine.cpp:12,630-753).
+void set_prefill_min_batch(int min_batch);
+int prefill_min_batch();
+
 class DeviceTensor {
 public:
     DeviceTensor(const std::vector<BlockRef>& blocks, uint64_t rows, uint64_t cols);
@@ -114,7 +122,7 @@ public:
     ~DeviceTensor();
     DeviceTensor(const DeviceTensor&) = delete;
     DeviceTensor& operator=(const DeviceTensor&) = delete;
-    void gemm(const float* X, float* Y, int B) const;
+    void gemm(const float* X, float* Y, int B) const;       // Y[B][rows] = X[B][cols] . W^T (Qwen35Engine::gemm); see set_prefill_min_batch
     void dequantize(float* out) const;                    // rows*cols floats, bit-exact with dequantize_block_all
     uint64_t rows() const { return rows_; }
     uint64_t cols() const { return cols_; }

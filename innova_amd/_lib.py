@@ -75,6 +75,8 @@ _SIGNATURES = {
     "oilhip_gemv_oil4_f32_noalloc": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_set_ordered_sums": (C.c_int, [C.c_int]),
     "oilhip_gemm_bf16": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_gemm_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
+    "oilhip_release_stream_scratch": (C.c_int, [vp]),
     "oilhip_profile_gemv": (C.c_int, [C.c_int, vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp]),
     "oilhip_read_probe": (C.c_int, [vp, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp]),
     "oilhip_tl_gemm": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),

@@ -46,7 +46,7 @@ int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes);
 // one and the old one stays allocated.  No allocation can happen while the stream is being captured, so the first
 // call of a given size on a stream has to be made outside capture; otherwise the call fails with OILHIP_E_ARG.
 // New buffers are zero-filled.
-enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1, kScratchTl = 2, kScratchGemmW = 3 };
+enum ScratchSlot { kScratchGemvPack = 0, kScratchGemmX = 1, kScratchTl = 2, kScratchGemmW = 3, kScratchGemmXb = 4 };
 int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out);
 
 // Tensors whose rows mix formats are stored as `nstreams` streams of windows of at most 4 KB, one wavefront per stream
@@ -140,6 +140,8 @@ int launch_gemv_seg(const oilhip_weights& w, const float* d_x, float* d_y, int M
 int launch_gemv_runs(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_oil4_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
 int launch_gemm_any_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_y, int M, hipStream_t s);
+// FP32 activations [M][K] rounded once to bf16 bit patterns (a scratch buffer of the stream)
+int launch_x_to_bf16(const float* d_x, uint64_t n, uint16_t** out, hipStream_t s);
 // plain uniform OIL4, more than 256 tokens: activations in fragment order straight from memory (gemm_oil4_frag.hip)
 int launch_gemm_oil4_frag(const oilhip_weights& w, const void* d_x, bool x_is_f32, float* d_y, int M, hipStream_t s);
 }  // namespace oilhip

@@ -504,6 +504,24 @@ int launch_pipe(const uint8_t* wmat, const uint16_t* x, float* d_y, uint32_t M, 
 
 }  // namespace
 
+// FP32 -> bf16 (round to nearest even), four values per thread
+__global__ void __launch_bounds__(256) x_to_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ o, uint64_t n) {
+    for (uint64_t i = ((uint64_t)blockIdx.x * 256u + threadIdx.x) * 4u; i < n; i += (uint64_t)gridDim.x * 1024u) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k)
+            if (i + k < n) { const __bf16 b = (__bf16)x[i + k]; o[i + k] = *reinterpret_cast<const uint16_t*>(&b); }
+    }
+}
+
+int launch_x_to_bf16(const float* d_x, uint64_t n, uint16_t** out, hipStream_t s) {
+    uint16_t* xb = nullptr;
+    if (int rc = stream_scratch(s, kScratchGemmXb, (size_t)n * 2, reinterpret_cast<void**>(&xb))) return rc;
+    hipLaunchKernelGGL(x_to_bf16_kernel, dim3((uint32_t)std::min<uint64_t>((n + 1023) / 1024, 8192)), dim3(256), 0, s, d_x, xb, n);
+    OILHIP_HIP(hipGetLastError());
+    *out = xb;
+    return OILHIP_OK;
+}
+
 // Prefill over a tensor of any format (full 256-weight blocks): slabs of weight rows are decoded to bf16 in a scratch
 // buffer of the stream (dequantize_block_all's values, each rounded once to bf16) and multiplied by the same pipelined
 // kernel reading a dense operand.  Returns 1 when the tensor's layout is not covered.

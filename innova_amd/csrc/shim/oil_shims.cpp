@@ -1,6 +1,7 @@
 // oil_shims.cpp -- host-pointer C++ shims over the C ABI (see include/oilhip_shims.hpp).
 #include "../../../include/oilhip_shims.hpp"
 
+#include <atomic>
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -246,10 +247,16 @@ DeviceTensor::DeviceTensor(const uint8_t* records, uint64_t record_bytes, const 
 
 DeviceTensor::~DeviceTensor() { oilhip_weights_destroy(static_cast<oilhip_weights*>(handle_)); }
 
+static std::atomic<int> g_prefill_min_batch{0};
+void set_prefill_min_batch(int min_batch) { g_prefill_min_batch.store(min_batch < 0 ? 0 : min_batch, std::memory_order_relaxed); }
+int prefill_min_batch() { return g_prefill_min_batch.load(std::memory_order_relaxed); }
+
 void DeviceTensor::gemm(const float* X, float* Y, int B) const {
     if (B <= 0) return;
     Dev<float> x(X, (size_t)B * cols_), y(nullptr, (size_t)B * rows_);
-    ok(oilhip_gemv_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm");
+    const int pmin = prefill_min_batch();
+    if (pmin > 0 && B >= pmin) ok(oilhip_gemm_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm (prefill)");
+    else ok(oilhip_gemv_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm");
     y.to_host(Y);
 }
 

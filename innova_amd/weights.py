@@ -125,3 +125,11 @@ class DeviceWeights:
         x2, M, out = self._xy(x, torch.bfloat16, out)
         _lib.check(_lib.lib().oilhip_gemm_bf16(self.handle, x2.data_ptr(), out.data_ptr(), M, _lib.current_stream()))
         return out
+
+    def gemm_f32(self, x, out=None):
+        """The prefill GEMM for FP32 activations (the reference's own gemm() arguments, qwen35_engine.cpp:47-85):
+        X is rounded once to bf16 inside the kernel's pre-pass; bf16 tolerance (rel-L2 <= 2e-3)."""
+        import torch
+        x2, M, out = self._xy(x, torch.float32, out)
+        _lib.check(_lib.lib().oilhip_gemm_f32(self.handle, x2.data_ptr(), out.data_ptr(), M, _lib.current_stream()))
+        return out

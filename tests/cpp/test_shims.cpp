@@ -139,6 +139,51 @@ int main() {
         try { gfx950::DeviceTensor bad(refs, rows + 1, cols); } catch (const oil::Error&) { threw = true; }
         CHECK(threw, "shape mismatch must throw oil::Error");
     }
+    {   // DeviceTensor::gemm at the reference's prefill batch (MAX_BATCH = 512, src/adapters/tools/qwen35_engine.cpp:12,
+        // 630-753) on the Llama-7B up projection: with the prefill threshold set, B = 512 runs on the bf16 matrix-core
+        // kernel (<= 2e-3), B = 8 stays on the FP32 decode kernels (<= 1e-5).  Yardstick: double dot of the tensor's
+        // own decode over a sample of weight rows.
+        const int rows = 11008, cols = 4096, bpr = cols / 256;
+        std::vector<float> W((size_t)rows * cols);
+        for (auto& v : W) v = frand() * 0.04f;
+        std::vector<std::vector<uint8_t>> idxs((size_t)rows * bpr), cbs((size_t)rows * bpr);
+        std::vector<gfx950::BlockRef> refs;
+        refs.reserve(idxs.size());
+        for (size_t b = 0; b < idxs.size(); ++b) {
+            quantize_block_all(Format::OIL4, W.data() + b * 256, 256, idxs[b], cbs[b]);
+            refs.push_back({Format::OIL4, cbs[b].data(), (uint32_t)cbs[b].size(), idxs[b].data(), (uint32_t)idxs[b].size(), 256});
+        }
+        gfx950::DeviceTensor t(refs, rows, cols);
+        t.dequantize(W.data());                                  // W is now the decoded tensor
+        std::vector<int> sel;
+        for (int r = 0; r < rows; r += 257) sel.push_back(r);
+        sel.push_back(rows - 1);
+        auto check = [&](int B, double tol, const char* what) {
+            std::vector<float> X((size_t)B * cols), Y((size_t)B * rows), got;
+            for (auto& v : X) v = frand() * 1.7f;
+            t.gemm(X.data(), Y.data(), B);
+            std::vector<double> want;
+            for (int b = 0; b < B; ++b)
+                for (int r : sel) {
+                    double a = 0;
+                    for (int c = 0; c < cols; ++c) a += (double)W[(size_t)r * cols + c] * X[(size_t)b * cols + c];
+                    want.push_back(a);
+                    got.push_back(Y[(size_t)b * rows + r]);
+                }
+            bool finite = true; for (float v : Y) finite &= std::isfinite(v);
+            CHECK(finite, "%s: non-finite output", what);
+            CHECK(rel_l2(got, want) <= tol, "%s: rel-L2 %.3g > %.1g", what, rel_l2(got, want), tol);
+            return rel_l2(got, want);
+        };
+        CHECK(gfx950::prefill_min_batch() == 0, "prefill threshold must default to off");
+        const double e0 = check(512, 1e-5, "gemm B=512, FP32 path");
+        gfx950::set_prefill_min_batch(32);
+        const double e1 = check(512, 2e-3, "gemm B=512, prefill path");
+        const double e2 = check(8, 1e-5, "gemm B=8 below the prefill threshold");
+        CHECK(e1 > 1e-5, "B=512 with the threshold set should have run on the bf16 kernel (rel-L2 %.3g)", e1);
+        std::printf("DeviceTensor::gemm 11008x4096: B=512 fp32 %.2g, B=512 prefill %.2g, B=8 %.2g\n", e0, e1, e2);
+        gfx950::set_prefill_min_batch(0);
+    }
     {   // OIL4KVCache: prefill + two decode appends; ranges are slices of the whole, the static pair round-trips
         // through the cache's own centroids, appends past max_seq_len are dropped but counted
         const int heads = 4, dim = 64, pt = heads * dim, n = 9;
