@@ -106,8 +106,8 @@ struct BlockRef {
 // reference's gemm (include/oil/qwen35_engine.h:29,38).  gemm() is that function:
 // Y[b*rows + r] = sum_c W[r][c] * X[b*cols + c], host pointers, FP32, any B >= 1.
 // Batches of at least `min_batch` activation rows go through the bf16 matrix-core prefill kernel (oilhip_gemm_f32:
-// X rounded once to bf16, relative L2 error <= 2e-3 against the FP32 contraction) instead of the FP32 decode kernels
-// (<= 1e-5).  0 (the default) keeps every batch on the FP32 path, as the reference computes it; 32 or more is where
+// X rounded once to bf16: relative L2 error <= 2e-3 against the FP32 contraction over the rounded activations, about
+// 2.4e-3 against the one over the FP32 activations for Gaussian data) instead of the FP32 decode kernels (<= 1e-5).  0 (the default) keeps every batch on the FP32 path, as the reference computes it; 32 or more is where
 // the prefill kernel is faster.  Process-wide; Qwen35Engine::prefill calls gemm with up to 512 rows
 // (src/adapters/tools/qwen35_engine.cpp:12,630-753).
 void set_prefill_min_batch(int min_batch);

@@ -1,6 +1,8 @@
 // test_reference_tree.cpp -- the reference-tree drop-ins at work, on a GPU: the patched backend dispatch
 // (ComputeBackend::create / probe_hardware / select_optimal_backend reaching the gfx950 backend object), the engine
 // classes' members and tl1_gemm / tl2_gemm defined by innova_amd/csrc/shim/oil_{backend,engines}_gfx950.cpp.
+// The patched Qwen35Engine (include/qwen35_engine_gfx950.patch): gemm straight from a .oil file's records on the
+// device against the same class's CPU loop.
 // Built by oracle/Makefile against the reference's headers and its compiled tensor / math sources; the CPU side of
 // every comparison is the reference's own math:: routine or a loop written out here.
 #include <cmath>
@@ -15,6 +17,11 @@
 #include "oil/kernel_production.h"
 #include "oil/math.h"
 #include "oil/oil_engines.h"
+#define private public                       // the test calls Qwen35Engine::resolve / gemm directly
+#include "oil/qwen35_engine.h"
+#undef private
+#include "oilhip.h"
+#include "oilhip_shims.hpp"
 
 using namespace oil;
 
@@ -242,6 +249,83 @@ static void test_profile() {
     CHECK(same_bits(y.data(), y2.data(), M), "profile_gemv_oil4 leaves the GEMV's result in y");
 }
 
+// Qwen35Engine::gemm (src/adapters/tools/qwen35_engine.cpp:47-85) through the patch: a small .oil file written by
+// oilhip_file_write (a uniform OIL4 tensor and one whose blocks alternate between three formats), opened by the
+// reference's OILReader, resolved by the engine's own resolve(); the device path against the engine's own CPU loop at
+// B = 1, 16 and 512, FP32 path (<= 1e-5) and, for B = 512, the bf16 prefill path (<= 2e-3).
+static void test_qwen35_engine() {
+    const uint32_t rows = 384, cols = 1024, bpr = cols / 256, nb = rows * bpr;
+    std::vector<float> w((size_t)2 * rows * cols);
+    std::normal_distribution<float> d(0.f, 0.02f);
+    for (auto& v : w) v = d(g_rng);
+    std::vector<uint8_t> fmts(2 * nb);
+    for (uint32_t b = 0; b < nb; ++b) fmts[b] = OILHIP_OIL4;
+    for (uint32_t b = 0; b < nb; ++b) fmts[nb + b] = b % 3 == 0 ? OILHIP_OIL4 : b % 3 == 1 ? OILHIP_OIL8_GRP : OILHIP_SPARK_Q0;
+    uint64_t cap = 0, total = 0;
+    CHECK(oilhip_quantize_tensor(fmts.data(), 2 * nb, w.data(), w.size(), nullptr, 0, nullptr, &cap, 0) == 0, "payload bound");
+    std::vector<uint8_t> payload(cap);
+    std::vector<oilhip_block_t> blocks(2 * nb);
+    CHECK(oilhip_quantize_tensor(fmts.data(), 2 * nb, w.data(), w.size(), payload.data(), cap, blocks.data(), &total, 0) == 0,
+          "quantize: %s", oilhip_last_error());
+    const char* path = "/tmp/oilhip_qwen35_engine_test.oil";
+    const char* names[2] = {"layer.up_proj.weight", "layer.mixed_proj.weight"};
+    const uint32_t counts[2] = {nb, nb};
+    const uint8_t config[4] = {1, 2, 3, 4};
+    CHECK(oilhip_file_write(path, 1, 0, config, 4, 2, names, counts, payload.data(), blocks.data(), 2 * nb) == 0,
+          "file_write: %s", oilhip_last_error());
+
+    Qwen35Engine eng;
+    CHECK(eng.gfx950_, "the patched engine did not find the device");
+    eng.reader_ = new OILReader(path);
+    CHECK(eng.reader_->valid(), "the reference's reader rejects the file");
+    for (int t = 0; t < 2; ++t) {
+        CHECK(eng.resolve(names[t], rows, cols), "resolve %s", names[t]);
+        const Qwen35Engine::Th* th = eng.th(names[t]);
+        CHECK(th && th->count == nb, "block range of %s", names[t]);
+        if (!th) continue;
+        for (int B : {1, 16, 512}) {
+            std::vector<float> X((size_t)B * cols), Yd((size_t)B * rows), Yc((size_t)B * rows), Yp((size_t)B * rows);
+            std::normal_distribution<float> dx(0.f, 1.0f);
+            for (auto& v : X) v = dx(g_rng);
+            eng.gfx950_ = false;
+            eng.gemm(*th, X.data(), Yc.data(), B);                 // the reference's loop
+            eng.gfx950_ = true;
+            gfx950::set_prefill_min_batch(0);
+            eng.gemm(*th, X.data(), Yd.data(), B);                 // device, FP32 path
+            double num = 0, den = 0;
+            for (size_t i = 0; i < Yc.size(); ++i) { num += ((double)Yd[i] - Yc[i]) * ((double)Yd[i] - Yc[i]); den += (double)Yc[i] * Yc[i]; }
+            CHECK(std::sqrt(num / den) <= 1e-5, "Qwen35Engine::gemm %s B=%d: rel-L2 %.3g", names[t], B, std::sqrt(num / den));
+            if (B == 512) {
+                // The prefill kernel rounds X once to bf16: against the reference's loop over the same rounded
+                // activations (what "bf16 activations" means) only the rounding of the weights is left (<= 2e-3);
+                // against the loop over the FP32 activations both roundings show (<= 3e-3 for Gaussian data).
+                std::vector<float> Xr(X.size()), Ycr(Yc.size());
+                for (size_t i = 0; i < X.size(); ++i) {
+                    uint32_t u; std::memcpy(&u, &X[i], 4);
+                    u = (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+                    std::memcpy(&Xr[i], &u, 4);
+                }
+                eng.gfx950_ = false;
+                eng.gemm(*th, Xr.data(), Ycr.data(), B);
+                eng.gfx950_ = true;
+                gfx950::set_prefill_min_batch(32);
+                eng.gemm(*th, X.data(), Yp.data(), B);             // device, bf16 prefill path
+                gfx950::set_prefill_min_batch(0);
+                double nr = 0, nf = 0, dr = 0;
+                for (size_t i = 0; i < Yc.size(); ++i) {
+                    nr += ((double)Yp[i] - Ycr[i]) * ((double)Yp[i] - Ycr[i]); dr += (double)Ycr[i] * Ycr[i];
+                    nf += ((double)Yp[i] - Yc[i]) * ((double)Yp[i] - Yc[i]);
+                }
+                const double er = std::sqrt(nr / dr), ef = std::sqrt(nf / den);
+                CHECK(er <= 2e-3 && er > 1e-5, "Qwen35Engine::gemm %s B=512 prefill: rel-L2 %.3g against the loop over bf16(X)", names[t], er);
+                CHECK(ef <= 3e-3, "Qwen35Engine::gemm %s B=512 prefill: rel-L2 %.3g against the loop over FP32 X", names[t], ef);
+            }
+        }
+    }
+    CHECK(eng.dev_.size() == 2, "one device tensor per resolved tensor, got %zu", eng.dev_.size());
+    std::remove(path);
+}
+
 int main() {
     std::printf("backend\n"); std::fflush(stdout);
     test_backend();
@@ -255,6 +339,8 @@ int main() {
     test_tl();
     std::printf("profile\n"); std::fflush(stdout);
     test_profile();
+    std::printf("qwen35 engine\n"); std::fflush(stdout);
+    test_qwen35_engine();
     std::printf(g_fail ? "%d check(s) failed\n" : "all reference-tree checks passed\n", g_fail);
     return g_fail ? 1 : 0;
 }

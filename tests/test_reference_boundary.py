@@ -66,3 +66,29 @@ def test_reference_tree_sources_compile(patched_tree):
     assert r.returncode == 0, r.stderr[-4000:]
     text = open(patched_tree / "src" / "backend.cpp").read()
     assert "case BackendType::GPU_HIP_GFX950" in text and "hw.has_hip_gfx950" in text
+
+
+ENGINE_PATCH = os.path.join(ROOT, "include", "qwen35_engine_gfx950.patch")
+
+
+def test_engine_patch_applies_to_the_reference():
+    r = subprocess.run(["patch", "--dry-run", "-p1", "-d", REF, "-i", ENGINE_PATCH], capture_output=True, text=True)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert "include/oil/qwen35_engine.h" in r.stdout and "src/adapters/tools/qwen35_engine.cpp" in r.stdout
+
+
+def test_patched_engine_compiles_with_and_without_the_device_path(tmp_path):
+    """Qwen35Engine with the patch: the translation unit compiles against the reference's headers with the device
+    path switched on (gemm goes through gfx950::DeviceTensor) and, unchanged in meaning, with it switched off."""
+    os.makedirs(tmp_path / "include" / "oil")
+    os.makedirs(tmp_path / "src" / "adapters" / "tools")
+    shutil.copy(os.path.join(REF, "include", "oil", "qwen35_engine.h"), tmp_path / "include" / "oil")
+    shutil.copy(os.path.join(REF, "src", "adapters", "tools", "qwen35_engine.cpp"), tmp_path / "src" / "adapters" / "tools")
+    subprocess.run(["patch", "-s", "-p1", "-d", str(tmp_path), "-i", ENGINE_PATCH], check=True)
+    src = str(tmp_path / "src" / "adapters" / "tools" / "qwen35_engine.cpp")
+    inc = [f"-I{tmp_path}/include", f"-I{REF}/include", f"-I{ROOT}/include"]
+    for flags in (["-DOIL_USE_HIP_GFX950"], []):
+        r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-w"] + flags + inc + [src], capture_output=True, text=True)
+        assert r.returncode == 0, r.stderr[-4000:]
+    text = open(src).read()
+    assert "gfx950_gemm(t, X, Y, B)" in text and "decode_block(*reader_, bid, 256, sc)" in text   # both paths are there
