@@ -466,17 +466,26 @@ def bench_prefill(torch, ia, payload, blocks):
 
 
 def bench_read_probe(torch, ia):
-    """What a pure reader reaches on this device with the GEMVs' load pattern (oilhip_read_probe): (a) steady state, one
+    """What a pure reader reaches on this device with the GEMVs' load pattern (liboilhip_probe.so, a measurement tool
+    built beside the product library): (a) steady state, one
     launch over a 902 MB buffer, swept over waves per SIMD (2 / 4 / 8) and loads in flight (2 / 4 / 8), plain and
     non-temporal loads; (b) the headline's shape of work, 22.5 MB per launch as a graph of 40 dependent launches over
     40 different slices, which adds the launch gap and the ramp the GEMV pays too."""
-    L = ia._lib.lib()
+    import ctypes
+    path = os.path.join(os.path.dirname(ia._lib.LIB_PATH), "liboilhip_probe.so")
+    if not os.path.exists(path):
+        return {"read_only_probe": "liboilhip_probe.so not built"}
+    L = ctypes.CDLL(path)
+    L.oilprobe_read.restype = ctypes.c_int
+    L.oilprobe_read.argtypes = [ctypes.c_void_p, ctypes.c_uint64] + [ctypes.c_int] * 5 + [ctypes.c_void_p, ctypes.c_void_p]
+    L.oilprobe_last_error.restype = ctypes.c_char_p
     one, copies = 22544384, 40
     buf = torch.empty(one * copies, dtype=torch.uint8, device="cuda").fill_(1)
     sink = torch.zeros(1 << 16, dtype=torch.int32, device="cuda")
 
     def launch(ptr, nbytes, u, nt, pat, wgs, thr):
-        ia._lib.check(L.oilhip_read_probe(ptr, nbytes, u, nt, pat, wgs, thr, sink.data_ptr(), ia._lib.current_stream()))
+        if L.oilprobe_read(ptr, nbytes, u, nt, pat, wgs, thr, sink.data_ptr(), ia._lib.current_stream()) != 0:
+            raise RuntimeError(L.oilprobe_last_error().decode())
 
     out, table = {}, {}
     best = 0.0

@@ -294,16 +294,6 @@ int oilhip_dense_norm_f32(int kind, const float* d_x, const float* d_gamma, cons
 int oilhip_dense_softmax_f32(const float* d_x, float* d_y, int64_t outer, int64_t dim, int64_t inner, void* stream);
 int oilhip_dense_map_f32(int op, const float* d_a, const float* d_b, float s, float* d_y, int64_t n, void* stream);
 
-/* A read-only streaming kernel with the decode GEMVs' load pattern (16 bytes per lane, 1 KB per wavefront and load;
- * the data is only XOR-ed): what a pure reader reaches on this device, to put beside the HBM peak.  `bytes` are read
- * once by workgroups x threads / 64 wavefronts, each with `in_flight` (1, 2, 4, 8) loads outstanding; streaming != 0
- * marks the loads non-temporal; pattern 0 gives each wavefront a contiguous share, 1 interleaves them KB by KB,
- * 2 is the multi-token GEMV's pattern (512 threads, 4 or 8 loads in flight: a load fetches 64 bytes of each of 16
- * rows of 2 KB).
- * d_sink needs workgroups x threads / 64 words (practically never written).  No reference counterpart. */
-int oilhip_read_probe(const void* d_buf, uint64_t bytes, int in_flight, int streaming, int pattern,
-                      int workgroups, int threads, uint32_t* d_sink, void* stream);
-
 /* ------------------------------------------------------------ decode-step pieces
  * oilhip_weights_stack_rows : several uploaded tensors of one width (full 256-weight blocks only) as one tensor of
  *                             their rows in order; the parts stay valid.  Parts of one format and regular layout

@@ -78,7 +78,6 @@ _SIGNATURES = {
     "oilhip_gemm_f32": (C.c_int, [vp, vp, vp, C.c_int, vp]),
     "oilhip_release_stream_scratch": (C.c_int, [vp]),
     "oilhip_profile_gemv": (C.c_int, [C.c_int, vp, vp, C.c_float, vp, vp, C.c_int, C.c_int, C.c_int, vp, vp]),
-    "oilhip_read_probe": (C.c_int, [vp, C.c_uint64, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, vp, vp]),
     "oilhip_tl_gemm": (C.c_int, [C.c_int, vp, vp, vp, C.c_int, C.c_int, C.c_int, vp]),
     "oilhip_dense_gemm_f32": (C.c_int, [C.c_float, vp, vp, C.c_float, vp, C.c_int64, C.c_int64, C.c_int64, vp]),
     "oilhip_dense_gemv_f32": (C.c_int, [C.c_float, vp, vp, C.c_float, vp, C.c_int64, C.c_int64, vp]),

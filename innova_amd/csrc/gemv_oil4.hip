@@ -27,24 +27,6 @@
 #include "common.h"
 #include "oil4_lds.h"
 
-#ifndef OILHIP_PFA
-#define OILHIP_PFA 3
-#define OILHIP_PFB 6
-#define OILHIP_PFC 6
-#endif
-#ifndef OILHIP_OIL4_WGT
-#define OILHIP_OIL4_WGT 512      // threads per workgroup of the decode kernel (512 or 1024)
-#endif
-#ifndef OILHIP_OIL4_LA
-#define OILHIP_OIL4_LA 0         // 0: chosen by the workgroup size
-#endif
-#ifndef OILHIP_OIL4_SKIP
-#define OILHIP_OIL4_SKIP 0       // 1: single-chunk launches skip the products of row slots past the group's rows
-#endif
-#ifndef OILHIP_OIL4_AUX
-#define OILHIP_OIL4_AUX 2        // cache policy of the weight loads: 2 = nt (streamed once, not kept in L2 / the Infinity Cache)
-#endif
-
 namespace oilhip {
 namespace {
 
@@ -69,7 +51,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
                  uint32_t rg_base, uint32_t rg_rem, uint32_t wave_groups_lo, uint32_t wave_groups_hi, float out_scale) {
     constexpr uint32_t NW = WGT / 64;   // wavefronts per workgroup
     constexpr int NL = CS * RPW;      // wave-loads per chunk
-    constexpr int LA = OILHIP_OIL4_LA ? OILHIP_OIL4_LA : (WGT == 1024 ? 1 : 4);   // dwords of a wave-load decoded per pipeline step
+    constexpr int LA = 4;             // dwords of a wave-load decoded per pipeline step: two wavefronts per SIMD stage a whole wave-load
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                               // LDS byte offset 0
     const uint32_t nblk = S * CS * 8;                                         // blocks covered by all slabs (>= cols/256)
@@ -158,13 +140,13 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     // lines; queueing more only stalls the wavefront in front of its prologue), the first three while the table
     // is written so that the younger wavefronts get their first rows early too; the rest follow once the
     // prologue is done, while the first ones are being consumed.
-    constexpr int PFA = NL < OILHIP_PFA ? NL : OILHIP_PFA;          // queued while the table is written
-    constexpr int PFB = NL < OILHIP_PFB ? NL : OILHIP_PFB;          // ... by the time x is staged
-    constexpr int PFC = NL < OILHIP_PFC ? NL : OILHIP_PFC;          // ... by the barrier
+    constexpr int PFA = NL < 3 ? NL : 3;          // queued while the table is written
+    constexpr int PFB = NL < 6 ? NL : 6;          // ... by the time x is staged
+    constexpr int PFC = NL < 6 ? NL : 6;          // ... by the barrier
     u32x4 wv[NL];
     auto issue_load = [&](int n, uint32_t rel) {           // rel: first row of the chunk, counted from r0
         const int it = n / CS, cs = n % CS;
-        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, OILHIP_OIL4_AUX);
+        wv[n] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, vcol[cs] + (rel + it) * row_bytes, 0, 2);   // aux 2 = nt: streamed once, not kept in L2 / the Infinity Cache
     };
     // The 64 KB pair table is written while the weight loads queue up: float4 number e of the
     // table is (lo, hi, lo, hi) of byte value v = e >> 4, and thread tid writes e = tid + WGT*k,
@@ -298,14 +280,9 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
         }
         float part[MB][RPW];                              // per-lane partial of each row, block scales applied
         // A wave-load is consumed in units of LA dwords (4 LA packed bytes): the table reads of the next unit are in
-        // flight while the products of the current one are formed.  Four wavefronts per SIMD hide the table latency
-        // between them, so their units are one dword and the two staging arrays 16 registers; two wavefronts per SIMD
-        // stage a whole wave-load.
+        // flight while the products of the current one are formed; with two wavefronts per SIMD a unit is a whole
+        // wave-load.
         constexpr int UPL = 4 / LA, UB = 4 * LA;          // units per wave-load, packed bytes per unit
-        // rows of this chunk that exist (single-chunk launches skip the products of the row slots past them; with
-        // rolling loads the count of outstanding loads must not depend on it, so there every slot is worked)
-        constexpr bool SKIP = OILHIP_OIL4_SKIP && !ROLL;
-        const uint32_t nvalid = !SKIP ? (uint32_t)RPW : (r1 > cbase ? r1 - cbase : 0u);
         LevelPair cur[UB];
         auto lookup_unit = [&](int u, LevelPair (&t)[UB]) {
             const u32x4 w4 = wv[u / UPL];
@@ -323,11 +300,6 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
 #pragma unroll
         for (int n = 0; n < NL; ++n) {
             const int it = n / CS, cs = n % CS;
-            if (SKIP && (uint32_t)it >= nvalid) {                             // wave-uniform: this row slot is past the group's rows
-#pragma unroll
-                for (int m = 0; m < MB; ++m) if (cs == 0) part[m][it] = 0.0f;
-                continue;
-            }
             // The wavefronts of a SIMD are served oldest first; left alone the older one runs ahead and the
             // younger finishes its rows on its own.  Priority falls with progress, so whichever is behind goes first.
             if (!ROLL && (n == 0 || (n * 4) / NL != ((n - 1) * 4) / NL)) {
@@ -344,7 +316,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
             for (int q = 0; q < UPL; ++q) {
                 const int u = n * UPL + q;
                 LevelPair nxt[UB];
-                const bool more = u + 1 < NL * UPL && (!SKIP || q + 1 < UPL || (uint32_t)((n + 1) / CS) < nvalid);
+                const bool more = u + 1 < NL * UPL;
                 if (more) lookup_unit(u + 1, nxt);                    // next unit's table reads fly during these FMAs
                 __builtin_amdgcn_sched_barrier(0);                    // keep them above the FMAs
 #pragma unroll
@@ -425,7 +397,7 @@ gemv_oil4_kernel(const uint8_t* __restrict__ W, const float* __restrict__ x, con
     }
 }
 
-constexpr int kWgt = OILHIP_OIL4_WGT;
+constexpr int kWgt = 512;          // threads per workgroup of the decode kernel
 
 // One launch configuration of the kernel above.
 struct Oil4Plan {
@@ -455,8 +427,8 @@ int launch(const oilhip_weights& w, const float* d_x, const float* d_xw, float* 
 // Chooses column sets per wave, slabs, waves per workgroup and chunking for a shape.
 bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan* p) {
     const uint32_t sets = ((cols >> 8) + 7) / 8;                  // column sets (1 KB wave-loads) per row
-    // register budget: 32*CS*MB activations per lane, out of 256 registers (two wavefronts per SIMD) or 128 (four)
-    const int cs_max = MB == 1 ? (kWgt == 1024 ? 2 : 3) : 1;
+    // register budget: 32*CS*MB activations per lane, out of 256 registers (two wavefronts per SIMD)
+    const int cs_max = MB == 1 ? 3 : 1;
     // fewest slabs first (less cross-wave reduction), then least padding
     int best_cs = 1; uint32_t best_S = sets; double best_cost = 1e30;
     for (int cs = 1; cs <= cs_max; ++cs) {
@@ -475,7 +447,7 @@ bool make_plan(uint32_t rows, uint32_t cols, int MB, int waves_target, Oil4Plan*
     if (grid == 0) grid = 1;
     const uint32_t Jn = grid * G;
     const uint32_t max_rows = (rows + Jn - 1) / Jn;                // rows of the largest row group
-    const int budget = (kWgt == 1024 ? 6 : 12) / best_cs;          // wave-loads in flight per wave (register budget)
+    const int budget = 12 / best_cs;                               // wave-loads in flight per wave (register budget)
     int rpw = 1;
     if (max_rows <= (uint32_t)budget) {                            // one chunk: the smallest that holds every row
         for (int cand : {1, 2, 3, 4, 6, 12}) if ((uint32_t)cand >= max_rows) { rpw = cand; break; }
@@ -505,14 +477,10 @@ int dispatch(const oilhip_weights& w, const float* d_x, const float* d_xw, float
     if (p.cs == CS_ && p.rpw == RPW_) \
         return p.nchunks > 1 ? launch<CS_, RPW_, MB, kWgt, XF, true>(w, d_x, d_xw, d_y, M, s, p, out_scale) \
                              : launch<CS_, RPW_, MB, kWgt, XF, false>(w, d_x, d_xw, d_y, M, s, p, out_scale);
-    OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6)
-    if constexpr (kWgt == 512) { OIL4_CASE(1, 12) }
+    OIL4_CASE(1, 1) OIL4_CASE(1, 2) OIL4_CASE(1, 3) OIL4_CASE(1, 4) OIL4_CASE(1, 6) OIL4_CASE(1, 12)
     if constexpr (MB == 1) {
-        OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3)
-        if constexpr (kWgt == 512) {
-            OIL4_CASE(2, 4) OIL4_CASE(2, 6)
-            OIL4_CASE(3, 1) OIL4_CASE(3, 2) OIL4_CASE(3, 3) OIL4_CASE(3, 4)
-        }
+        OIL4_CASE(2, 1) OIL4_CASE(2, 2) OIL4_CASE(2, 3) OIL4_CASE(2, 4) OIL4_CASE(2, 6)
+        OIL4_CASE(3, 1) OIL4_CASE(3, 2) OIL4_CASE(3, 3) OIL4_CASE(3, 4)
     }
 #undef OIL4_CASE
     return 1;

@@ -1,10 +1,25 @@
 // probe_kernels.hip -- a read-only streaming kernel with the decode GEMVs' load pattern (16 bytes per lane, a KB per
 // wavefront and load, nothing but an XOR done with the data), so that the rate a pure reader reaches on the device at
 // hand is a measured number beside the HBM peak the roofline fractions are quoted against.  No reference counterpart.
-#include "common.h"
+//
+// Built into liboilhip_probe.so, a measurement tool beside the product library (bench.py loads it; nothing in
+// liboilhip.so or its header refers to it).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <string>
 
 namespace oilhip {
 namespace {
+
+thread_local std::string g_probe_error;
+int fail(int code, const char* msg) { g_probe_error = msg; return code; }
+constexpr int OILHIP_OK = 0, OILHIP_E_ARG = -1, OILHIP_E_DEVICE = -3;
+#define OILHIP_HIP(call)                                                                              \
+    do {                                                                                              \
+        hipError_t e_ = (call);                                                                       \
+        if (e_ != hipSuccess) { g_probe_error = std::string(#call) + ": " + hipGetErrorString(e_); return OILHIP_E_DEVICE; } \
+    } while (0)
 
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 
@@ -72,7 +87,13 @@ void launch_nt(int streaming, int pattern, dim3 g, dim3 b, hipStream_t s, const 
 
 using namespace oilhip;
 
-extern "C" int oilhip_read_probe(const void* d_buf, uint64_t bytes, int in_flight, int streaming, int pattern,
+extern "C" const char* oilprobe_last_error() { return g_probe_error.c_str(); }
+
+// bytes are read once by workgroups x threads / 64 wavefronts, each with in_flight (1, 2, 4, 8) loads outstanding;
+// streaming != 0 marks the loads non-temporal; pattern 0 gives each wavefront a contiguous share, 1 interleaves them
+// KB by KB, 2 is the multi-token GEMV's pattern (512 threads, 4 or 8 loads in flight: a load fetches 64 bytes of each
+// of 16 rows of 2 KB).  d_sink needs workgroups x threads / 64 words (practically never written).  0 = ok.
+extern "C" int oilprobe_read(const void* d_buf, uint64_t bytes, int in_flight, int streaming, int pattern,
                                  int workgroups, int threads, uint32_t* d_sink, void* stream) {
     if (!d_buf || !d_sink) return fail(OILHIP_E_ARG, "read_probe: null pointer");
     if (bytes < 1024 || ((uintptr_t)d_buf & 15u)) return fail(OILHIP_E_ARG, "read_probe: needs at least 1 KB, 16-byte aligned");

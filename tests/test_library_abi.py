@@ -90,11 +90,6 @@ def test_entry_points_reject_bad_arguments_before_touching_the_device():
     refused(L.oilhip_dense_gemm_f32(1.0, p, p, 0.0, p, -1, 1, 1, None), "negative")
     refused(L.oilhip_dense_gemv_f32(1.0, None, p, 0.0, p, 2, 2, None), "null")
     refused(L.oilhip_dense_softmax_f32(None, p, 1, 4, 1, None), "null")
-    refused(L.oilhip_read_probe(p, 4096, 3, 0, 0, 256, 512, p, None), "in flight")
-    refused(L.oilhip_read_probe(p, 4096, 4, 0, 0, 256, 100, p, None), "threads")
-    refused(L.oilhip_read_probe(p, 4096, 4, 0, 3, 256, 512, p, None), "pattern")
-    refused(L.oilhip_read_probe(p, 1 << 20, 4, 0, 2, 256, 256, p, None), "pattern 2")      # needs 512 threads
-    refused(L.oilhip_read_probe(p, 1 << 20, 4, 0, 2, 256, 512, p, None), "pattern 2")      # less than 32 KB per workgroup
     refused(L.oilhip_profile_gemv(4, p, p, 1.0, p, p, 4, 16, 10, None, None), "null result")
     perf = (C.c_uint64 * 4)()
     refused(L.oilhip_profile_gemv(5, p, p, 1.0, p, p, 4, 16, 10, C.addressof(perf), None), "kind")
