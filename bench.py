@@ -128,6 +128,64 @@ def cpu_baseline(payload, blocks, rows, cols, x):
                       f"oracle restatement of Qwen35Engine::gemm (per-block bit-stream decode + FP32 dot)"}
 
 
+def time_calls(torch, fn, min_ms=50.0, warm=3):
+    """Seconds per call of fn(): whole batches of calls between two events, the batch doubled until it spans at least
+    min_ms of device time (the 3-5 warm-ups and mean-over-iterations convention of bench/bench_oil_quant.cpp:22-31)."""
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    n = 8
+    while True:
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(n):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        if ms >= min_ms or n >= 1 << 16:
+            return ms * 1e-3 / n
+        n *= 2
+
+
+def cpu_flat_oil8(with_reference=True):
+    """The flat-codebook CPU leg: kernel::oil8_gemm gather semantics (src/kernel_oil8.cpp:35-68: eight-lane
+    accumulators, horizontal add) at config 1's M=1, K=N=4096 on ONE thread, as the reference runs it: 3 warm-ups,
+    mean of 100 timed iterations (bench/bench_oil_quant.cpp:22-31).  The oracle's restatement, and beside it the
+    compiled reference's own oil8_gemm where oracle/_ref is built."""
+    import numpy as np
+    import oracle as O
+    rng = np.random.default_rng(8)
+    N = K = 4096
+    idx = rng.integers(0, 256, N * K, dtype=np.uint8)
+    cb = np.linspace(-8.0, 8.0, 256, dtype=np.float32)
+    act = rng.standard_normal(K).astype(np.float32)
+    out = {}
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        t0 = time.perf_counter()
+        for _ in range(100):
+            fn()
+        return (time.perf_counter() - t0) / 100
+
+    res = np.zeros(N, dtype=np.float32)
+    L = O.lib()
+    pi, pc, pa, po = (O._p(idx, O._u8p), O._p(cb, O._f32p), O._p(act, O._f32p), O._p(res, O._f32p))
+    t = timed(lambda: L.orc_oil8_gemm(pi, pc, pa, po, 1, N, K, 1))
+    out["cpu_flat_oil8_GBps"] = round(N * K / t / 1e9, 3)
+    out["cpu_flat_oil8_ms"] = round(t * 1e3, 3)
+    out["cpu_flat_oil8_threads"] = 1
+    out["cpu_flat_oil8_kind"] = "port (oracle restatement of kernel::oil8_gemm, AVX2 summation order), 100 iterations after 3 warm-ups"
+    R = O.ref() if with_reference else None
+    if R is not None:
+        t = timed(lambda: R.ref_oil8_gemm(pi, pc, pa, po, 1, N, K))
+        out["cpu_flat_oil8_reference_GBps"] = round(N * K / t / 1e9, 3)
+        out["cpu_flat_oil8_reference_kind"] = "reference (oracle/_ref: the reference's own kernel::oil8_gemm compiled with -mavx2 -mfma), one thread"
+    return out
+
+
 def time_gemvs(torch, items, xs, ys, reps):
     """Seconds per pass over `items` (a list of (DeviceWeights, x index)), graph replay."""
     for d, k in items:
@@ -409,33 +467,21 @@ def bench_prefill(torch, ia, payload, blocks):
             for M in (512, 2048):
                 x = torch.randn(M, cols, device="cuda").to(torch.bfloat16)
                 y = torch.empty((M, rows), dtype=torch.float32, device="cuda")
-                for _ in range(3):
-                    d.gemm_bf16(x, out=y)
-                torch.cuda.synchronize()
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-                for _ in range(20):
-                    d.gemm_bf16(x, out=y)
-                e1.record()
-                torch.cuda.synchronize()
-                t = e0.elapsed_time(e1) * 1e-3 / 20
+                t = time_calls(torch, lambda: d.gemm_bf16(x, out=y))          # at least 50 ms of launches
                 out[f"prefill_M{M}_N{rows}_TFLOPs"] = round(2.0 * M * rows * cols / t / 1e12, 1)
+                out[f"prefill_M{M}_N{rows}_us"] = round(t * 1e6, 1)
+                if M == 512 and rows == 11008:                                # the reference's own call: FP32 activations
+                    xf = x.float()
+                    tf = time_calls(torch, lambda: d.gemm_f32(xf, out=y))
+                    out["prefill_fp32_in_M512_N11008_us"] = round(tf * 1e6, 1)
     # a tensor that is not uniform OIL4 (here SPARK_Q0): decoded to bf16 slab by slab, then the same kernel over a dense operand
     ws = make_weights(11008, 4096, seed=12)
     ps, bs = ia.block_codec.quantize_tensor(ws, ia.Format.SPARK_Q0)
     with ia.DeviceWeights.from_blocks(ps, bs, 11008, 4096) as d:
         x = torch.randn(2048, 4096, device="cuda").to(torch.bfloat16)
         y = torch.empty((2048, 11008), dtype=torch.float32, device="cuda")
-        for _ in range(3):
-            d.gemm_bf16(x, out=y)
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        for _ in range(10):
-            d.gemm_bf16(x, out=y)
-        e1.record()
-        torch.cuda.synchronize()
-        out["prefill_spark_q0_M2048_N11008_TFLOPs"] = round(2.0 * 2048 * 11008 * 4096 / (e0.elapsed_time(e1) * 1e-3 / 10) / 1e12, 1)
+        t = time_calls(torch, lambda: d.gemm_bf16(x, out=y))
+        out["prefill_spark_q0_M2048_N11008_TFLOPs"] = round(2.0 * 2048 * 11008 * 4096 / t / 1e12, 1)
     # what this box reaches with a plain bf16 GEMM of the largest shape (rocBLAS / hipBLASLt through torch), and with a
     # plain device-to-device copy: the practical ceilings next to the vendor peaks
     a = torch.randn(2048, 4096, device="cuda").to(torch.bfloat16)
@@ -661,15 +707,7 @@ def bench_moe(torch, ia):
     _, idx, w = moe.softmax_with_topk(logits, K)
     hist = np.bincount(idx.ravel(), minlength=E).tolist()
     x = torch.randn(T, D, device="cuda")
-    for _ in range(2):
-        moe.moe_dispatch_batched(x, experts, idx, w, want_z_loss=False)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    reps = 5
-    for _ in range(reps):
-        moe.moe_dispatch_batched(x, experts, idx, w, want_z_loss=False)
-    torch.cuda.synchronize()
-    t = (time.perf_counter() - t0) / reps
+    t = time_calls(torch, lambda: moe.moe_dispatch_batched(x, experts, idx, w, want_z_loss=False), warm=2)   # >= 50 ms of steps
     touched = sum(3 * D * F // 2 for h in hist if h > 0)
     for e in experts:
         for d in (e.gate_proj, e.up_proj, e.down_proj):
@@ -835,6 +873,7 @@ def main():
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(payload, blocks, ROWS, COLS, xh)
+        out.setdefault("extra", {}).update(cpu_flat_oil8())      # the second CPU leg: flat-codebook gather, one thread
 
     print(json.dumps(out), flush=True)
 
