@@ -67,8 +67,8 @@ struct FragGrid {
     uint32_t halves;        // ... or into two halves along the weight rows (2; 256-row tiles only), each with all of K
 };
 
-// X ([M][K], bf16 bit patterns or FP32) -> X' in A-fragment order, rows >= M zero.  One wavefront writes one 1 KB
-// fragment: lane = 32 * (column half) + token % 32 holds columns 16 g + 8 half .. + 7 of X' (nibble order).
+// X ([M][K], bf16 bit patterns or FP32) -> X' in A-fragment order, rows >= M zero: fragment (32-token block, 16-column
+// group g) is 1 KB, lane = 32 * (column half) + token % 32 holds columns 16 g + 8 half .. + 7 of X' (nibble order).
 // Workgroups past the packing ones clear the Y tiles whose K parts are added: tile nfull + (index).
 template <bool F32, int TM, int TN>
 __global__ void __launch_bounds__(256)
@@ -86,56 +86,68 @@ pack_x_frag_kernel(const void* __restrict__ xin, uint16_t* __restrict__ xf, uint
         }
         return;
     }
-    const uint32_t G = K >> 4, gq = G >> 2;
-    const uint32_t mb = blockIdx.x / gq, g = (blockIdx.x % gq) * 4u + (tid >> 6);
-    const uint32_t lane = tid & 63u, m = mb * 32u + (lane & 31u);
-    const uint32_t c = g * 16u + (lane >> 5) * 8u, p0 = c & 255u;
-    // X' column p of a block (p >= 4) is X column p - 4 + (slots before it): the eight columns of this lane come
-    // from the 16 aligned X columns [c - 8, c + 8), window index k + 4 + slots
-    uint16_t e[16];
+    // One workgroup = 32 tokens x one 256-column block: rows are read whole (a wavefront reads eight rows of 512
+    // bytes, FP32: 1 KB), rounded to bf16 and parked in LDS; then every wavefront writes four of the block's sixteen
+    // 1 KB fragments.  X' column p of a block (p >= 4) is X column p - 4 + (slots before it): the eight columns of a
+    // lane come from the 16 aligned X columns [c - 8, c + 8) of the block, window index k + 4 + slots.
+    constexpr uint32_t PITCH = 256u + 8u;                                    // bf16 per parked row: 16-byte reads of 16 rows hit every bank once
+    __shared__ __align__(16) uint16_t park[32u * PITCH];
+    const uint32_t bpr = K >> 8, G = K >> 4;
+    const uint32_t mb = blockIdx.x / bpr, blk = blockIdx.x % bpr;
+    {
+        const uint32_t r = tid >> 3, q = tid & 7u, m = mb * 32u + r;         // row of the tile; 8-column pieces q, q + 8, q + 16, q + 24 of it
+        uint4 v[4];
 #pragma unroll
-    for (int k = 0; k < 16; ++k) e[k] = 0;
-    if (m < M) {
-        if constexpr (F32) {
-            const float* xr = reinterpret_cast<const float*>(xin) + (size_t)m * K + c;
+        for (int j = 0; j < 4; ++j) v[j] = make_uint4(0u, 0u, 0u, 0u);
+        if (m < M) {
+            if constexpr (F32) {
+                const float4* xr = reinterpret_cast<const float4*>(reinterpret_cast<const float*>(xin) + (size_t)m * K + blk * 256u);
 #pragma unroll
-            for (int h = 0; h < 4; ++h) {
-                if (h < 2 && p0 == 0u) continue;
-                const float4 f = *reinterpret_cast<const float4*>(xr - 8 + 4 * h);
-                const __bf16 b0 = (__bf16)f.x, b1 = (__bf16)f.y, b2 = (__bf16)f.z, b3 = (__bf16)f.w;
-                e[4 * h] = *reinterpret_cast<const uint16_t*>(&b0); e[4 * h + 1] = *reinterpret_cast<const uint16_t*>(&b1);
-                e[4 * h + 2] = *reinterpret_cast<const uint16_t*>(&b2); e[4 * h + 3] = *reinterpret_cast<const uint16_t*>(&b3);
-            }
-        } else {
-            const uint16_t* xr = reinterpret_cast<const uint16_t*>(xin) + (size_t)m * K + c;
+                for (int j = 0; j < 4; ++j) {
+                    const float4 f0 = xr[2u * (q + 8u * j)], f1 = xr[2u * (q + 8u * j) + 1u];
+                    const bf16x2 p0 = bf16x2{(__bf16)f0.x, (__bf16)f0.y}, p1 = bf16x2{(__bf16)f0.z, (__bf16)f0.w};
+                    const bf16x2 p2 = bf16x2{(__bf16)f1.x, (__bf16)f1.y}, p3 = bf16x2{(__bf16)f1.z, (__bf16)f1.w};
+                    v[j] = make_uint4(*reinterpret_cast<const uint32_t*>(&p0), *reinterpret_cast<const uint32_t*>(&p1),
+                                      *reinterpret_cast<const uint32_t*>(&p2), *reinterpret_cast<const uint32_t*>(&p3));
+                }
+            } else {
+                const uint4* xr = reinterpret_cast<const uint4*>(reinterpret_cast<const uint16_t*>(xin) + (size_t)m * K + blk * 256u);
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                if (h == 0 && p0 == 0u) continue;
-                const uint4 q = *reinterpret_cast<const uint4*>(xr - 8 + 8 * h);
-                e[8 * h] = (uint16_t)q.x; e[8 * h + 1] = (uint16_t)(q.x >> 16); e[8 * h + 2] = (uint16_t)q.y; e[8 * h + 3] = (uint16_t)(q.y >> 16);
-                e[8 * h + 4] = (uint16_t)q.z; e[8 * h + 5] = (uint16_t)(q.z >> 16); e[8 * h + 6] = (uint16_t)q.w; e[8 * h + 7] = (uint16_t)(q.w >> 16);
+                for (int j = 0; j < 4; ++j) v[j] = xr[q + 8u * j];
             }
         }
-    }
-    uint16_t v[8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) {
-        const uint32_t p = p0 + k, sl = (p >= 67u) + (p >= 130u) + (p >= 193u);
-        const uint16_t t = sl == 0u ? e[k + 4] : sl == 1u ? e[k + 5] : sl == 2u ? e[k + 6] : e[k + 7];
-        v[k] = p >= 4u ? t : (uint16_t)0;
+        for (int j = 0; j < 4; ++j) *reinterpret_cast<uint4*>(park + r * PITCH + (q + 8u * j) * 8u) = v[j];
     }
-    uint4 o;
-    o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
-    o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
-    *reinterpret_cast<uint4*>(xf + (((size_t)mb * G + g) * 64u + lane) * 8u) = o;
+    __syncthreads();
+    const uint32_t lane = tid & 63u, r = lane & 31u, half = lane >> 5;
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+        const uint32_t gl = (tid >> 6) + 4u * f, p0 = gl * 16u + half * 8u;   // fragment of the block, first X' column of the lane
+        uint4 w0 = make_uint4(0u, 0u, 0u, 0u);
+        if (p0 != 0u) w0 = *reinterpret_cast<const uint4*>(park + r * PITCH + p0 - 8u);
+        const uint4 w1 = *reinterpret_cast<const uint4*>(park + r * PITCH + p0);
+        const uint32_t wd[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w};
+        uint16_t e[16];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { e[2 * k] = (uint16_t)wd[k]; e[2 * k + 1] = (uint16_t)(wd[k] >> 16); }
+        uint16_t v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const uint32_t p = p0 + k, sl = (p >= 67u) + (p >= 130u) + (p >= 193u);
+            const uint16_t t = sl == 0u ? e[k + 4] : sl == 1u ? e[k + 5] : sl == 2u ? e[k + 6] : e[k + 7];
+            v[k] = p >= 4u ? t : (uint16_t)0;
+        }
+        uint4 o;
+        o.x = v[0] | ((uint32_t)v[1] << 16); o.y = v[2] | ((uint32_t)v[3] << 16);
+        o.z = v[4] | ((uint32_t)v[5] << 16); o.w = v[6] | ((uint32_t)v[7] << 16);
+        *reinterpret_cast<uint4*>(xf + (((size_t)mb * G + blk * 16u + gl) * 64u + lane) * 8u) = o;
+    }
 }
 
 template <int V> using IC = std::integral_constant<int, V>;
 
-#ifndef OILHIP_FRAG_AHEAD
-#define OILHIP_FRAG_AHEAD 2
-#endif
-constexpr int kFragAhead = OILHIP_FRAG_AHEAD;
+constexpr int kFragAhead = 2;
 
 // One workgroup's tile: tokens [m0, m0 + 64 FM), weight rows [n0, n0 + 64 FN), part kpart of `parts` along K.
 template <int FM, int FN>
@@ -447,7 +459,7 @@ int launch_frag(const oilhip_weights& w, const void* d_x, float* d_y, uint32_t M
     const uint32_t Mpad = gr.MT * TM;
     uint16_t* xf = nullptr;
     if (int rc = stream_scratch(s, kScratchGemmX, (size_t)Mpad * K * 2, reinterpret_cast<void**>(&xf))) return rc;
-    const uint32_t npack = (Mpad / 32u) * (K >> 6), nzero = gr.ksplit > 1u ? tiles - gr.nfull : 0u;
+    const uint32_t npack = (Mpad / 32u) * (K >> 8), nzero = gr.ksplit > 1u ? tiles - gr.nfull : 0u;
     hipLaunchKernelGGL((pack_x_frag_kernel<F32, TM, TN>), dim3(npack + nzero), dim3(256), 0, s, d_x, xf, M, K, npack, d_y, N, N, gr);
     OILHIP_HIP(hipGetLastError());
     static std::atomic<uint64_t> attr_done{0};
