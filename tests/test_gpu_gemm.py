@@ -40,6 +40,41 @@ def test_small_shapes(rows, cols, M):
     assert err <= TOL
 
 
+@pytest.mark.parametrize("rows,cols,M", [(130, 256, 300), (257, 512, 1000), (640, 1024, 1025), (1, 256, 258),
+                                          (300, 2816, 513), (896, 768, 2304)])
+def test_fragment_kernel_edges(rows, cols, M):
+    """More than 256 tokens (the fragment-order kernel): weight rows that end inside a 32-row block and inside a
+    256-row tile, a single 256-column block per row, token counts that end inside a 32-token block, more token tiles
+    than one group of four, a last round of tiles that is cut in halves."""
+    err, y, want = run(rows, cols, M, seed=3 * rows + cols + M)
+    assert y.shape == (M, rows)
+    assert err <= TOL
+    assert np.all(np.isfinite(y))
+
+
+def test_fragment_kernel_takes_misaligned_activations_another_way():
+    """An activation pointer that is not 16-byte aligned cannot use the kernel's 16-byte loads: same result through
+    the older path."""
+    rows, cols, M = 256, 512, 300
+    w = gaussian_weights(rows * cols, 21)
+    payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+    base = torch.randn(M * cols + 8, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).cuda()
+    xa = base[:M * cols].view(M, cols).contiguous()
+    xm = base[1:1 + M * cols].view(M, cols)                   # 2 bytes past a 16-byte boundary
+    assert xm.data_ptr() % 16 != 0
+    with ia.DeviceWeights.from_blocks(payload, blocks, rows, cols) as dw:
+        L = ia._lib.lib()
+        ya = dw.gemm_bf16(xa)
+        ym = torch.empty(M, rows, device="cuda")
+        ia._lib.check(L.oilhip_gemm_bf16(dw.handle, xm.data_ptr(), ym.data_ptr(), M, ia._lib.current_stream()))
+    X = xm.float().cpu().numpy()
+    want = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, X, wide=True)
+    assert rel_l2(ym.cpu().numpy(), want) <= TOL
+    # the two kernels round the same products (levels held as FP32 there, as FP16 here): they agree far inside the bound
+    ya2 = O.block_gemm(payload, to_orc_blocks(blocks), rows, cols, xa.float().cpu().numpy(), wide=True)
+    assert rel_l2(ya.cpu().numpy(), ya2) <= TOL
+
+
 def test_layout_is_not_transposed():
     """Distinct M, N, K and a single hot activation column / weight row pin the index maps."""
     rows, cols, M = 96, 512, 40
