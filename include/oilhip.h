@@ -173,8 +173,11 @@ int oilhip_gemv_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M
 /* The same product for uniform OIL4 tensors, for callers that cannot allocate device memory (code under HIP graph
  * capture, serving loops and harnesses that forbid hipMalloc).  No counterpart in the reference.  It calls no
  * hipMalloc/hipFree: the scratch its multi-row kernel needs (packed activations and their exponents, 8 MB) is a fixed array in the
- * library's code object, one per GPU.  Limits: uniform OIL4 in the plain block layout, cols <= 32768; anything else
- * returns OILHIP_E_ARG.  All calls on one GPU share that array: calls that overlap on one GPU (two streams, two
+ * library's code object, one per GPU.  Limits: uniform OIL4 in the plain block layout, cols <= 32768; and, where
+ * the rows are cut into three or more parts along K whose sums meet in the scratch (M >= 3 with cols > 8192, or
+ * M > 16 with cols > 4096, ordered sums on), parts * tokens_per_pass * rows <= 1,043,456 floats (parts =
+ * ceil(cols / 4096) for passes of up to 16 tokens, ceil(cols / 2048) for passes of 32; e.g. cols = 11008, M <= 16:
+ * rows <= 21,738).  Anything else returns OILHIP_E_ARG.  All calls on one GPU share that array: calls that overlap on one GPU (two streams, two
  * threads) race on it and must be serialized by the caller. */
 int oilhip_gemv_oil4_f32_noalloc(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream);
 
@@ -206,9 +209,9 @@ int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x_bf16, float* d
 int oilhip_gemm_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream);
 
 /* Frees the scratch buffers the library holds for `stream` on the current device (packed activations of the
- * multi-token GEMV, X' and decoded slabs of the prefill GEMM, the lookup kernels' codes): after a stream is destroyed, or
- * to trim after a large batch.  Synchronizes the stream first; no captured graph may still replay launches that were
- * recorded on it.  (No counterpart in the reference, which owns no device memory.) */
+ * multi-token GEMV, X' and decoded slabs of the prefill GEMM, the lookup kernels' codes; buffers that a larger request
+ * has replaced included): before a stream is destroyed, or to trim after a large batch.  Synchronizes the stream
+ * first, so the stream must still exist; no captured graph may still replay launches that were recorded on it.  (No counterpart in the reference, which owns no device memory.) */
 int oilhip_release_stream_scratch(void* stream);
 
 /* ---------------------------------------------------- flat-codebook kernels

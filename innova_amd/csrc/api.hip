@@ -76,7 +76,12 @@ int ensure_max_lds(std::atomic<uint64_t>& done, const void* kernel, int bytes) {
 }
 
 static std::mutex g_scratch_mu;
-static std::map<std::tuple<int, void*, int>, std::pair<void*, size_t>> g_scratch;
+struct ScratchBuffers {
+    void* first = nullptr;              // the buffer in use
+    size_t second = 0;                  // its size
+    std::vector<void*> outgrown;        // earlier, smaller buffers: kept because a captured graph may still point at them
+};
+static std::map<std::tuple<int, void*, int>, ScratchBuffers> g_scratch;
 
 int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out) {
     int dev = 0;
@@ -101,7 +106,9 @@ int stream_scratch(hipStream_t s, int slot, size_t bytes, void** out) {
             (void)hipFree(p);
             return fail(OILHIP_E_DEVICE, "hipMemset of the new scratch failed");
         }
-        e = {p, want};                       // the smaller buffer stays allocated (see common.h)
+        if (e.first) e.outgrown.push_back(e.first);   // the smaller buffer stays allocated until the stream's scratch is released
+        e.first = p;
+        e.second = want;
     }
     *out = e.first;
     return OILHIP_OK;
@@ -605,6 +612,7 @@ int oilhip_release_stream_scratch(void* stream) {
     for (auto it = g_scratch.begin(); it != g_scratch.end();) {
         if (std::get<0>(it->first) == dev && std::get<1>(it->first) == stream) {
             (void)hipFree(it->second.first);
+            for (void* old : it->second.outgrown) (void)hipFree(old);
             it = g_scratch.erase(it);
         } else {
             ++it;

@@ -104,6 +104,7 @@ inline bool plain_oil8(const oilhip_weights& w) {
 // kernels (each returns an OILHIP_* code and sets the error text)
 int launch_dequant(const oilhip_weights& w, float* d_out, hipStream_t s);
 int launch_dequant_bf16_blocks(const oilhip_weights& w, uint32_t b0, uint32_t nb, uint16_t* d_out, hipStream_t s);
+bool dequant_bf16_blocks_covers(const oilhip_weights& w);   // whether launch_dequant_bf16_blocks takes this tensor's layout
 int launch_gemv_generic(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);
 // fast paths return 1 when they do not cover the case (caller falls through to the general kernel)
 int launch_gemv_oil4(const oilhip_weights& w, const float* d_x, float* d_y, int M, hipStream_t s);

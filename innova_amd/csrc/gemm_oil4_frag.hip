@@ -308,7 +308,7 @@ __device__ __forceinline__ void frag_tile(const uint8_t* __restrict__ W, const u
 #pragma unroll
             for (int t = 0; t < NBW; ++t)                        // piece t is complete behind the rounding of its unit 4 t
                 if (mslot(NU - 1 - 4 * t) + 1 == n) q_store(q0, t, wbuf);
-            if (n % FM == FM - 1 && (NM != 16 || n != 3 && n != 7)) read_frag1(rk, rbuf, j);
+            if (n % FM == FM - 1 && (NM != 16 || (n != 3 && n != 7))) read_frag1(rk, rbuf, j);
             if (NM == 16 && (n == 4 || n == 9)) read_frag1(rk, rbuf, n == 4 ? 0 : 1);
 #pragma unroll
             for (int u = 0; u < NU; ++u)

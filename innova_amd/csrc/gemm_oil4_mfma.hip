@@ -400,6 +400,11 @@ gemm_oil4_bf16_pipe_kernel(const uint8_t* __restrict__ W, const uint16_t* __rest
     __syncthreads();                                   // table complete
     store_tiles(0, 0);
     load_regs(0, clampk(kbeg + (uint32_t)D));
+    // The two wavefront groups run different instantiations of `run` and meet at workgroup barriers written at
+    // different places of the code: the hardware barrier only counts arrivals, so the two instantiations must execute
+    // the same number of barriers in total (group 0: 1 + 2 per step + 1, group 1: 2 + 2 per step).  Any change to one
+    // instantiation's barriers needs the matching change in the other.
+    static_assert(D >= 2 && D % 2 == 0, "the tile buffer of a step is (u + 1 + G) & 1: the unrolled steps must come in pairs");
     auto run = [&](auto gc) {
         constexpr int G = decltype(gc)::value;
         if constexpr (G == 1) {                        // the late group also brings its share of tile 1
@@ -529,6 +534,7 @@ int launch_gemm_any_bf16(const oilhip_weights& w, const uint16_t* d_x, float* d_
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
     const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols, bpr = K >> 8;
     if ((uint64_t)M * K * 2u >= 0x80000000ull) return fail(OILHIP_E_ARG, "activation matrix too large for the prefill kernel");
+    if (!dequant_bf16_blocks_covers(w)) return 1;      // before any scratch is allocated for it
     // slab: at most 64 MB of bf16, a multiple of 128 rows
     uint32_t slab = (uint32_t)std::min<uint64_t>(N, std::max<uint64_t>(128, ((64ull << 20) / ((uint64_t)K * 2u)) & ~127ull));
     uint16_t* wd = nullptr;

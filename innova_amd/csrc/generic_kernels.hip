@@ -252,6 +252,8 @@ static int full_block_layout(const oilhip_weights& w) {
     return by_desc ? 2 : 0;
 }
 
+bool dequant_bf16_blocks_covers(const oilhip_weights& w) { return full_block_layout(w) != 0; }
+
 // The blocks [b0, b0 + nb) decoded to bf16 at d_out (nb * 256 values).  Returns 1 when the tensor's blocks are not
 // full blocks of nominal size.
 int launch_dequant_bf16_blocks(const oilhip_weights& w, uint32_t b0, uint32_t nb, uint16_t* d_out, hipStream_t s) {

@@ -291,3 +291,39 @@ def test_two_streams_run_multi_token_gemvs_concurrently():
         assert np.array_equal(mid, again.cpu().numpy()), i
     for h in handles:
         h.close()
+
+
+def test_release_stream_scratch_frees_every_buffer_of_the_stream():
+    """A stream's scratch grows with the requests (the smaller buffer is kept for graphs that may point at it);
+    oilhip_release_stream_scratch returns all of it, and the next call on the stream allocates afresh and agrees."""
+    st = torch.cuda.Stream()
+    rng = np.random.default_rng(31)
+    cases = []
+    for rows, cols, M in ((256, 4096, 5), (8192, 11008, 16)):       # packed activations (4 MB), then partial sums on top
+        w = gaussian_weights(rows * cols, rows + M)
+        payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
+        cases.append((ia.DeviceWeights.from_blocks(payload, blocks, rows, cols),
+                      torch.from_numpy(rng.standard_normal((M, cols)).astype(np.float32)).cuda(),
+                      torch.empty(M, rows, device="cuda"), torch.empty(M, rows, device="cuda")))
+    release = ia._lib.lib().oilhip_release_stream_scratch
+    with torch.cuda.stream(st):
+        cases[0][3].zero_()                                          # the runtime sets up the stream's queue on its first launch
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    with torch.cuda.stream(st):
+        for dw, x, y, _ in cases:
+            dw.gemv(x, out=y)
+    st.synchronize()
+    held = free0 - torch.cuda.mem_get_info()[0]
+    assert held >= 12 << 20                                          # the first buffer and the one that replaced it
+    ia._lib.check(release(st.cuda_stream))
+    assert torch.cuda.mem_get_info()[0] >= free0
+    with torch.cuda.stream(st):
+        for dw, x, _, y2 in cases:
+            dw.gemv(x, out=y2)
+    st.synchronize()
+    for dw, x, y, y2 in cases:
+        assert np.array_equal(y.cpu().numpy(), y2.cpu().numpy())
+    ia._lib.check(release(st.cuda_stream))
+    for dw, *_ in cases:
+        dw.close()
