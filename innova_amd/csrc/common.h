@@ -121,9 +121,9 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
                            float* d_y2 = nullptr, uint32_t ldy2 = 0, const float* d_x2 = nullptr, uint32_t* d_pack = nullptr,
                            size_t pack_cap = 0);
 void g_ordered_sums_set(int v);
-// several batches of one tensor shape in one launch (gemv_oil4_multi.hip); kind 0 / 1 / 2: batches of up to 8 / 16 / 32 rows
-size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t cols);
-int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const* wa, float* const* ya,
+// several batches of one tensor shape in one launch (gemv_oil4_multi.hip); kinds[b] = 0 / 1 / 2: batch b holds up to 8 / 16 / 32 rows
+size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols);
+int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
                                    uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean = false);

@@ -25,6 +25,7 @@
 
 #include <algorithm>
 #include <mutex>
+#include <numeric>
 
 #include "common.h"
 #include "oil4_lds.h"
@@ -85,6 +86,10 @@ struct PackJobs {
     uint32_t n, wgs_per_job;
     int M[kMaxJobs], row0[kMaxJobs];
     uint32_t xp_off[kMaxJobs], exp_off[kMaxJobs];
+    uint8_t kind[kMaxJobs];     // pass size of the batch: 0 = 8 tokens, 1 = 16, 2 = 32 (wgs_per_job is that of the largest one present)
+    float* clear0[kMaxJobs];    // outputs of the batch (M rows of clear_rows floats) that two row parts add into: they start at zero
+    float* clear1[kMaxJobs];
+    uint32_t clear_rows, clear_ld;
     int use_list;
     int list[kMaxListed];
 };
@@ -102,6 +107,15 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
         bid -= job * jobs.wgs_per_job;
         M = jobs.M[job]; row0 = jobs.row0[job];
         xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+        const uint32_t kind = jobs.kind[job];
+        half = kind == 0u ? 1 : 0;
+        for (int o = 0; o < 2; ++o) {
+            float* yc = o ? jobs.clear1[job] : jobs.clear0[job];
+            if (yc)
+                for (uint32_t i = bid * 256u + tid; i < jobs.clear_rows * (uint32_t)M; i += jobs.wgs_per_job * 256u)
+                    yc[(size_t)(i / jobs.clear_rows) * jobs.clear_ld + i % jobs.clear_rows] = 0.0f;
+        }
+        if (bid >= (kind == 0u ? 8u : kind == 1u ? 16u : 32u) * (((cols >> 8) + 3u) / 4u)) return;   // a smaller pass than the launch's largest
     }
     // outputs that the main kernel's two row parts add into start at zero
     const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
@@ -167,10 +181,12 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
 // NT = 2: passes of 32 tokens.  A wavefront then owns one block of the row per K-pass (8 blocks per pass) and keeps
 // the split activations of two token tiles of it, so a decoded weight operand serves two matrix instructions per
 // product term; a row tile is two groups of 16 rows.
-// Several tensors of one shape in one launch (the experts of a mixture-of-experts step): workgroup blockIdx.x serves
-// tensor blockIdx.x / wgs_per_job with that tensor's packed activations, batch size and output.
+// Several tensors of one shape in one launch (the experts of a mixture-of-experts step): each tensor (job) owns a range
+// of the launch's workgroups and brings its packed activations, batch size and output.
 struct MultiJobs {
-    uint32_t n, wgs_per_job;
+    uint32_t n;
+    uint32_t wg_begin[kMaxJobs + 1];   // job j runs workgroups [wg_begin[j], wg_begin[j + 1]): as many as its share of the launch's work
+    uint32_t g_base[kMaxJobs], g_rem[kMaxJobs];   // row groups per slab of the job: g_base, and one more for the first g_rem slabs
     const uint8_t* W[kMaxJobs];
     float* y[kMaxJobs];
     int M[kMaxJobs];
@@ -178,18 +194,10 @@ struct MultiJobs {
 };
 
 template <bool HALF, int NT>
-__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
-gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
-                       uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
-                       uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, const MultiJobs jobs) {
-    uint32_t bid = blockIdx.x;
-    if (jobs.n) {
-        const uint32_t job = bid / jobs.wgs_per_job;
-        bid -= job * jobs.wgs_per_job;
-        W = jobs.W[job]; y = jobs.y[job]; M = jobs.M[job];
-        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
-        partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
-    }
+__device__ __forceinline__ void
+multi_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
+           uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
+           uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, uint32_t bid) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
@@ -455,6 +463,52 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
     }
 }
 
+template <bool HALF, int NT>
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
+                       uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
+                       uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, const MultiJobs jobs) {
+    uint32_t bid = blockIdx.x;
+    if (jobs.n) {
+        uint32_t job = 0;
+        while (job + 1u < jobs.n && bid >= jobs.wg_begin[job + 1u]) ++job;   // uniform: a few scalar steps
+        bid -= jobs.wg_begin[job];
+        W = jobs.W[job]; y = jobs.y[job]; M = jobs.M[job];
+        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+        partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
+        g_base = jobs.g_base[job]; g_rem = jobs.g_rem[job];
+    }
+    multi_body<HALF, NT>(W, xp, xp_exp, y, rows, cols, m0, M, ldy, g_base, g_rem, ksplit, partial, counter, ordered, bid);
+}
+
+// Batches of different pass sizes in one launch: the job's pass size selects the body, and with it the number of K
+// parts (a job's workgroup count is a multiple of it).
+struct MixedPlan {
+    uint8_t kind[kMaxJobs];
+    uint32_t ksplit[3];
+};
+
+__global__ void __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2)))
+gemv_oil4_multi_mixed_kernel(const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, uint32_t rows, uint32_t cols, uint32_t ldy,
+                             float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, const MultiJobs jobs,
+                             const MixedPlan plan) {
+    uint32_t job = 0;
+    while (job + 1u < jobs.n && blockIdx.x >= jobs.wg_begin[job + 1u]) ++job;
+    const uint32_t bid = blockIdx.x - jobs.wg_begin[job], g_base = jobs.g_base[job], g_rem = jobs.g_rem[job];
+    const uint8_t* W = jobs.W[job];
+    float* y = jobs.y[job];
+    const int M = jobs.M[job];
+    xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+    partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
+    const uint32_t kind = plan.kind[job];                                   // workgroup-uniform
+    if (kind == 0u)
+        multi_body<true, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[0], partial, counter, ordered, bid);
+    else if (kind == 1u)
+        multi_body<false, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[1], partial, counter, ordered, bid);
+    else
+        multi_body<false, 2>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[2], partial, counter, ordered, bid);
+}
+
 
 // the packed activations of one pass (two token tiles) live in a scratch buffer of the stream the call runs on, or in
 // the buffer the caller hands in
@@ -567,25 +621,41 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
 
 
 // ---- several batches in one launch (the experts of a mixture-of-experts step) ---------------------------------------
-// Batch b multiplies M[b] <= (8, 16, 32 for kind 0, 1, 2) activation rows with tensor wa[b] (and, with wb, with a
+// Batch b multiplies M[b] <= (8, 16, 32 for kinds[b] = 0, 1, 2) activation rows with tensor wa[b] (and, with wb, with a
 // second tensor of the same shape: an expert's gate and up projections share their activations).  All tensors have
-// one shape.  The activation rows of batch b are rows list[row0[b] + m] of x when `list` is given (the list is passed
-// by value with the launch), else rows row0[b] + m; with x2 they are silu(x) * x2.  Outputs: ya[b][m * ldy + r].
-// Workspace layout: packed activations and exponents per batch, one counter block and one partial-sum area per job.
-size_t gemv_oil4_multi_batches_bytes(int kind, int nb, uint64_t rows, uint64_t cols) {
-    const uint32_t bpr = (uint32_t)(cols >> 8), NT = kind == 2 ? 2u : 1u, tokens = kind == 0 ? 8u : kind == 1 ? 16u : 32u;
-    const uint32_t pb = kind == 2 ? 8u : 16u, ks = (bpr + pb - 1u) / pb;
-    size_t per_batch = (size_t)NT * bpr * 16384u + (size_t)NT * bpr * 64u;
-    size_t per_job = ks > 2u ? (size_t)ks * tokens * rows * 4u : 0u;
-    return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)2 * nb * per_job + 256u;
-}
-
-// Whether a grouped launch over tensors with rows of `cols` weights adds partial sums into its outputs with atomics
-// (two K parts, or more with the ordered sums switched off): the outputs must then start at zero.
-bool gemv_oil4_multi_batches_accumulate(int kind, uint64_t cols) {
-    const uint32_t bpr = (uint32_t)(cols >> 8), pb = kind == 2 ? 8u : 16u;
+// one shape; the batches may differ in pass size (one launch then runs the three kernel bodies side by side).  The
+// activation rows of batch b are rows list[row0[b] + m] of x when `list` is given (the list is passed by value with
+// the launch), else rows row0[b] + m; with x2 they are silu(x) * x2.  Outputs: ya[b][m * ldy + r].
+// Workspace layout: one counter page per job, then packed activations and exponents per batch (sized for two token
+// tiles), then one partial-sum area per job (sized for the pass size that needs most).
+namespace {
+uint32_t parts_of(int kind, uint32_t bpr) {
+    const uint32_t pb = kind == 2 ? 8u : 16u;
     uint32_t ks = (bpr + pb - 1u) / pb;
     if (ks < 2u || ks > (uint32_t)device_cu_count()) ks = 1u;
+    return ks;
+}
+uint32_t tokens_of(int kind) { return kind == 0 ? 8u : kind == 1 ? 16u : 32u; }
+size_t job_partial_floats(uint32_t bpr, uint64_t rows) {
+    size_t m = 0;
+    for (int kind = 0; kind < 3; ++kind) {
+        const uint32_t ks = parts_of(kind, bpr);
+        if (ks > 2u) m = std::max(m, (size_t)ks * tokens_of(kind) * rows);
+    }
+    return m;
+}
+}  // namespace
+
+size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols) {
+    const uint32_t bpr = (uint32_t)(cols >> 8);
+    const size_t per_batch = (size_t)2 * bpr * 16384u + (size_t)2 * bpr * 64u;
+    return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)2 * nb * job_partial_floats(bpr, rows) * 4u + 256u;
+}
+
+// Whether a grouped launch with passes of this size over tensors with rows of `cols` weights adds partial sums into its
+// outputs with atomics (two K parts, or more with the ordered sums switched off): the outputs must then start at zero.
+bool gemv_oil4_multi_batches_accumulate(int kind, uint64_t cols) {
+    const uint32_t ks = parts_of(kind, (uint32_t)(cols >> 8));
     return ks == 2u || (ks > 2u && g_ordered_sums.load(std::memory_order_relaxed) == 0);
 }
 
@@ -598,52 +668,69 @@ int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s) {
     return OILHIP_OK;
 }
 
-int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const* wa, float* const* ya,
+int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
                                    uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean) {
-    if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || kind < 0 || kind > 2 || nlist > kMaxListed) return 1;
+    if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || nlist > kMaxListed) return 1;
     const oilhip_weights& w0 = *wa[0];
     if (w0.rows == 0 || w0.rows > 0x7FFFFFFFull || w0.cols > kMaxPackCols || (w0.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
-    if (ws_bytes < gemv_oil4_multi_batches_bytes(kind, nb, w0.rows, w0.cols)) return 1;
-    static std::atomic<uint64_t> attr_done[3];
+    if (ws_bytes < gemv_oil4_multi_batches_bytes(nb, w0.rows, w0.cols)) return 1;
+    static std::atomic<uint64_t> attr_done[4];
     if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>), kMaxLds)) return rc;
     if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>), kMaxLds)) return rc;
     if (int rc = ensure_max_lds(attr_done[2], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<true, 1>), kMaxLds)) return rc;
+    if (int rc = ensure_max_lds(attr_done[3], reinterpret_cast<const void*>(gemv_oil4_multi_mixed_kernel), kMaxLds)) return rc;
     const bool ordered = g_ordered_sums.load(std::memory_order_relaxed) != 0;
-    const uint32_t bpr = (uint32_t)(w0.cols >> 8), NT = kind == 2 ? 2u : 1u, tokens = kind == 0 ? 8u : kind == 1 ? 16u : 32u;
-    const uint32_t pb = kind == 2 ? 8u : 16u;
-    uint32_t ks = (bpr + pb - 1u) / pb;
-    if (ks < 2u || ks > (uint32_t)device_cu_count()) ks = 1u;
-    const size_t xp_dwords = (size_t)NT * bpr * 4096u, exp_ints = (size_t)NT * bpr * 16u;
+    const uint32_t bpr = (uint32_t)(w0.cols >> 8);
+    bool present[3] = {false, false, false};
+    for (int b = 0; b < nb; ++b) {
+        if (kinds[b] < 0 || kinds[b] > 2) return 1;
+        present[kinds[b]] = true;
+    }
+    const int nkinds = (int)present[0] + (int)present[1] + (int)present[2];
+    const int only = present[0] ? 0 : present[1] ? 1 : 2;                   // the kind of a launch with one pass size
+    const size_t xp_dwords = (size_t)2 * bpr * 4096u, exp_ints = (size_t)2 * bpr * 16u;
     uint32_t* counter = static_cast<uint32_t*>(d_ws);
     uint8_t* base = static_cast<uint8_t*>(d_ws) + kBatchCounterBytes;
     uint32_t* xp = reinterpret_cast<uint32_t*>(base);
     int* xp_exp = reinterpret_cast<int*>(base + (size_t)nb * xp_dwords * 4u);
     const int njobs = wb ? 2 * nb : nb;
     uint8_t* jobs_base = base + (size_t)nb * (xp_dwords * 4u + exp_ints * 4u);
-    const size_t part_floats = ks > 2u ? (size_t)ks * tokens * w0.rows : 0u;
+    const size_t part_floats = job_partial_floats(bpr, w0.rows);
     float* partial = reinterpret_cast<float*>(jobs_base);
     // 32-bit offsets: a job's place in the areas (in dwords and floats), and bytes within one job's partial sums
     if (xp_dwords * (size_t)nb > 0xFFFFFFFFull || part_floats * (size_t)njobs > 0xFFFFFFFFull || part_floats * 4u >= 0x100000000ull) return 1;
 
+    // The launch as a whole fills the device about twice over, so that a workgroup keeps its table and its activations
+    // for many row groups.  A job's share of the workgroups follows its cost (a pass of 32 tokens costs 1.36 times a pass
+    // of 16, a pass of 8 tokens 0.87 times: measured on single tensors), so that all workgroups run about equally long;
+    // a job's count is a multiple of its K parts.
+    const uint32_t groups = ((uint32_t)w0.rows + 15u) / 16u;
+    static const double kCost[3] = {0.87, 1.0, 1.36};
+    uint32_t ks[3];
+    bool any_ordered_parts = false;
+    double cost_sum = 0.0;
+    for (int k = 0; k < 3; ++k) {
+        ks[k] = parts_of(k, bpr);
+        any_ordered_parts = any_ordered_parts || (present[k] && ks[k] > 2u);
+    }
+    for (int b = 0; b < nb; ++b) cost_sum += kCost[kinds[b]] * (wb ? 2.0 : 1.0);
+    const double total = 2.0 * (double)device_cu_count();
+    MixedPlan plan{};
+    for (int k = 0; k < 3; ++k) plan.ksplit[k] = ks[k];
     PackJobs pj{};
     pj.n = (uint32_t)nb;
-    pj.wgs_per_job = (kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u);
+    pj.wgs_per_job = tokens_of(present[2] ? 2 : present[1] ? 1 : 0) * ((bpr + 3u) / 4u);
     pj.use_list = list ? 1 : 0;
     for (int i = 0; i < nlist; ++i) pj.list[i] = list[i];
     MultiJobs mj{};
     mj.n = (uint32_t)njobs;
-    const uint32_t groups = ((uint32_t)w0.rows + 15u) / 16u;
-    // workgroups per tensor: the launch as a whole fills the device about twice over, so that a workgroup keeps its
-    // table and its activations for many row groups
-    uint32_t slabs = std::max<uint32_t>(1u, 2u * (uint32_t)device_cu_count() / ((uint32_t)njobs * ks));
-    if (slabs > groups) slabs = groups;
-    if (slabs > 1024u) slabs = 1024u;
-    mj.wgs_per_job = slabs * ks;
+    pj.clear_rows = (uint32_t)w0.rows; pj.clear_ld = ldy;
+    uint32_t job_slabs[kMaxJobs];
     for (int b = 0; b < nb; ++b) {
-        if (M[b] < 1 || M[b] > (int)tokens) return fail(OILHIP_E_ARG, "multi-row batches: a batch exceeds the pass size");
-        pj.M[b] = M[b]; pj.row0[b] = row0[b];
+        if (M[b] < 1 || M[b] > (int)tokens_of(kinds[b])) return fail(OILHIP_E_ARG, "multi-row batches: a batch exceeds the pass size");
+        pj.M[b] = M[b]; pj.row0[b] = row0[b]; pj.kind[b] = (uint8_t)kinds[b];
         pj.xp_off[b] = (uint32_t)(b * xp_dwords); pj.exp_off[b] = (uint32_t)(b * exp_ints);
         for (int t = 0; t < (wb ? 2 : 1); ++t) {
             const int j = t * nb + b;
@@ -652,17 +739,32 @@ int launch_gemv_oil4_multi_batches(int kind, int nb, const oilhip_weights* const
             mj.W[j] = w->d_payload; mj.y[j] = t ? yb[b] : ya[b]; mj.M[j] = M[b];
             mj.xp_off[j] = pj.xp_off[b]; mj.exp_off[j] = pj.exp_off[b];
             mj.partial_off[j] = (uint32_t)(j * part_floats); mj.counter_off[j] = (uint32_t)(j * 1024);
+            plan.kind[j] = (uint8_t)kinds[b];
+            const uint32_t k = ks[kinds[b]];
+            uint32_t slabs = (uint32_t)(total * kCost[kinds[b]] / cost_sum / (double)k);   // rounded down: one workgroup past two rounds costs a third
+            slabs = std::min(std::max(slabs, 1u), std::min(groups, 1024u));      // a slab holds at least one group; 1024 counters per job
+            job_slabs[j] = slabs;
+            mj.g_base[j] = groups / slabs; mj.g_rem[j] = groups % slabs;
         }
+        // two row parts add into the outputs with atomics: the pack launch clears them
+        if (gemv_oil4_multi_batches_accumulate(kinds[b], w0.cols)) { pj.clear0[b] = ya[b]; pj.clear1[b] = wb ? yb[b] : nullptr; }
     }
-    if (ks > 2u && ordered && !counters_clean)                            // the caller's workspace is not known to be zero
+    for (int j = 0; j < njobs; ++j) mj.wg_begin[j + 1] = mj.wg_begin[j] + job_slabs[j] * ks[plan.kind[j]];
+    const uint32_t wgs_total = mj.wg_begin[njobs];
+    if (any_ordered_parts && ordered && !counters_clean)                  // the caller's workspace is not known to be zero
         hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
     hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
-                       (uint32_t)w0.cols, 0, 0, ldx, xrows, kind == 0 ? 1 : 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
+                       (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
     OILHIP_HIP(hipGetLastError());
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;
-    auto kern = kind == 0 ? gemv_oil4_multi_kernel<true, 1> : kind == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
-    hipLaunchKernelGGL(kern, dim3(mj.wgs_per_job * (uint32_t)njobs), dim3(512), lds_bytes, s, (const uint8_t*)nullptr, xp, xp_exp, (float*)nullptr,
-                       (uint32_t)w0.rows, (uint32_t)w0.cols, 0, 0, ldy, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0, mj);
+    if (nkinds == 1) {
+        auto kern = only == 0 ? gemv_oil4_multi_kernel<true, 1> : only == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
+        hipLaunchKernelGGL(kern, dim3(wgs_total), dim3(512), lds_bytes, s, (const uint8_t*)nullptr, xp, xp_exp, (float*)nullptr,
+                           (uint32_t)w0.rows, (uint32_t)w0.cols, 0, 0, ldy, 0u, 0u, ks[only], partial, counter, ordered ? 1 : 0, mj);
+    } else {
+        hipLaunchKernelGGL(gemv_oil4_multi_mixed_kernel, dim3(wgs_total), dim3(512), lds_bytes, s, xp, xp_exp, (uint32_t)w0.rows,
+                           (uint32_t)w0.cols, ldy, partial, counter, ordered ? 1 : 0, mj, plan);
+    }
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;
 }

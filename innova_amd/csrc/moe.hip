@@ -128,16 +128,10 @@ struct Workspace {
 };
 
 constexpr int kChunk = 16;      // expert batches per grouped launch (gate and up together are 32 tensors)
-constexpr int kMergeBelow = 4;  // fewer remainders of 8 tokens or less than this join the passes of 16
 
 // scratch of one grouped launch: the larger of the gate/up side (rows F, cols D) and the down side (rows D, cols F)
 size_t batch_scratch_bytes(int64_t D, int64_t F) {
-    size_t m = 0;
-    for (int kind = 0; kind < 2; ++kind) {         // passes of 8 and of 16 tokens
-        m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)F, (uint64_t)D));
-        m = std::max(m, gemv_oil4_multi_batches_bytes(kind, kChunk, (uint64_t)D, (uint64_t)F));
-    }
-    return m;
+    return std::max(gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)F, (uint64_t)D), gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)D, (uint64_t)F));
 }
 
 Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
@@ -254,57 +248,55 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
             if (tok[(size_t)i] == tok[(size_t)i - 1]) distinct[(size_t)e] = 0;
     if (dropped) *dropped = drop;
     // ---- grouped path: uniform OIL4 experts, lists small enough to travel with the launches ---------------------
-    // Per pass size (16 or 8 tokens) and chunk of experts: one launch that splits the gathered activations, one
-    // launch over the gate and up projections of all those experts, one that forms silu(gate) * up while splitting it,
-    // one over their down projections; then one combine.  No copy, no synchronisation: the step can be captured.
+    // Per chunk of expert batches (passes of 32, 16 and 8 tokens side by side): one launch that splits the gathered
+    // activations, one launch over the gate and up projections of all those experts, one that forms silu(gate) * up
+    // while splitting it, one over their down projections; then one combine.  No copy, no synchronisation: the step can
+    // be captured.
     bool grouped = ws.batch_bytes > 0 && (int64_t)tok.size() <= kMaxPairs && T * K <= kMaxPairs && !tok.empty();
     for (int e = 0; e < E && grouped; ++e) grouped = plain_oil4(*gate[e]) && plain_oil4(*up[e]) && plain_oil4(*down[e]);
     if (grouped) {
         const int64_t pairs = (int64_t)tok.size();
-        // outputs of row parts that meet through atomics start at zero; so do the z-loss accumulator and the slab
-        // counters at the start of the batch workspace (every launch leaves them at zero again)
-        bool adds = false;                                       // the expert buffers only where a launch adds into them
-        for (int kind = 0; kind < 2; ++kind)
-            adds = adds || gemv_oil4_multi_batches_accumulate(kind, (uint64_t)D) || gemv_oil4_multi_batches_accumulate(kind, (uint64_t)F);
-        hipLaunchKernelGGL(fill_zero3_kernel, dim3(adds ? 1024 : 64), dim3(256), 0, s, ws.g, adds ? (size_t)(pairs * (2 * F + D)) : (size_t)0,
-                           (float*)ws.z, (size_t)2, (float*)ws.batch, kGemvBatchCounterBytes / 4);
+        // the z-loss accumulator and the slab counters at the start of the batch workspace start at zero (every launch
+        // leaves the counters at zero again); outputs that row parts add into are cleared by the launch that splits
+        // the activations
+        hipLaunchKernelGGL(fill_zero3_kernel, dim3(64), dim3(256), 0, s, ws.g, (size_t)0, (float*)ws.z, (size_t)2, (float*)ws.batch,
+                           kGemvBatchCounterBytes / 4);
         OILHIP_HIP(hipGetLastError());
-        struct Batch { int e, pair0, m; };
-        std::vector<Batch> byKind[2];
-        for (int e = 0; e < E; ++e) {
-            int n = begin[(size_t)e + 1] - begin[(size_t)e], pos = begin[(size_t)e];
-            while (n > 0) {
-                const int take = n > 16 ? 16 : n;                 // passes of 16: two of them beat one pass of 32 (twice the products per table read)
-                byKind[take <= 8 ? 0 : 1].push_back(Batch{e, pos, take});
-                pos += take; n -= take;
-            }
-        }
-        // A few remainders ride along with the passes of 16 (a pass of 16 costs the same whatever it holds, about 29 us
-        // per expert here, while launches of their own add four launch gaps and run the device half empty: 43 us each)
-        if (!byKind[1].empty() && byKind[0].size() < (size_t)kMergeBelow && byKind[1].size() + byKind[0].size() <= (size_t)kChunk) {
-            byKind[1].insert(byKind[1].end(), byKind[0].begin(), byKind[0].end());
-            byKind[0].clear();
-        }
-        for (int kind = 1; kind >= 0; --kind)
-            for (size_t c0 = 0; c0 < byKind[kind].size(); c0 += kChunk) {
-                const int nb = (int)std::min<size_t>(kChunk, byKind[kind].size() - c0);
-                const oilhip_weights *wg[kChunk], *wu[kChunk], *wd[kChunk];
-                float *yg[kChunk], *yu[kChunk], *yo[kChunk];
-                int Mb[kChunk], r0[kChunk];
-                for (int b = 0; b < nb; ++b) {
-                    const Batch& B = byKind[kind][c0 + b];
-                    wg[b] = gate[B.e]; wu[b] = up[B.e]; wd[b] = down[B.e];
-                    yg[b] = ws.g + (size_t)B.pair0 * F; yu[b] = ws.u + (size_t)B.pair0 * F; yo[b] = ws.o + (size_t)B.pair0 * D;
-                    Mb[b] = B.m; r0[b] = B.pair0;
+        struct Batch { int e, pair0, m, kind; };
+        std::vector<Batch> batches;
+        for (int pass = 2; pass >= 0; --pass)                     // the longest passes first: they end last
+            for (int e = 0; e < E; ++e) {
+                int n = begin[(size_t)e + 1] - begin[(size_t)e], pos = begin[(size_t)e];
+                while (n > 0) {
+                    // more than 16 tokens: a pass of 32 (its table reads serve two token tiles: 1.36 times the cost of a
+                    // pass of 16); then what is left as a pass of 16 or of 8
+                    const int take = n > 32 ? 32 : n, kind = take <= 8 ? 0 : take <= 16 ? 1 : 2;
+                    if (kind == pass) batches.push_back(Batch{e, pos, take, kind});
+                    pos += take; n -= take;
                 }
-                int rc = launch_gemv_oil4_multi_batches(kind, nb, wg, yg, wu, yu, Mb, r0, tok.data(), (int)tok.size(), d_x, nullptr,
-                                                        (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s, true);
-                if (rc == 0)
-                    rc = launch_gemv_oil4_multi_batches(kind, nb, wd, yo, nullptr, nullptr, Mb, r0, nullptr, 0, ws.g, ws.u,
-                                                        (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s, true);
-                if (rc < 0) return rc;
-                if (rc == 1) return fail(OILHIP_E_ARG, "moe_forward: the grouped launch refused a shape it was planned for");
             }
+        // all pass sizes of a chunk of batches share one launch per side: one launch that splits the gathered
+        // activations, one over the gate and up projections, one that forms silu(gate) * up while splitting it, one
+        // over the down projections
+        for (size_t c0 = 0; c0 < batches.size(); c0 += kChunk) {
+            const int nb = (int)std::min<size_t>(kChunk, batches.size() - c0);
+            const oilhip_weights *wg[kChunk], *wu[kChunk], *wd[kChunk];
+            float *yg[kChunk], *yu[kChunk], *yo[kChunk];
+            int Mb[kChunk], r0[kChunk], kd[kChunk];
+            for (int b = 0; b < nb; ++b) {
+                const Batch& B = batches[c0 + b];
+                wg[b] = gate[B.e]; wu[b] = up[B.e]; wd[b] = down[B.e];
+                yg[b] = ws.g + (size_t)B.pair0 * F; yu[b] = ws.u + (size_t)B.pair0 * F; yo[b] = ws.o + (size_t)B.pair0 * D;
+                Mb[b] = B.m; r0[b] = B.pair0; kd[b] = B.kind;
+            }
+            int rc = launch_gemv_oil4_multi_batches(nb, kd, wg, yg, wu, yu, Mb, r0, tok.data(), (int)tok.size(), d_x, nullptr,
+                                                    (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s, true);
+            if (rc == 0)
+                rc = launch_gemv_oil4_multi_batches(nb, kd, wd, yo, nullptr, nullptr, Mb, r0, nullptr, 0, ws.g, ws.u,
+                                                    (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s, true);
+            if (rc < 0) return rc;
+            if (rc == 1) return fail(OILHIP_E_ARG, "moe_forward: the grouped launch refused a shape it was planned for");
+        }
         CombineLists L{};
         L.K = (int)K;
         for (int64_t i = 0; i < T * K; ++i) { L.pair[i] = -1; L.wgt[i] = 0.0f; }

@@ -29,9 +29,20 @@ class ExpertFFN:
         self.gate_proj, self.up_proj, self.down_proj = gate, up, down
 
 
-def moe_dispatch_batched(x, experts, indices, weights, want_z_loss: bool = True):
+def moe_workspace(x, experts, K: int):
+    """A device buffer of the size one step over x needs (oilhip_moe_workspace_bytes): a caller that passes it to
+    moe_dispatch_batched owns it across steps, and the call then neither allocates nor waits for the stream."""
+    import torch
+    T, D = x.shape
+    nbytes = _lib.lib().oilhip_moe_workspace_bytes(T, K, D, experts[0].gate_proj.rows)
+    return torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+
+
+def moe_dispatch_batched(x, experts, indices, weights, want_z_loss: bool = True, workspace=None, out=None):
     """x: float32 cuda tensor [T][D]; experts: list of ExpertFFN; indices/weights: [T][K] host arrays.
-    -> (out cuda tensor [T][D], z_loss or None, dropped)   (src/moe_variants.cpp:767-827)"""
+    -> (out cuda tensor [T][D], z_loss or None, dropped)   (src/moe_variants.cpp:767-827)
+    With `workspace` (moe_workspace) and without the z-loss the call only queues launches on the current stream: it
+    can be captured into a graph, and the caller keeps workspace and out alive until the work is done."""
     import torch
     assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous() and x.dim() == 2
     T, D = x.shape
@@ -45,11 +56,16 @@ def moe_dispatch_batched(x, experts, indices, weights, want_z_loss: bool = True)
     g, u, d = arr([e.gate_proj for e in experts]), arr([e.up_proj for e in experts]), arr([e.down_proj for e in experts])
     L = _lib.lib()
     nbytes = L.oilhip_moe_workspace_bytes(T, K, D, F)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
-    out = torch.empty((T, D), dtype=torch.float32, device=x.device)
+    own_ws = workspace is None
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device) if own_ws else workspace
+    assert ws.is_cuda and ws.dtype == torch.uint8 and ws.numel() >= nbytes
+    if out is None:
+        out = torch.empty((T, D), dtype=torch.float32, device=x.device)
+    assert out.is_cuda and out.dtype == torch.float32 and out.is_contiguous() and tuple(out.shape) == (T, D)
     z, dropped = C.c_float(0), C.c_int64(0)
     _lib.check(L.oilhip_moe_forward(g, u, d, E, x.data_ptr(), idx.ctypes.data, w.ctypes.data, T, K, out.data_ptr(),
                                     ws.data_ptr(), nbytes, C.byref(z) if want_z_loss else None, C.byref(dropped),
                                     _lib.current_stream()))
-    torch.cuda.current_stream().synchronize()       # ws is released when this returns
+    if own_ws:
+        torch.cuda.current_stream().synchronize()   # ws is released when this returns
     return out, (z.value if want_z_loss else None), dropped.value

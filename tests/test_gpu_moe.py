@@ -55,7 +55,7 @@ def test_dispatch_matches_reference_fixture():
 @pytest.mark.parametrize("T,E,K,D,F,fmts", [(24, 4, 2, 512, 768, (3, 3, 3)),        # OIL4 experts: fast kernel, 1..many tokens each
                                              (40, 2, 2, 256, 512, (3, 3, 3)),        # > 16 tokens per expert: several passes
                                              (12, 8, 2, 256, 512, (3, 3, 3)),        # a few tokens per expert: passes of 8 only
-                                             (50, 6, 2, 256, 512, (3, 3, 3)),        # passes of 16 and six remainders, which get launches of their own
+                                             (50, 6, 2, 256, 512, (3, 3, 3)),        # passes of 32, 16 and 8 side by side in one launch
                                              (9, 3, 1, 256, 512, (4, 10, 1))])       # OIL8 / OIL4_GRP / SPARK_Q0: general kernel
 def test_dispatch_against_oracle(T, E, K, D, F, fmts):
     packs, dense = MF.moe_experts(5 + T, E, D, F, fmts)
@@ -69,6 +69,39 @@ def test_dispatch_against_oracle(T, E, K, D, F, fmts):
     assert rel(out.cpu().numpy(), want) <= TOL
     assert dropped == dw == 0
     assert abs(z - zw) <= 1e-4 * zw
+
+
+def test_step_with_caller_workspace_is_captured_and_replays_bit_for_bit():
+    """With the caller's workspace and without the z-loss a step only queues launches: captured into a graph, every
+    replay returns the bits of the eager step (passes of 32, 16 and 8 tokens; rows cut along K with ordered sums)."""
+    T, E, K, D, F = 44, 3, 2, 512, 12288                                  # d_ff 12288: the down projection's rows are cut in three
+    packs, dense = MF.moe_experts(91, E, D, F, (3, 3, 3))
+    ex = upload(packs, D, F)
+    rng = np.random.default_rng(92)
+    xh = rng.standard_normal((T, D)).astype(np.float32)
+    logits = rng.standard_normal((T, E)).astype(np.float32)
+    logits[:, 0] += 1.5
+    _, idx, w = moe.softmax_with_topk(logits, K)
+    hist = np.bincount(idx.ravel(), minlength=E)
+    assert hist.max() > 32 and hist.min() >= 1
+    x = torch.from_numpy(xh).cuda()
+    ws, out = moe.moe_workspace(x, ex, K), torch.zeros(T, D, device="cuda")
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        moe.moe_dispatch_batched(x, ex, idx, w, want_z_loss=False, workspace=ws, out=out)
+        st.synchronize()
+        eager = out.clone()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=st):
+            moe.moe_dispatch_batched(x, ex, idx, w, want_z_loss=False, workspace=ws, out=out)
+        for _ in range(3):
+            out.zero_()
+            g.replay()
+            st.synchronize()
+            assert torch.equal(out, eager)
+    gd, ud, dd = ([e[j] for e in dense] for j in range(3))
+    want, _, _ = O.moe_dispatch(xh, gd, ud, dd, idx, w, wide=True)
+    assert rel(eager.cpu().numpy(), want) <= TOL
 
 
 def test_bad_arguments():
