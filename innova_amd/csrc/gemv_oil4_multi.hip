@@ -60,17 +60,15 @@ constexpr int kRedBytes = 8 * kGroups * kRedTile * 4;
 // low parts.  Piece j (dwords 4j .. 4j+3 of the 32) of all 64 lanes is one contiguous KB at
 // ((blk*2 + h)*8 + j)*1024 + l*16 bytes, so that a wavefront fetches it with one coalesced 16-byte load per lane.  Nibble p = 32*(kq + 4h) + s of a block holds weight
 // i = q + q/63 with q = p - 4 (p < 4: the block's scale, activation 0).
-// A wavefront packs one block of one token column (256 activations): it finds their largest magnitude, scales them by
+// A workgroup packs one block of the row for all token columns of a tile (or a quarter of them), a wavefront one token
+// column (256 activations) at a time: it finds their largest magnitude, scales them by
 // the power of two that brings it to [2^14, 2^15) (so the FP16 split keeps 22 bits whatever the magnitude of the
 // activations; blocks that are zero or hold a non-finite value stay unscaled) and leaves the exponent at
 // xp_exp[(tile * bpr + blk) * 16 + column] for the main kernel, which undoes it on the block's partial sums.
-__device__ __forceinline__ float pack_value(const float* __restrict__ x, const float* __restrict__ x2, size_t at) {
-    float v = x[at];
-    // x2: the activations are silu(x) * x2, the SwiGLU product in front of an expert's down projection
-    // (ExpertFFN::forward, src/moe_variants.cpp:77-91), formed here instead of in a kernel of its own
-    if (x2) v = (v / (1.0f + expf(-v))) * x2[at];
-    return v;
-}
+
+// silu(a) * b, the SwiGLU product in front of an expert's down projection (ExpertFFN::forward,
+// src/moe_variants.cpp:77-91), formed while the activations are split instead of in a kernel of its own
+__device__ __forceinline__ float swiglu_value(float a, float b) { return (a / (1.0f + expf(-a))) * b; }
 
 __global__ void __launch_bounds__(256) zero_words_kernel(uint32_t* __restrict__ p, uint32_t n) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -96,9 +94,12 @@ struct PackJobs {
 
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
-              int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
+              int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half, int aligned, uint32_t quarters,
               float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld,
               const PackJobs jobs) {
+    // scaled activations of the workgroup's block, by nibble position: row (chunk of 32 positions, token column), 36
+    // floats apart
+    __shared__ __align__(16) float park[8 * 16 * 36];
     const uint32_t bpr = cols >> 8, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     uint32_t bid = blockIdx.x;
     int row0 = 0;
@@ -109,69 +110,112 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
         xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
         const uint32_t kind = jobs.kind[job];
         half = kind == 0u ? 1 : 0;
+        // outputs of the batch that two row parts add into start at zero
+        const uint32_t crows = jobs.clear_rows, cld = jobs.clear_ld, cstep = jobs.wgs_per_job * 256u;
         for (int o = 0; o < 2; ++o) {
             float* yc = o ? jobs.clear1[job] : jobs.clear0[job];
-            if (yc)
-                for (uint32_t i = bid * 256u + tid; i < jobs.clear_rows * (uint32_t)M; i += jobs.wgs_per_job * 256u)
-                    yc[(size_t)(i / jobs.clear_rows) * jobs.clear_ld + i % jobs.clear_rows] = 0.0f;
+            if (!yc) continue;
+            if (((reinterpret_cast<uintptr_t>(yc) & 15u) | (crows & 3u) | (cld & 3u)) == 0u) {
+                for (int mm = 0; mm < M; ++mm)
+                    for (uint32_t r = (bid * 256u + tid) * 4u; r < crows; r += cstep * 4u)
+                        *reinterpret_cast<float4*>(yc + (size_t)mm * cld + r) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            } else {
+                for (int mm = 0; mm < M; ++mm)
+                    for (uint32_t r = bid * 256u + tid; r < crows; r += cstep) yc[(size_t)mm * cld + r] = 0.0f;
+            }
         }
-        if (bid >= (kind == 0u ? 8u : kind == 1u ? 16u : 32u) * (((cols >> 8) + 3u) / 4u)) return;   // a smaller pass than the launch's largest
+        if (bid >= (kind == 2u ? 2u : 1u) * bpr * quarters) return;        // one token tile where the launch's largest pass has two
     }
     // outputs that the main kernel's two row parts add into start at zero
     const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
     if (yc0)
-        for (uint32_t i = gid; i < yc0_rows * (uint32_t)(M - m0); i += gn) yc0[(size_t)(m0 + i / yc0_rows) * yc0_ld + i % yc0_rows] = 0.0f;
+        for (int mm = m0; mm < M; ++mm)
+            for (uint32_t r = gid; r < yc0_rows; r += gn) yc0[(size_t)mm * yc0_ld + r] = 0.0f;
     if (yc1)
-        for (uint32_t i = gid; i < yc1_rows * (uint32_t)(M - m0); i += gn) yc1[(size_t)(m0 + i / yc1_rows) * yc1_ld + i % yc1_rows] = 0.0f;
-    // workgroup = 4 blocks of token column t of a tile (a pass of 32 tokens is two tiles of 16, the second one's data
-    // behind the first's); passes of 8 tokens have 8 token columns: columns 0..7 of the operand carry their high
-    // parts and columns 8..15 their low parts, in the pieces that otherwise hold the high parts of 16 tokens
-    const uint32_t ncol = half ? 8u : 16u, nbg = (bpr + 3u) / 4u;
-    const uint32_t blk = (bid % nbg) * 4u + wave, t = (bid / nbg) % ncol, tile = bid / (nbg * ncol);
-    if (blk >= bpr) return;
-    const int m = m0 + 16 * (int)tile + (int)t;
+        for (int mm = m0; mm < M; ++mm)
+            for (uint32_t r = gid; r < yc1_rows; r += gn) yc1[(size_t)mm * yc1_ld + r] = 0.0f;
+    // workgroup = one block of the row for the 16 token columns of a tile (a pass of 32 tokens is two tiles of 16, the
+    // second one's data behind the first's); passes of 8 tokens have 8 token columns: columns 0..7 of the operand
+    // carry their high parts and columns 8..15 their low parts, in the pieces that otherwise hold the high parts of 16
+    // tokens.  quarters = 4 (small launches): a workgroup takes a quarter of the token columns, one per wavefront, so
+    // that four times as many workgroups share the launch's round trips
+    const uint32_t ncol = half ? 8u : 16u;
+    const uint32_t tq = bid % quarters, blk = (bid / quarters) % bpr, tile = bid / (quarters * bpr);
+    const uint32_t t_lo = quarters == 4u ? 4u * tq : 0u, t_hi = quarters == 4u ? t_lo + 4u : ncol;
+    if (t_lo >= ncol) return;
     xp += (size_t)tile * bpr * 4096u;
-    uint32_t src = 0xFFFFFFFFu;
-    if (m < M) src = jobs.n ? (jobs.use_list ? (uint32_t)jobs.list[row0 + m] : (uint32_t)(row0 + m)) : (tok ? (uint32_t)tok[m] : (uint32_t)m);
-    const bool live = src < xrows;
-    const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u : 0;
-    // this lane's two pairs: pair id = lane + 64 k holds positions 2c, 2c+1 of chunk kq + 4h
-    float v[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
-    uint32_t mx = 0u;
+    // ---- a wavefront takes one token column at a time: 256 columns of x as one 16-byte load per lane, the largest
+    // magnitude of the 252 that carry a weight, the power of two that brings it to [2^14, 2^15), the scaled values
+    // parked by nibble position (column i of the block sits at nibble 4 + i - i/64; columns 63, 127, 191, 255 meet the
+    // block's empty slots and are dropped; nibbles 0..3 hold the block's scale and see activation 0) ---------------
+    float v[4][4];                                                         // [token column of this wavefront][column of the lane]
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
+    for (int k = 0; k < 4; ++k) {                                          // all loads first: one round trip for the wavefront's columns
+        const uint32_t t = t_lo + wave + 4u * (uint32_t)k;
+        const int m = m0 + 16 * (int)tile + (int)t;
+        uint32_t src = 0xFFFFFFFFu;
+        if (t < t_hi && m < M)
+            src = jobs.n ? (jobs.use_list ? (uint32_t)jobs.list[row0 + m] : (uint32_t)(row0 + m)) : (tok ? (uint32_t)tok[m] : (uint32_t)m);
+        const bool live = src < xrows;
+        const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u + 4u * lane : 0;
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const uint32_t pn = 32u * (kq + 4u * h) + 2u * c + e;
-            if (live && pn >= 4u) {
-                const uint32_t q = pn - 4u;
-                v[k][e] = pack_value(x, x2, at + q + q / 63u);
+        for (int e = 0; e < 4; ++e) v[k][e] = 0.0f;
+        if (live && aligned) {                                             // rows that start on 16-byte boundaries
+            const float4 a = *reinterpret_cast<const float4*>(x + at);
+            v[k][0] = a.x; v[k][1] = a.y; v[k][2] = a.z; v[k][3] = a.w;
+            if (x2) {
+                const float4 b = *reinterpret_cast<const float4*>(x2 + at);
+                v[k][0] = swiglu_value(v[k][0], b.x); v[k][1] = swiglu_value(v[k][1], b.y);
+                v[k][2] = swiglu_value(v[k][2], b.z); v[k][3] = swiglu_value(v[k][3], b.w);
             }
-            mx = max(mx, __float_as_uint(v[k][e]) & 0x7FFFFFFFu);
+        } else if (live) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[k][e] = x2 ? swiglu_value(x[at + e], x2[at + e]) : x[at + e];
         }
-    }
-    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
-    const int ex = (int)(mx >> 23);
-    const int e2 = (mx == 0u || ex == 255) ? 0 : 14 - (ex - 127);
-    if (lane == 0) {
-        xp_exp[(tile * bpr + blk) * 16u + t] = e2;
-        if (half) xp_exp[(tile * bpr + blk) * 16u + t + 8u] = e2;
     }
 #pragma unroll
-    for (int k = 0; k < 2; ++k) {
-        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
-        const float s0 = ldexpf(v[k][0], e2), s1 = ldexpf(v[k][1], e2);
-        const auto ph = __builtin_amdgcn_cvt_pkrtz(s0, s1);           // x = xh + xl, both FP16 (round toward zero)
-        const auto pl = __builtin_amdgcn_cvt_pkrtz(s0 - (float)ph[0], s1 - (float)ph[1]);
-        uint32_t* o = xp + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (c & 3u);     // piece 0 of lane 16 kq + t, element c & 3
-        if (half) {
-            o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
-            o[(size_t)(c >> 2) * 256u + 32u] = __builtin_bit_cast(uint32_t, pl);                   // lane 16 kq + t + 8
-        } else {
-            o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
-            o[(size_t)(4u + (c >> 2)) * 256u] = __builtin_bit_cast(uint32_t, pl);
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t t = t_lo + wave + 4u * (uint32_t)k;
+        if (t >= t_hi) break;
+        if ((lane & 15u) == 15u) v[k][3] = 0.0f;                           // column 64 n + 63: no weight there
+        uint32_t mx = 0u;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mx = max(mx, __float_as_uint(v[k][e]) & 0x7FFFFFFFu);
+        for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
+        const int ex = (int)(mx >> 23);
+        const int e2 = (mx == 0u || ex == 255) ? 0 : 14 - (ex - 127);
+        if (lane == 0) {
+            xp_exp[(tile * bpr + blk) * 16u + t] = e2;
+            if (half) xp_exp[(tile * bpr + blk) * 16u + t + 8u] = e2;
         }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t i = 4u * lane + (uint32_t)e, pn = 4u + i - (i >> 6);
+            if ((i & 63u) != 63u) park[((pn >> 5) * 16u + t) * 36u + (pn & 31u)] = ldexpf(v[k][e], e2);
+        }
+        if (lane < 4u) park[t * 36u + lane] = 0.0f;                        // nibbles 0..3 (chunk 0)
+    }
+    __syncthreads();
+    // ---- a thread takes 8 consecutive nibble positions of one token column: four FP16 pairs of high parts
+    // (x = xh + xl, both FP16, round toward zero) and four of low parts, 16 bytes each.  Piece j (dwords 4j .. 4j+3 of a
+    // lane's 32) of lanes 16 kq + t is one contiguous KB, written here by 64 neighbouring threads -------------------
+    const uint32_t nt = t_hi - t_lo;
+    for (uint32_t task = tid; task < 32u * nt; task += 256u) {
+        const uint32_t t = t_lo + task % nt, kq = (task / nt) & 3u, jj = (task / (nt * 4u)) & 3u, h = task / (nt * 16u);
+        const float* p = park + ((kq + 4u * h) * 16u + t) * 36u + 8u * jj;
+        const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+        const float sv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        uint32_t hi[4], lo[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const float s0 = sv[2 * c], s1 = sv[2 * c + 1];
+            const auto ph = __builtin_amdgcn_cvt_pkrtz(s0, s1);
+            const auto pl = __builtin_amdgcn_cvt_pkrtz(s0 - (float)ph[0], s1 - (float)ph[1]);
+            hi[c] = __builtin_bit_cast(uint32_t, ph); lo[c] = __builtin_bit_cast(uint32_t, pl);
+        }
+        uint32_t* o = xp + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (size_t)jj * 256u;   // piece jj of lane 16 kq + t
+        *reinterpret_cast<uint4*>(o) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
+        *reinterpret_cast<uint4*>(o + (half ? 32u : 1024u)) = make_uint4(lo[0], lo[1], lo[2], lo[3]);   // lane + 8 of the piece, or piece 4 + jj
     }
 }
 
@@ -598,14 +642,16 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         hipLaunchKernelGGL(kern, dim3(slabs * ks), dim3(512), lds_bytes, s, t.d_payload, xp, xp_exp, y, (uint32_t)t.rows,
                            (uint32_t)t.cols, m0, m1, ld, groups / slabs, groups % slabs, ks, partial, counter, ordered ? 1 : 0, MultiJobs{});
     };
+    const int x_aligned = ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_x2)) & 15u) == 0 && (ldx & 3u) == 0;
     for (int m0 = 0; m0 < M;) {       // passes of 32 tokens while more than 16 are left, then one of 16 or of 8
         const int left = M - m0;
         const int kind = left <= 8 ? 0 : left <= 16 ? 1 : 2;
         const int m1 = left <= 32 ? M : m0 + 32;
         const uint32_t ksp = split_of(kind == 2 ? 8u : 16u);
         const bool two = ksp == 2u || (ksp > 2u && !ordered);              // row parts that add into y, which then starts at zero
-        hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
-                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
+        const uint32_t quarters = (kind == 2 ? 2u : 1u) * bpr < 128u ? 4u : 1u;
+        hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 2 ? 2u : 1u) * bpr * quarters), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
+                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, x_aligned, quarters, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
                            w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2, PackJobs{});
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, kind, m0, m1);
@@ -703,11 +749,12 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     if (xp_dwords * (size_t)nb > 0xFFFFFFFFull || part_floats * (size_t)njobs > 0xFFFFFFFFull || part_floats * 4u >= 0x100000000ull) return 1;
 
     // The launch as a whole fills the device about twice over, so that a workgroup keeps its table and its activations
-    // for many row groups.  A job's share of the workgroups follows its cost (a pass of 32 tokens costs 1.36 times a pass
-    // of 16, a pass of 8 tokens 0.87 times: measured on single tensors), so that all workgroups run about equally long;
-    // a job's count is a multiple of its K parts.
+    // for many row groups.  A job's share of the workgroups follows its cost, so that all workgroups run about equally
+    // long: a pass of 32 tokens counts 1.5 times a pass of 16 (1.36 on single tensors, where the fixed costs weigh
+    // more), a pass of 8 the same as one of 16 (0.87 on single tensors; shares below 1 only left workgroups that end
+    // late) -- the step time is flat within 1 % around these values.  A job's count is a multiple of its K parts.
     const uint32_t groups = ((uint32_t)w0.rows + 15u) / 16u;
-    static const double kCost[3] = {0.87, 1.0, 1.36};
+    static const double kCost[3] = {1.0, 1.0, 1.5};
     uint32_t ks[3];
     bool any_ordered_parts = false;
     double cost_sum = 0.0;
@@ -719,9 +766,11 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     const double total = 2.0 * (double)device_cu_count();
     MixedPlan plan{};
     for (int k = 0; k < 3; ++k) plan.ksplit[k] = ks[k];
+    const int x_aligned = ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_x2)) & 15u) == 0 && (ldx & 3u) == 0;
+    const uint32_t quarters = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb < 128u ? 4u : 1u;
     PackJobs pj{};
     pj.n = (uint32_t)nb;
-    pj.wgs_per_job = tokens_of(present[2] ? 2 : present[1] ? 1 : 0) * ((bpr + 3u) / 4u);
+    pj.wgs_per_job = (present[2] ? 2u : 1u) * bpr * quarters;
     pj.use_list = list ? 1 : 0;
     for (int i = 0; i < nlist; ++i) pj.list[i] = list[i];
     MultiJobs mj{};
@@ -754,7 +803,7 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     if (any_ordered_parts && ordered && !counters_clean)                  // the caller's workspace is not known to be zero
         hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
     hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
-                       (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
+                       (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, x_aligned, quarters, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
     OILHIP_HIP(hipGetLastError());
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;
     if (nkinds == 1) {
