@@ -738,6 +738,7 @@ def main():
     ap.add_argument("--no-extra", action="store_true", help="skip the secondary shapes")
     ap.add_argument("--kv-only", action="store_true", help="only run the KV-cache leg (for profiling its kernels)")
     ap.add_argument("--prefill-only", action="store_true", help="only run the prefill GEMM leg (for profiling its kernels)")
+    ap.add_argument("--moe-only", action="store_true", help="only run the MoE step leg (for profiling its kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run plain 1 GiB device copies (reference for the FETCH_SIZE/WRITE_SIZE counters)")
     args = ap.parse_args()
@@ -756,6 +757,9 @@ def main():
     log(f"device: {info['name']} gfx{info['gfx']} {info['compute_units']} CUs")
     if args.kv_only:
         print(json.dumps({"kv_cache_leg": bench_kv_cache(torch, ia, with_cpu=not args.no_cpu)}), flush=True)
+        return
+    if args.moe_only:
+        print(json.dumps({"moe_leg": bench_moe(torch, ia)}), flush=True)
         return
     if args.prefill_only:
         payload, blocks = ia.block_codec.quantize_tensor(make_weights(ROWS, COLS, seed=20260803), ia.Format.OIL4)

@@ -92,9 +92,110 @@ struct PackJobs {
     int list[kMaxListed];
 };
 
+// Rows [m_lo, m_hi) of y (n floats each, ld apart) set to zero by `threads` threads of which this one is number `id`:
+// the threads are dealt over (row, 16-byte piece) so that all of them store, with one division per thread.
+__device__ __forceinline__ void clear_rows_2d(float* __restrict__ y, uint32_t n, uint32_t ld, int m_lo, int m_hi, uint32_t id, uint32_t threads) {
+    if (!y) return;
+    const bool vec = ((reinterpret_cast<uintptr_t>(y) & 15u) | (n & 3u) | (ld & 3u)) == 0u;
+    const uint32_t per_row = vec ? n >> 2 : n;                             // stores per row
+    const uint32_t lanes = per_row < threads ? per_row : threads;          // threads that share a row
+    const uint32_t rows_at_once = threads / lanes, slot = id / lanes, col = id - slot * lanes;
+    if (slot >= rows_at_once) return;
+    for (int mm = m_lo + (int)slot; mm < m_hi; mm += (int)rows_at_once)
+        for (uint32_t c = col; c < per_row; c += lanes) {
+            if (vec) *reinterpret_cast<float4*>(y + (size_t)mm * ld + 4u * c) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            else y[(size_t)mm * ld + c] = 0.0f;
+        }
+}
+
+// What both pre-pass kernels do first: a workgroup of a grouped launch finds its batch (activation rows, pass size,
+// place of the packed data), and the outputs that the main kernel's two row parts add into are cleared.  PARKED selects
+// the workgroup count of a batch.  Returns false for workgroups beyond the batch's own count.
+template <bool PARKED>
+__device__ __forceinline__ bool pack_prologue(uint32_t& bid, int& M, int& row0, int& half, uint32_t*& xp, int*& xp_exp, uint32_t cols, int m0,
+                                              float* yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* yc1, uint32_t yc1_rows, uint32_t yc1_ld,
+                                              const PackJobs& jobs) {
+    const uint32_t bpr = cols >> 8, tid = threadIdx.x;
+    if (jobs.n) {                                                          // workgroup -> (batch, index within the batch)
+        const uint32_t job = bid / jobs.wgs_per_job;
+        bid -= job * jobs.wgs_per_job;
+        M = jobs.M[job]; row0 = jobs.row0[job];
+        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
+        const uint32_t kind = jobs.kind[job];
+        half = kind == 0u ? 1 : 0;
+        for (int o = 0; o < 2; ++o) clear_rows_2d(o ? jobs.clear1[job] : jobs.clear0[job], jobs.clear_rows, jobs.clear_ld, 0, M, bid * 256u + tid, jobs.wgs_per_job * 256u);
+        // a smaller pass than the launch's largest: fewer workgroups
+        const uint32_t own = PARKED ? (kind == 2u ? 2u : 1u) * bpr : (kind == 0u ? 8u : kind == 1u ? 16u : 32u) * ((bpr + 3u) / 4u);
+        if (bid >= own) return false;
+    }
+    clear_rows_2d(yc0, yc0_rows, yc0_ld, m0, M, blockIdx.x * 256u + tid, gridDim.x * 256u);
+    clear_rows_2d(yc1, yc1_rows, yc1_ld, m0, M, blockIdx.x * 256u + tid, gridDim.x * 256u);
+    return true;
+}
+
+// Small launches (a single tensor, few blocks per row): a wavefront packs one block of one token column straight from
+// memory to memory -- the shortest chain of round trips, at the price of 4-byte stores that share their lines with
+// other workgroups.  Workgroup = 4 blocks of token column t of a tile.
+__global__ void __launch_bounds__(256)
+pack_x_cols_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
+                   int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half,
+                   float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld,
+                   const PackJobs jobs) {
+    const uint32_t bpr = cols >> 8, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t bid = blockIdx.x;
+    int row0 = 0;
+    uint32_t* xq = xp;
+    int* xe = xp_exp;
+    if (!pack_prologue<false>(bid, M, row0, half, xq, xe, cols, m0, yc0, yc0_rows, yc0_ld, yc1, yc1_rows, yc1_ld, jobs)) return;
+    const uint32_t ncol = half ? 8u : 16u, nbg = (bpr + 3u) / 4u;
+    const uint32_t blk = (bid % nbg) * 4u + wave, t = (bid / nbg) % ncol, tile = bid / (nbg * ncol);
+    if (blk >= bpr) return;
+    const int m = m0 + 16 * (int)tile + (int)t;
+    xq += (size_t)tile * bpr * 4096u;
+    uint32_t src = 0xFFFFFFFFu;
+    if (m < M) src = jobs.n ? (jobs.use_list ? (uint32_t)jobs.list[row0 + m] : (uint32_t)(row0 + m)) : (tok ? (uint32_t)tok[m] : (uint32_t)m);
+    const bool live = src < xrows;
+    const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u : 0;
+    // this lane's two pairs: pair id = lane + 64 k holds positions 2c, 2c+1 of chunk kq + 4h
+    float v[2][2] = {{0.0f, 0.0f}, {0.0f, 0.0f}};
+    uint32_t mx = 0u;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const uint32_t pn = 32u * (kq + 4u * h) + 2u * c + e;
+            if (live && pn >= 4u) {
+                const uint32_t q = pn - 4u, col = q + q / 63u;
+                v[k][e] = x2 ? swiglu_value(x[at + col], x2[at + col]) : x[at + col];
+            }
+            mx = max(mx, __float_as_uint(v[k][e]) & 0x7FFFFFFFu);
+        }
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = max(mx, (uint32_t)__shfl_xor((int)mx, o, 64));
+    const int ex = (int)(mx >> 23);
+    const int e2 = (mx == 0u || ex == 255) ? 0 : 14 - (ex - 127);
+    if (lane == 0) {
+        xe[(tile * bpr + blk) * 16u + t] = e2;
+        if (half) xe[(tile * bpr + blk) * 16u + t + 8u] = e2;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const uint32_t id = lane + 64u * k, c = id & 15u, kq = (id >> 4) & 3u, h = id >> 6;
+        const float s0 = ldexpf(v[k][0], e2), s1 = ldexpf(v[k][1], e2);
+        const auto ph = __builtin_amdgcn_cvt_pkrtz(s0, s1);           // x = xh + xl, both FP16 (round toward zero)
+        const auto pl = __builtin_amdgcn_cvt_pkrtz(s0 - (float)ph[0], s1 - (float)ph[1]);
+        uint32_t* o = xq + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (c & 3u);     // piece 0 of lane 16 kq + t, element c & 3
+        o[(size_t)(c >> 2) * 256u] = __builtin_bit_cast(uint32_t, ph);
+        o[(size_t)(c >> 2) * 256u + (half ? 32u : 1024u)] = __builtin_bit_cast(uint32_t, pl);      // lane 16 kq + t + 8, or piece 4 + (c >> 2)
+    }
+}
+
+// Bulk launches (the batches of a mixture-of-experts step, wide rows): a workgroup parks a block's scaled activations for
+// all token columns of a tile in LDS and writes whole 1 KB operand pieces.
 __global__ void __launch_bounds__(256)
 pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const int* __restrict__ tok, uint32_t* __restrict__ xp,
-              int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half, int aligned, uint32_t quarters,
+              int* __restrict__ xp_exp, uint32_t cols, int m0, int M, uint32_t ldx, uint32_t xrows, int half, int aligned,
               float* __restrict__ yc0, uint32_t yc0_rows, uint32_t yc0_ld, float* __restrict__ yc1, uint32_t yc1_rows, uint32_t yc1_ld,
               const PackJobs jobs) {
     // scaled activations of the workgroup's block, by nibble position: row (chunk of 32 positions, token column), 36
@@ -103,47 +204,16 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
     const uint32_t bpr = cols >> 8, tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     uint32_t bid = blockIdx.x;
     int row0 = 0;
-    if (jobs.n) {                                                          // workgroup -> (batch, index within the batch)
-        const uint32_t job = bid / jobs.wgs_per_job;
-        bid -= job * jobs.wgs_per_job;
-        M = jobs.M[job]; row0 = jobs.row0[job];
-        xp += jobs.xp_off[job]; xp_exp += jobs.exp_off[job];
-        const uint32_t kind = jobs.kind[job];
-        half = kind == 0u ? 1 : 0;
-        // outputs of the batch that two row parts add into start at zero
-        const uint32_t crows = jobs.clear_rows, cld = jobs.clear_ld, cstep = jobs.wgs_per_job * 256u;
-        for (int o = 0; o < 2; ++o) {
-            float* yc = o ? jobs.clear1[job] : jobs.clear0[job];
-            if (!yc) continue;
-            if (((reinterpret_cast<uintptr_t>(yc) & 15u) | (crows & 3u) | (cld & 3u)) == 0u) {
-                for (int mm = 0; mm < M; ++mm)
-                    for (uint32_t r = (bid * 256u + tid) * 4u; r < crows; r += cstep * 4u)
-                        *reinterpret_cast<float4*>(yc + (size_t)mm * cld + r) = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            } else {
-                for (int mm = 0; mm < M; ++mm)
-                    for (uint32_t r = bid * 256u + tid; r < crows; r += cstep) yc[(size_t)mm * cld + r] = 0.0f;
-            }
-        }
-        if (bid >= (kind == 2u ? 2u : 1u) * bpr * quarters) return;        // one token tile where the launch's largest pass has two
-    }
-    // outputs that the main kernel's two row parts add into start at zero
-    const uint32_t gid = blockIdx.x * 256u + tid, gn = gridDim.x * 256u;
-    if (yc0)
-        for (int mm = m0; mm < M; ++mm)
-            for (uint32_t r = gid; r < yc0_rows; r += gn) yc0[(size_t)mm * yc0_ld + r] = 0.0f;
-    if (yc1)
-        for (int mm = m0; mm < M; ++mm)
-            for (uint32_t r = gid; r < yc1_rows; r += gn) yc1[(size_t)mm * yc1_ld + r] = 0.0f;
+    uint32_t* xq = xp;
+    int* xe = xp_exp;
+    if (!pack_prologue<true>(bid, M, row0, half, xq, xe, cols, m0, yc0, yc0_rows, yc0_ld, yc1, yc1_rows, yc1_ld, jobs)) return;
     // workgroup = one block of the row for the 16 token columns of a tile (a pass of 32 tokens is two tiles of 16, the
     // second one's data behind the first's); passes of 8 tokens have 8 token columns: columns 0..7 of the operand
     // carry their high parts and columns 8..15 their low parts, in the pieces that otherwise hold the high parts of 16
-    // tokens.  quarters = 4 (small launches): a workgroup takes a quarter of the token columns, one per wavefront, so
-    // that four times as many workgroups share the launch's round trips
+    // tokens
     const uint32_t ncol = half ? 8u : 16u;
-    const uint32_t tq = bid % quarters, blk = (bid / quarters) % bpr, tile = bid / (quarters * bpr);
-    const uint32_t t_lo = quarters == 4u ? 4u * tq : 0u, t_hi = quarters == 4u ? t_lo + 4u : ncol;
-    if (t_lo >= ncol) return;
-    xp += (size_t)tile * bpr * 4096u;
+    const uint32_t blk = bid % bpr, tile = bid / bpr;
+    xq += (size_t)tile * bpr * 4096u;
     // ---- a wavefront takes one token column at a time: 256 columns of x as one 16-byte load per lane, the largest
     // magnitude of the 252 that carry a weight, the power of two that brings it to [2^14, 2^15), the scaled values
     // parked by nibble position (column i of the block sits at nibble 4 + i - i/64; columns 63, 127, 191, 255 meet the
@@ -151,10 +221,10 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
     float v[4][4];                                                         // [token column of this wavefront][column of the lane]
 #pragma unroll
     for (int k = 0; k < 4; ++k) {                                          // all loads first: one round trip for the wavefront's columns
-        const uint32_t t = t_lo + wave + 4u * (uint32_t)k;
+        const uint32_t t = wave + 4u * (uint32_t)k;
         const int m = m0 + 16 * (int)tile + (int)t;
         uint32_t src = 0xFFFFFFFFu;
-        if (t < t_hi && m < M)
+        if (t < ncol && m < M)
             src = jobs.n ? (jobs.use_list ? (uint32_t)jobs.list[row0 + m] : (uint32_t)(row0 + m)) : (tok ? (uint32_t)tok[m] : (uint32_t)m);
         const bool live = src < xrows;
         const size_t at = live ? (size_t)src * ldx + (size_t)blk * 256u + 4u * lane : 0;
@@ -175,8 +245,8 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
     }
 #pragma unroll
     for (int k = 0; k < 4; ++k) {
-        const uint32_t t = t_lo + wave + 4u * (uint32_t)k;
-        if (t >= t_hi) break;
+        const uint32_t t = wave + 4u * (uint32_t)k;
+        if (t >= ncol) break;
         if ((lane & 15u) == 15u) v[k][3] = 0.0f;                           // column 64 n + 63: no weight there
         uint32_t mx = 0u;
 #pragma unroll
@@ -185,8 +255,8 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
         const int ex = (int)(mx >> 23);
         const int e2 = (mx == 0u || ex == 255) ? 0 : 14 - (ex - 127);
         if (lane == 0) {
-            xp_exp[(tile * bpr + blk) * 16u + t] = e2;
-            if (half) xp_exp[(tile * bpr + blk) * 16u + t + 8u] = e2;
+            xe[(tile * bpr + blk) * 16u + t] = e2;
+            if (half) xe[(tile * bpr + blk) * 16u + t + 8u] = e2;
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
@@ -199,9 +269,8 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
     // ---- a thread takes 8 consecutive nibble positions of one token column: four FP16 pairs of high parts
     // (x = xh + xl, both FP16, round toward zero) and four of low parts, 16 bytes each.  Piece j (dwords 4j .. 4j+3 of a
     // lane's 32) of lanes 16 kq + t is one contiguous KB, written here by 64 neighbouring threads -------------------
-    const uint32_t nt = t_hi - t_lo;
-    for (uint32_t task = tid; task < 32u * nt; task += 256u) {
-        const uint32_t t = t_lo + task % nt, kq = (task / nt) & 3u, jj = (task / (nt * 4u)) & 3u, h = task / (nt * 16u);
+    for (uint32_t task = tid; task < 32u * ncol; task += 256u) {
+        const uint32_t t = task % ncol, kq = (task / ncol) & 3u, jj = (task / (ncol * 4u)) & 3u, h = task / (ncol * 16u);
         const float* p = park + ((kq + 4u * h) * 16u + t) * 36u + 8u * jj;
         const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
         const float sv[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
@@ -213,7 +282,7 @@ pack_x_kernel(const float* __restrict__ x, const float* __restrict__ x2, const i
             const auto pl = __builtin_amdgcn_cvt_pkrtz(s0 - (float)ph[0], s1 - (float)ph[1]);
             hi[c] = __builtin_bit_cast(uint32_t, ph); lo[c] = __builtin_bit_cast(uint32_t, pl);
         }
-        uint32_t* o = xp + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (size_t)jj * 256u;   // piece jj of lane 16 kq + t
+        uint32_t* o = xq + ((size_t)(blk * 2u + h) * 8u * 64u + 16u * kq + t) * 4u + (size_t)jj * 256u;   // piece jj of lane 16 kq + t
         *reinterpret_cast<uint4*>(o) = make_uint4(hi[0], hi[1], hi[2], hi[3]);
         *reinterpret_cast<uint4*>(o + (half ? 32u : 1024u)) = make_uint4(lo[0], lo[1], lo[2], lo[3]);   // lane + 8 of the piece, or piece 4 + jj
     }
@@ -649,9 +718,13 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         const int m1 = left <= 32 ? M : m0 + 32;
         const uint32_t ksp = split_of(kind == 2 ? 8u : 16u);
         const bool two = ksp == 2u || (ksp > 2u && !ordered);              // row parts that add into y, which then starts at zero
-        const uint32_t quarters = (kind == 2 ? 2u : 1u) * bpr < 128u ? 4u : 1u;
-        hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 2 ? 2u : 1u) * bpr * quarters), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
-                           (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, x_aligned, quarters, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
+        if ((kind == 2 ? 2u : 1u) * bpr < 128u)
+            hipLaunchKernelGGL(pack_x_cols_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
+                               (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
+                           w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2, PackJobs{});
+        else
+            hipLaunchKernelGGL(pack_x_kernel, dim3((kind == 2 ? 2u : 1u) * bpr), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
+                               (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, x_aligned, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
                            w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2, PackJobs{});
         OILHIP_HIP(hipGetLastError());
         main_launch(w, d_y, ldy, kind, m0, m1);
@@ -767,10 +840,10 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     MixedPlan plan{};
     for (int k = 0; k < 3; ++k) plan.ksplit[k] = ks[k];
     const int x_aligned = ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_x2)) & 15u) == 0 && (ldx & 3u) == 0;
-    const uint32_t quarters = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb < 128u ? 4u : 1u;
+    const bool parked = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb >= 128u;   // else the memory-to-memory pre-pass of small launches
     PackJobs pj{};
     pj.n = (uint32_t)nb;
-    pj.wgs_per_job = (present[2] ? 2u : 1u) * bpr * quarters;
+    pj.wgs_per_job = parked ? (present[2] ? 2u : 1u) * bpr : tokens_of(present[2] ? 2 : present[1] ? 1 : 0) * ((bpr + 3u) / 4u);
     pj.use_list = list ? 1 : 0;
     for (int i = 0; i < nlist; ++i) pj.list[i] = list[i];
     MultiJobs mj{};
@@ -802,8 +875,12 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     const uint32_t wgs_total = mj.wg_begin[njobs];
     if (any_ordered_parts && ordered && !counters_clean)                  // the caller's workspace is not known to be zero
         hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
-    hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
-                       (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, x_aligned, quarters, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
+    if (parked)
+        hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
+                           (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, x_aligned, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
+    else
+        hipLaunchKernelGGL(pack_x_cols_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
+                           (uint32_t)w0.cols, 0, 0, ldx, xrows, 0, (float*)nullptr, 0u, 0u, (float*)nullptr, 0u, 0u, pj);
     OILHIP_HIP(hipGetLastError());
     const size_t lds_bytes = (size_t)kRedBase + kRedBytes + kGemvPackExpBytes + 64;
     if (nkinds == 1) {
