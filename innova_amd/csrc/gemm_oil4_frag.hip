@@ -10,18 +10,27 @@
 //  * Activations never pass through LDS.  A pre-pass writes X' in the order the matrix instruction wants its
 //    A operand: [32-token block][16-column group][lane][8 bf16], columns in nibble order (the 4-bit index of
 //    weight i of a 256-weight block sits at nibble 4 + i - i/64; nibbles 0..3 are the FP16 scale and meet
-//    zeros in X').  A fragment is then one coalesced 1 KB load straight into registers, issued one 64-column
-//    step ahead.
-//  * Weights: a lane loads 16 bytes (32 nibbles) of one weight row per step, turns every packed byte into two
-//    FP32 levels through the byte -> (level, level) pair table in LDS (the table of the decode GEMV), multiplies
-//    by the block's FP16 scale, rounds once to bf16 and stores the result in B-operand fragment order.  Each
-//    weight is decoded once per workgroup; the four wavefronts read the fragments back with conflict-free
-//    16-byte LDS reads.  Two tile buffers, one workgroup barrier per step: the fragments of step s are read
-//    and the tile of step s + 1 is written between the same two barriers, and the decode is cut into four
-//    quarters that ride behind the four groups of matrix instructions of a step.
-//  * Tiles that do not fill a whole round of compute units are cut in two along K (two addends into a zeroed Y:
-//    the sum does not depend on their order); tile order keeps the workgroups of one XCD on few token blocks and
-//    neighbouring weight rows so that its L2 serves most of their reads.
+//    zeros in X').  A fragment is then one coalesced 1 KB load straight into registers, issued two 64-column
+//    steps ahead through a buffer resource (the scalar offset of a step is clamped on the host side of the loop:
+//    the hardware does not range-check it).
+//  * Weights: a lane loads 16 bytes (32 nibbles) of one weight row per step, four steps ahead.  Every packed byte
+//    becomes an LDS address (v_perm_b32) into a 64 KB table whose row v holds 64 lane-private copies of the FP16 pair
+//    (level[v & 15], level[v >> 4]); a 4-byte read returns both levels, v_fma_mix_f32 multiplies each by the block's
+//    FP16 scale in FP32, one v_cvt_pk_bf16_f32 rounds the pair, and 16-byte stores put the result in B-operand
+//    fragment order.  Each weight is decoded once per workgroup; the four wavefronts read the fragments back with
+//    conflict-free 16-byte LDS reads.  Two tile buffers, one workgroup barrier per step: the fragments of step s
+//    are read and the tile of step s + 1 is written between the same two barriers.
+//  * Issue order is fixed by hand.  A 32x32x16 matrix instruction keeps the wavefront's issue port for half of its
+//    32 cycles, which leaves four slots for other instructions; the decode of a step is cut into quarters of three
+//    stages (addresses, table reads, multiply/round/store) that ride in those slots behind the four groups of sixteen
+//    matrix instructions of a step, every side instruction at a fixed place (a scheduling barrier after each
+//    matrix instruction), fragment re-reads after the last use of a register, A loads after the group's last
+//    matrix instruction.
+//  * A shape whose tiles do not fill whole rounds of compute units runs its last round as half tiles: 256 tokens x
+//    128 rows with all of K (no partial sums) for the 256 x 256 tiling; two K halves added into a zeroed Y with
+//    float atomics (two addends: the sum does not depend on their order) for the 128 x 128 tiling.  Tile order
+//    keeps the workgroups of one XCD on few token blocks and neighbouring weight rows so that its L2 serves most of
+//    their reads.
 #include <hip/hip_fp16.h>
 
 #include <algorithm>
