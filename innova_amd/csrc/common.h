@@ -122,7 +122,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
                            size_t pack_cap = 0);
 void g_ordered_sums_set(int v);
 // several batches of one tensor shape in one launch (gemv_oil4_multi.hip); kinds[b] = 0 / 1 / 2: batch b holds up to 8 / 16 / 32 rows
-size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols);
+size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols, bool two_tensors);   // two_tensors: every batch goes through wa[b] and wb[b]
 int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,

@@ -765,10 +765,10 @@ size_t job_partial_floats(uint32_t bpr, uint64_t rows) {
 }
 }  // namespace
 
-size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols) {
+size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols, bool two_tensors) {
     const uint32_t bpr = (uint32_t)(cols >> 8);
     const size_t per_batch = (size_t)2 * bpr * 16384u + (size_t)2 * bpr * 64u;
-    return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)2 * nb * job_partial_floats(bpr, rows) * 4u + 256u;
+    return kBatchCounterBytes + (size_t)nb * per_batch + (size_t)(two_tensors ? 2 : 1) * nb * job_partial_floats(bpr, rows) * 4u + 256u;
 }
 
 // Whether a grouped launch with passes of this size over tensors with rows of `cols` weights adds partial sums into its
@@ -794,7 +794,7 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || nlist > kMaxListed) return 1;
     const oilhip_weights& w0 = *wa[0];
     if (w0.rows == 0 || w0.rows > 0x7FFFFFFFull || w0.cols > kMaxPackCols || (w0.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
-    if (ws_bytes < gemv_oil4_multi_batches_bytes(nb, w0.rows, w0.cols)) return 1;
+    if (ws_bytes < gemv_oil4_multi_batches_bytes(nb, w0.rows, w0.cols, wb != nullptr)) return 1;
     static std::atomic<uint64_t> attr_done[4];
     if (int rc = ensure_max_lds(attr_done[0], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 1>), kMaxLds)) return rc;
     if (int rc = ensure_max_lds(attr_done[1], reinterpret_cast<const void*>(gemv_oil4_multi_kernel<false, 2>), kMaxLds)) return rc;

@@ -131,7 +131,7 @@ constexpr int kChunk = 16;      // expert batches per grouped launch (gate and u
 
 // scratch of one grouped launch: the larger of the gate/up side (rows F, cols D) and the down side (rows D, cols F)
 size_t batch_scratch_bytes(int64_t D, int64_t F) {
-    return std::max(gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)F, (uint64_t)D), gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)D, (uint64_t)F));
+    return std::max(gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)F, (uint64_t)D, true), gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)D, (uint64_t)F, false));
 }
 
 Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
