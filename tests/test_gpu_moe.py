@@ -56,6 +56,7 @@ def test_dispatch_matches_reference_fixture():
                                              (40, 2, 2, 256, 512, (3, 3, 3)),        # > 16 tokens per expert: several passes
                                              (12, 8, 2, 256, 512, (3, 3, 3)),        # a few tokens per expert: passes of 8 only
                                              (50, 6, 2, 256, 512, (3, 3, 3)),        # passes of 32, 16 and 8 side by side in one launch
+                                             (30, 20, 2, 256, 12288, (3, 3, 3)),     # twenty batches: two grouped launches per side over one workspace; rows cut in three
                                              (9, 3, 1, 256, 512, (4, 10, 1))])       # OIL8 / OIL4_GRP / SPARK_Q0: general kernel
 def test_dispatch_against_oracle(T, E, K, D, F, fmts):
     packs, dense = MF.moe_experts(5 + T, E, D, F, fmts)
