@@ -126,7 +126,10 @@ size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols, bool 
 int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
-                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean = false);
+                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean = false,
+                                   float* d_parts = nullptr, uint32_t parts_rows = 0);
+uint32_t gemv_oil4_multi_parts(int kind, uint64_t cols);
+bool gemv_oil4_multi_ordered();
 // clears the slab counters at the start of a batch workspace; launches over it may then be told that they are clean
 constexpr size_t kGemvBatchCounterBytes = 32u * 4096u;   // slab counters at the start of a batch workspace: a 4 KB page per job
 int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s);

@@ -486,7 +486,9 @@ int launch_frag(const oilhip_weights& w, const void* d_x, float* d_y, uint32_t M
 int launch_gemm_oil4_frag(const oilhip_weights& w, const void* d_x, bool x_is_f32, float* d_y, int M, hipStream_t s) {
     if (w.rows > 0x7FFFFFFFull || w.cols > 0x7FFFFFFFull) return fail(OILHIP_E_ARG, "matrix too large for the prefill kernel");
     const uint32_t N = (uint32_t)w.rows, K = (uint32_t)w.cols, cus = (uint32_t)device_cu_count();
-    if ((uint64_t)256 * (K >> 8) * 128u >= 0x80000000ull) return fail(OILHIP_E_ARG, "rows too wide for the prefill kernel");
+    // 32-bit byte offsets inside a workgroup's 256 weight rows and inside a wavefront's four token blocks of X'
+    if ((uint64_t)256 * (K >> 8) * 128u >= 0x80000000ull || (uint64_t)K * 256u >= 0x80000000ull)
+        return fail(OILHIP_E_ARG, "rows too wide for the prefill kernel");
     // 256 x 256 tiles unless they would leave three quarters of the compute units without work even when cut along K
     const uint32_t big_tiles = (((uint32_t)M + 255u) / 256u) * ((N + 255u) / 256u);
     const bool small = big_tiles * 4u <= cus;

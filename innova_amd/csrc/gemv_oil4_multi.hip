@@ -300,6 +300,7 @@ struct MultiJobs {
     uint32_t n;
     uint32_t wg_begin[kMaxJobs + 1];   // job j runs workgroups [wg_begin[j], wg_begin[j + 1]): as many as its share of the launch's work
     uint32_t g_base[kMaxJobs], g_rem[kMaxJobs];   // row groups per slab of the job: g_base, and one more for the first g_rem slabs
+    uint32_t pstride;                  // floats between two K parts of one output row when the parts are left for a later launch to sum
     const uint8_t* W[kMaxJobs];
     float* y[kMaxJobs];
     int M[kMaxJobs];
@@ -310,7 +311,7 @@ template <bool HALF, int NT>
 __device__ __forceinline__ void
 multi_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const int* __restrict__ xp_exp, float* __restrict__ y,
            uint32_t rows, uint32_t cols, int m0, int M, uint32_t ldy, uint32_t g_base, uint32_t g_rem,
-           uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, uint32_t bid) {
+           uint32_t ksplit, float* __restrict__ partial, uint32_t* __restrict__ counter, int ordered, uint32_t pstride, uint32_t bid) {
     extern __shared__ __align__(16) uint8_t lds[];
     float* tab = reinterpret_cast<float*>(lds);                            // 64 KB pair table, built once
     float* red = reinterpret_cast<float*>(lds + kRedBase);                 // [8 waves][kGroups][kRedTile]
@@ -514,13 +515,14 @@ multi_body(const uint8_t* __restrict__ W, const uint32_t* __restrict__ xp, const
                 }
                 if (ksplit == 2u || (ksplit > 2u && !ordered)) unsafeAtomicAdd(y + (size_t)(m0 + jj) * ldy + r, s);
                 else if (ksplit > 2u)
-                    __hip_atomic_store(&partial[((size_t)part * (uint32_t)(M - m0) + jj) * rows + r], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (ordered == 2) partial[(size_t)part * pstride + (size_t)jj * rows + r] = s;   // summed by a later launch
+                    else __hip_atomic_store(&partial[((size_t)part * (uint32_t)(M - m0) + jj) * rows + r], s, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 else y[(size_t)(m0 + jj) * ldy + r] = s;
             }
         }
         if (tile + 1 < ntiles) __syncthreads();                            // red is rewritten by the next tile
     }
-    if (ksplit <= 2u || !ordered) return;
+    if (ksplit <= 2u || ordered != 1) return;                              // (ordered == 2: the parts are summed by the caller's next launch)
     // ---- rows cut into three or more parts: the last workgroup of the slab adds the parts in ascending order, so the result does
     // not depend on the order in which workgroups run.  The parts' sums are written and read with device-scope
     // accesses that go through to memory (no cache of another XCD can hold a stale copy), so no cache-wide write-back
@@ -591,9 +593,12 @@ gemv_oil4_multi_kernel(const uint8_t* __restrict__ W, const uint32_t* __restrict
         partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
         g_base = jobs.g_base[job]; g_rem = jobs.g_rem[job];
     }
-    multi_body<HALF, NT>(W, xp, xp_exp, y, rows, cols, m0, M, ldy, g_base, g_rem, ksplit, partial, counter, ordered, bid);
+    multi_body<HALF, NT>(W, xp, xp_exp, y, rows, cols, m0, M, ldy, g_base, g_rem, ksplit, partial, counter, ordered, jobs.pstride, bid);
 }
 
+// `ordered` in these kernels: 0 = three or more K parts add into y with atomics, 1 = the parts meet in `partial` and the
+// workgroup that arrives last sums them in ascending order, 2 (grouped launches only) = the parts are stored at
+// partial[part * pstride + token * rows + row] and left for the caller's next launch to sum in ascending order.
 // Batches of different pass sizes in one launch: the job's pass size selects the body, and with it the number of K
 // parts (a job's workgroup count is a multiple of it).
 struct MixedPlan {
@@ -615,11 +620,11 @@ gemv_oil4_multi_mixed_kernel(const uint32_t* __restrict__ xp, const int* __restr
     partial += jobs.partial_off[job]; counter += jobs.counter_off[job];
     const uint32_t kind = plan.kind[job];                                   // workgroup-uniform
     if (kind == 0u)
-        multi_body<true, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[0], partial, counter, ordered, bid);
+        multi_body<true, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[0], partial, counter, ordered, jobs.pstride, bid);
     else if (kind == 1u)
-        multi_body<false, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[1], partial, counter, ordered, bid);
+        multi_body<false, 1>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[1], partial, counter, ordered, jobs.pstride, bid);
     else
-        multi_body<false, 2>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[2], partial, counter, ordered, bid);
+        multi_body<false, 2>(W, xp, xp_exp, y, rows, cols, 0, M, ldy, g_base, g_rem, plan.ksplit[2], partial, counter, ordered, jobs.pstride, bid);
 }
 
 
@@ -765,6 +770,10 @@ size_t job_partial_floats(uint32_t bpr, uint64_t rows) {
 }
 }  // namespace
 
+// K parts of a row of `cols` weights for a pass size (1: the row is not cut)
+uint32_t gemv_oil4_multi_parts(int kind, uint64_t cols) { return parts_of(kind, (uint32_t)(cols >> 8)); }
+bool gemv_oil4_multi_ordered() { return g_ordered_sums.load(std::memory_order_relaxed) != 0; }
+
 size_t gemv_oil4_multi_batches_bytes(int nb, uint64_t rows, uint64_t cols, bool two_tensors) {
     const uint32_t bpr = (uint32_t)(cols >> 8);
     const size_t per_batch = (size_t)2 * bpr * 16384u + (size_t)2 * bpr * 64u;
@@ -790,7 +799,8 @@ int zero_gemv_oil4_multi_batch_counters(void* d_ws, hipStream_t s) {
 int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weights* const* wa, float* const* ya,
                                    const oilhip_weights* const* wb, float* const* yb, const int* M, const int* row0,
                                    const int* list, int nlist, const float* d_x, const float* d_x2, uint32_t ldx, uint32_t xrows,
-                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean) {
+                                   uint32_t ldy, void* d_ws, size_t ws_bytes, hipStream_t s, bool counters_clean, float* d_parts,
+                                   uint32_t parts_rows) {
     if (nb < 1 || nb > kMaxJobs / (wb ? 2 : 1) || nlist > kMaxListed) return 1;
     const oilhip_weights& w0 = *wa[0];
     if (w0.rows == 0 || w0.rows > 0x7FFFFFFFull || w0.cols > kMaxPackCols || (w0.cols & 255u) || (uint64_t)xrows * ldx > 0x1FFFFFFFull) return 1;
@@ -839,6 +849,10 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     const double total = 2.0 * (double)device_cu_count();
     MixedPlan plan{};
     for (int k = 0; k < 3; ++k) plan.ksplit[k] = ks[k];
+    // d_parts: batch b's three or more K parts go to d_parts[part * parts_rows * rows + (row0[b] + m) * rows + r] and
+    // are summed by the caller (one tensor per batch only: two would share the rows)
+    const bool leave_parts = d_parts && ordered && any_ordered_parts && !wb;
+    if (leave_parts && (uint64_t)parts_rows * w0.rows * std::max(ks[0], std::max(ks[1], ks[2])) > 0xFFFFFFFFull) return 1;
     const int x_aligned = ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_x2)) & 15u) == 0 && (ldx & 3u) == 0;
     const bool parked = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb >= 128u;   // else the memory-to-memory pre-pass of small launches
     PackJobs pj{};
@@ -860,7 +874,8 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
             if (!plain_oil4(*w) || w->rows != w0.rows || w->cols != w0.cols) return 1;
             mj.W[j] = w->d_payload; mj.y[j] = t ? yb[b] : ya[b]; mj.M[j] = M[b];
             mj.xp_off[j] = pj.xp_off[b]; mj.exp_off[j] = pj.exp_off[b];
-            mj.partial_off[j] = (uint32_t)(j * part_floats); mj.counter_off[j] = (uint32_t)(j * 1024);
+            mj.partial_off[j] = leave_parts ? (uint32_t)((uint64_t)row0[b] * w0.rows) : (uint32_t)(j * part_floats);
+            mj.counter_off[j] = (uint32_t)(j * 1024);
             plan.kind[j] = (uint8_t)kinds[b];
             const uint32_t k = ks[kinds[b]];
             uint32_t slabs = (uint32_t)(total * kCost[kinds[b]] / cost_sum / (double)k);   // rounded down: one workgroup past two rounds costs a third
@@ -873,7 +888,10 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     }
     for (int j = 0; j < njobs; ++j) mj.wg_begin[j + 1] = mj.wg_begin[j] + job_slabs[j] * ks[plan.kind[j]];
     const uint32_t wgs_total = mj.wg_begin[njobs];
-    if (any_ordered_parts && ordered && !counters_clean)                  // the caller's workspace is not known to be zero
+    mj.pstride = leave_parts ? (uint32_t)((uint64_t)parts_rows * w0.rows) : 0u;
+    if (leave_parts) partial = d_parts;
+    const int mode = !ordered ? 0 : leave_parts ? 2 : 1;
+    if (any_ordered_parts && ordered && !counters_clean && !leave_parts)  // the caller's workspace is not known to be zero
         hipLaunchKernelGGL(zero_words_kernel, dim3((uint32_t)njobs * 4u), dim3(256), 0, s, counter, (uint32_t)njobs * 1024u);
     if (parked)
         hipLaunchKernelGGL(pack_x_kernel, dim3(pj.wgs_per_job * (uint32_t)nb), dim3(256), 0, s, d_x, d_x2, (const int*)nullptr, xp, xp_exp,
@@ -886,10 +904,10 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     if (nkinds == 1) {
         auto kern = only == 0 ? gemv_oil4_multi_kernel<true, 1> : only == 1 ? gemv_oil4_multi_kernel<false, 1> : gemv_oil4_multi_kernel<false, 2>;
         hipLaunchKernelGGL(kern, dim3(wgs_total), dim3(512), lds_bytes, s, (const uint8_t*)nullptr, xp, xp_exp, (float*)nullptr,
-                           (uint32_t)w0.rows, (uint32_t)w0.cols, 0, 0, ldy, 0u, 0u, ks[only], partial, counter, ordered ? 1 : 0, mj);
+                           (uint32_t)w0.rows, (uint32_t)w0.cols, 0, 0, ldy, 0u, 0u, ks[only], partial, counter, mode, mj);
     } else {
         hipLaunchKernelGGL(gemv_oil4_multi_mixed_kernel, dim3(wgs_total), dim3(512), lds_bytes, s, xp, xp_exp, (uint32_t)w0.rows,
-                           (uint32_t)w0.cols, ldy, partial, counter, ordered ? 1 : 0, mj, plan);
+                           (uint32_t)w0.cols, ldy, partial, counter, mode, mj, plan);
     }
     OILHIP_HIP(hipGetLastError());
     return OILHIP_OK;

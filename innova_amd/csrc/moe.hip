@@ -91,13 +91,19 @@ __global__ void __launch_bounds__(256) combine_distinct_kernel(const float* __re
 constexpr int kMaxPairs = 448;
 struct CombineLists {
     int K;
-    int pair[kMaxPairs];        // pair[t * K + k]: row of o behind the k-th contribution of token t, or -1
+    int16_t pair[kMaxPairs];    // pair[t * K + k]: row of o behind the k-th contribution of token t, or -1
+    uint8_t nparts[kMaxPairs];  // nparts[row of o]: K parts of that row left in `parts` by the down projection (0: the row is in o)
     float wgt[kMaxPairs];       // its weight (<= 0: dropped)
 };
 
-// zacc == nullptr: the caller does not want the z-loss, and the workgroups skip their atomic on its one address
-__global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __restrict__ o, uint32_t D, float* __restrict__ out,
-                                                              double* __restrict__ zacc, const CombineLists L) {
+static_assert(sizeof(CombineLists) <= 3584, "the lists travel in the kernel arguments (4 KB with the other arguments)");
+
+// zacc == nullptr: the caller does not want the z-loss, and the workgroups skip their atomic on its one address.
+// Rows whose down projection was cut into three or more K parts arrive as those parts (parts[p * pstride + row * D + d])
+// and are summed here in ascending part order: the sum does not depend on the order in which workgroups ran.
+__global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __restrict__ o, const float* __restrict__ parts, uint32_t pstride,
+                                                              uint32_t D, float* __restrict__ out, double* __restrict__ zacc,
+                                                              const CombineLists L) {
     __shared__ double part[4];
     const uint32_t d = blockIdx.x * 256 + threadIdx.x, t = blockIdx.y;
     double z = 0.0;
@@ -107,7 +113,11 @@ __global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __res
             const int i = L.pair[t * L.K + k];
             const float w = L.wgt[t * L.K + k];
             if (i < 0 || !(w > 0.0f)) continue;
-            const float v = w * o[(size_t)i * D + d];
+            float y = 0.0f;
+            const uint32_t np = L.nparts[i];
+            if (np == 0u) y = o[(size_t)i * D + d];
+            for (uint32_t p = 0; p < np; ++p) y += parts[(size_t)p * pstride + (size_t)i * D + d];
+            const float v = w * y;
             sum += v;
             z += (double)v * (double)v;
         }
@@ -123,7 +133,7 @@ __global__ void __launch_bounds__(256) combine_grouped_kernel(const float* __res
 size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
 
 struct Workspace {
-    int* tok; float* wgt; float* g; float* u; float* o; float* xg; double* z; uint8_t* batch;
+    int* tok; float* wgt; float* g; float* u; float* o; float* xg; float* parts; double* z; uint8_t* batch;
     size_t bytes, batch_bytes;
 };
 
@@ -132,6 +142,13 @@ constexpr int kChunk = 16;      // expert batches per grouped launch (gate and u
 // scratch of one grouped launch: the larger of the gate/up side (rows F, cols D) and the down side (rows D, cols F)
 size_t batch_scratch_bytes(int64_t D, int64_t F) {
     return std::max(gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)F, (uint64_t)D, true), gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)D, (uint64_t)F, false));
+}
+
+// the most K parts a down projection (rows of F weights) is cut into, over the pass sizes; 0 when no pass size cuts it in three or more
+uint32_t down_parts_max(int64_t F) {
+    uint32_t m = 0;
+    for (int kind = 0; kind < 3; ++kind) m = std::max(m, gemv_oil4_multi_parts(kind, (uint64_t)F));
+    return m > 2u ? m : 0u;
 }
 
 Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
@@ -148,6 +165,8 @@ Workspace carve(void* base, int64_t pairs, int64_t D, int64_t F) {
     w.xg = (float*)take((size_t)pairs * D * 4);
     w.batch_bytes = (D % 256 == 0 && F % 256 == 0 && D <= 32768 && F <= 32768) ? batch_scratch_bytes(D, F) : 0;
     w.batch = take(w.batch_bytes);
+    // K parts of the down projections' outputs (rows of F weights cut into three or more parts), summed by the combine
+    w.parts = (float*)take(w.batch_bytes ? (size_t)down_parts_max(F) * pairs * D * 4 : 0);
     w.bytes = off;
     return w;
 }
@@ -262,6 +281,9 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         hipLaunchKernelGGL(fill_zero3_kernel, dim3(64), dim3(256), 0, s, ws.g, (size_t)0, (float*)ws.z, (size_t)2, (float*)ws.batch,
                            kGemvBatchCounterBytes / 4);
         OILHIP_HIP(hipGetLastError());
+        // down projections cut into three or more K parts leave the parts to the combine (ordered sums; with the
+        // atomic sums switched on they add into their outputs instead)
+        const bool parts_mode = gemv_oil4_multi_ordered() && down_parts_max(F) > 0u;
         struct Batch { int e, pair0, m, kind; };
         std::vector<Batch> batches;
         for (int pass = 2; pass >= 0; --pass)                     // the longest passes first: they end last
@@ -293,23 +315,28 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
                                                     (uint32_t)D, (uint32_t)T, (uint32_t)F, ws.batch, ws.batch_bytes, s, true);
             if (rc == 0)
                 rc = launch_gemv_oil4_multi_batches(nb, kd, wd, yo, nullptr, nullptr, Mb, r0, nullptr, 0, ws.g, ws.u,
-                                                    (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s, true);
+                                                    (uint32_t)F, (uint32_t)pairs, (uint32_t)D, ws.batch, ws.batch_bytes, s, true,
+                                                    parts_mode ? ws.parts : nullptr, (uint32_t)pairs);
             if (rc < 0) return rc;
             if (rc == 1) return fail(OILHIP_E_ARG, "moe_forward: the grouped launch refused a shape it was planned for");
         }
         CombineLists L{};
         L.K = (int)K;
         for (int64_t i = 0; i < T * K; ++i) { L.pair[i] = -1; L.wgt[i] = 0.0f; }
+        for (const Batch& B : batches) {
+            const uint32_t np = parts_mode ? gemv_oil4_multi_parts(B.kind, (uint64_t)F) : 0u;
+            for (int m = 0; m < B.m; ++m) L.nparts[B.pair0 + m] = (uint8_t)(np > 2u ? np : 0u);
+        }
         std::vector<int> filled((size_t)T, 0);
         for (int e = 0; e < E; ++e)                      // ascending expert, list order: the order of the reference's additions
             for (int i = begin[(size_t)e]; i < begin[(size_t)e + 1]; ++i) {
                 const int t = tok[(size_t)i];
-                L.pair[t * K + filled[(size_t)t]] = i;
+                L.pair[t * K + filled[(size_t)t]] = (int16_t)i;
                 L.wgt[t * K + filled[(size_t)t]] = wgt[(size_t)i];
                 filled[(size_t)t]++;
             }
-        hipLaunchKernelGGL(combine_grouped_kernel, dim3((uint32_t)((D + 255) / 256), (uint32_t)T), dim3(256), 0, s, ws.o, (uint32_t)D,
-                           d_out, z_loss ? ws.z : (double*)nullptr, L);
+        hipLaunchKernelGGL(combine_grouped_kernel, dim3((uint32_t)((D + 255) / 256), (uint32_t)T), dim3(256), 0, s, ws.o, ws.parts,
+                           (uint32_t)(pairs * D), (uint32_t)D, d_out, z_loss ? ws.z : (double*)nullptr, L);
         OILHIP_HIP(hipGetLastError());
         if (z_loss) {
             double z = 0.0;
