@@ -723,7 +723,7 @@ int launch_gemv_oil4_multi(const oilhip_weights& w, const float* d_x, const int*
         const int m1 = left <= 32 ? M : m0 + 32;
         const uint32_t ksp = split_of(kind == 2 ? 8u : 16u);
         const bool two = ksp == 2u || (ksp > 2u && !ordered);              // row parts that add into y, which then starts at zero
-        if ((kind == 2 ? 2u : 1u) * bpr < 128u)
+        if ((kind == 2 ? 2u : 1u) * bpr < 512u)
             hipLaunchKernelGGL(pack_x_cols_kernel, dim3((kind == 0 ? 8u : kind == 1 ? 16u : 32u) * ((bpr + 3u) / 4u)), dim3(256), 0, s, d_x, d_x2, d_tok, xp, xp_exp,
                                (uint32_t)w.cols, m0, m1, ldx, xrows, kind == 0 ? 1 : 0, two ? d_y : nullptr, (uint32_t)w.rows, ldy,
                            w2 && two ? d_y2 : nullptr, w2 ? (uint32_t)w2->rows : 0u, ldy2, PackJobs{});
@@ -854,7 +854,9 @@ int launch_gemv_oil4_multi_batches(int nb, const int* kinds, const oilhip_weight
     const bool leave_parts = d_parts && ordered && any_ordered_parts && !wb;
     if (leave_parts && (uint64_t)parts_rows * w0.rows * std::max(ks[0], std::max(ks[1], ks[2])) > 0xFFFFFFFFull) return 1;
     const int x_aligned = ((reinterpret_cast<uintptr_t>(d_x) | reinterpret_cast<uintptr_t>(d_x2)) & 15u) == 0 && (ldx & 3u) == 0;
-    const bool parked = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb >= 128u;   // else the memory-to-memory pre-pass of small launches
+    // the LDS-parked pre-pass from 512 (tile, block) pairs on (the SwiGLU pre-pass of a MoE step: 1008), below that the
+    // memory-to-memory one (the step's first pre-pass, 288 pairs: 3 us faster that way)
+    const bool parked = (present[2] ? 2u : 1u) * bpr * (uint32_t)nb >= 512u;
     PackJobs pj{};
     pj.n = (uint32_t)nb;
     pj.wgs_per_job = parked ? (present[2] ? 2u : 1u) * bpr : tokens_of(present[2] ? 2 : present[1] ? 1 : 0) * ((bpr + 3u) / 4u);

@@ -144,7 +144,7 @@ size_t batch_scratch_bytes(int64_t D, int64_t F) {
     return std::max(gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)F, (uint64_t)D, true), gemv_oil4_multi_batches_bytes(kChunk, (uint64_t)D, (uint64_t)F, false));
 }
 
-// the most K parts a down projection (rows of F weights) is cut into, over the pass sizes; 0 when no pass size cuts it in three or more
+// the most K parts a row of F weights is cut into, over the pass sizes; 0 when no pass size cuts it in three or more
 uint32_t down_parts_max(int64_t F) {
     uint32_t m = 0;
     for (int kind = 0; kind < 3; ++kind) m = std::max(m, gemv_oil4_multi_parts(kind, (uint64_t)F));
@@ -278,12 +278,17 @@ int oilhip_moe_forward(const oilhip_weights* const* gate, const oilhip_weights* 
         // the z-loss accumulator and the slab counters at the start of the batch workspace start at zero (every launch
         // leaves the counters at zero again); outputs that row parts add into are cleared by the launch that splits
         // the activations
-        hipLaunchKernelGGL(fill_zero3_kernel, dim3(64), dim3(256), 0, s, ws.g, (size_t)0, (float*)ws.z, (size_t)2, (float*)ws.batch,
-                           kGemvBatchCounterBytes / 4);
-        OILHIP_HIP(hipGetLastError());
-        // down projections cut into three or more K parts leave the parts to the combine (ordered sums; with the
-        // atomic sums switched on they add into their outputs instead)
+        // (the launch is skipped when nothing needs it: no z-loss asked for, and no launch of the step counts arrivals --
+        // the gate/up rows are cut in at most two parts and the down projections leave their parts to the combine)
         const bool parts_mode = gemv_oil4_multi_ordered() && down_parts_max(F) > 0u;
+        const bool counters = gemv_oil4_multi_ordered() && (down_parts_max(D) > 0u || (down_parts_max(F) > 0u && !parts_mode));
+        if (z_loss || counters) {
+            hipLaunchKernelGGL(fill_zero3_kernel, dim3(64), dim3(256), 0, s, ws.g, (size_t)0, (float*)ws.z, (size_t)2, (float*)ws.batch,
+                               kGemvBatchCounterBytes / 4);
+            OILHIP_HIP(hipGetLastError());
+        }
+        // down projections cut into three or more K parts leave the parts to the combine (parts_mode: ordered sums; with
+        // the atomic sums switched on they add into their outputs instead)
         struct Batch { int e, pair0, m, kind; };
         std::vector<Batch> batches;
         for (int pass = 2; pass >= 0; --pass)                     // the longest passes first: they end last
