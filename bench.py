@@ -554,31 +554,41 @@ def bench_read_probe(torch, ia):
                     best = max(best, gbs)
     out["read_only_probe_GBps"] = round(best, 1)
     out["read_only_probe_steady_table_GBps"] = table
-    # the headline's launch pattern
+    # the GEMVs' own launch pattern: dependent launches of one tensor's bytes each over a ring of slices (graph replay),
+    # for the payload sizes of the M=1 legs -- what a kernel that did nothing with the data would score per shape
     stream = torch.cuda.Stream()
-    best_us = None
-    for (wgs, thr, u) in ((256, 512, 4), (512, 512, 4), (1024, 512, 2), (1024, 512, 4)):
-        with torch.cuda.stream(stream):
-            for c in range(copies):
-                launch(buf.data_ptr() + c * one, one, u, 1, 0, wgs, thr)
-            stream.synchronize()
-            g = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(g, stream=stream):
-                for c in range(copies):
-                    launch(buf.data_ptr() + c * one, one, u, 1, 0, wgs, thr)
-            for _ in range(3):
-                g.replay()
-            stream.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(stream)
-            for _ in range(50):
-                g.replay()
-            e1.record(stream)
-            e1.synchronize()
-        us = e0.elapsed_time(e1) * 1e3 / (50 * copies)
-        best_us = us if best_us is None else min(best_us, us)
-    out["read_only_probe_22MB_per_launch_us"] = round(best_us, 2)
-    out["read_only_probe_22MB_per_launch_GBps"] = round(one / best_us / 1e3, 1)
+    per_shape = {}
+    for label, nbytes in (("oil4_4096x4096", 4096 * 4096 // 2), ("oil8_4096x4096", 4096 * 4096 + 4096 * 16 * 4),
+                          ("oil4_11008x4096", one), ("oil4_22016x4096", 2 * one), ("oil4_131072x4096", 131072 * 4096 // 2)):
+        nbytes = (nbytes + 1023) // 1024 * 1024
+        ncopies = max(2, min(copies, buf.numel() // nbytes))
+        best_us = None
+        for (wgs, thr, u) in ((256, 512, 4), (512, 512, 4), (1024, 512, 2), (1024, 512, 4)):
+            with torch.cuda.stream(stream):
+                for c in range(ncopies):
+                    launch(buf.data_ptr() + c * nbytes, nbytes, u, 1, 0, wgs, thr)
+                stream.synchronize()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for c in range(ncopies):
+                        launch(buf.data_ptr() + c * nbytes, nbytes, u, 1, 0, wgs, thr)
+                reps = max(3, min(50, int(2.0e9 // (nbytes * ncopies))))
+                for _ in range(3):
+                    g.replay()
+                stream.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(reps):
+                    g.replay()
+                e1.record(stream)
+                e1.synchronize()
+            us = e0.elapsed_time(e1) * 1e3 / (reps * ncopies)
+            best_us = us if best_us is None else min(best_us, us)
+        per_shape[label] = {"bytes": nbytes, "us_per_launch": round(best_us, 2), "GBps": round(nbytes / best_us / 1e3, 1),
+                            "frac_of_hbm_peak": round(nbytes / best_us / 1e3 / HBM_PEAK_GBS, 4)}
+    out["read_only_probe_per_launch"] = per_shape
+    out["read_only_probe_22MB_per_launch_us"] = per_shape["oil4_11008x4096"]["us_per_launch"]
+    out["read_only_probe_22MB_per_launch_GBps"] = per_shape["oil4_11008x4096"]["GBps"]
     return out
 
 
