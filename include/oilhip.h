@@ -201,8 +201,8 @@ int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x_bf16, float* d
 
 /* The same prefill GEMM for the reference's own call: FP32 activations X[M][cols], as Qwen35Engine::prefill hands
  * them to gemm() in chunks of up to 512 tokens (src/adapters/tools/qwen35_engine.cpp:47-85,630-753).  X is rounded
- * once to bf16 on its way into the kernel's operand order (no extra pass for plain OIL4 and M > 256; otherwise
- * one conversion launch into a scratch buffer of the stream).  The result is bit for bit what oilhip_gemm_bf16
+ * once to bf16 on its way into the kernel's operand order (no extra pass for plain OIL4 and 16-byte aligned X;
+ * otherwise one conversion launch into a scratch buffer of the stream).  The result is bit for bit what oilhip_gemm_bf16
  * returns for bf16(X): relative L2 <= 2e-3 against the FP32 contraction over the rounded activations, about 2.4e-3
  * against the one over the FP32 activations themselves (both operands' roundings, Gaussian data), where
  * oilhip_gemv_f32 keeps 1e-5: a caller chooses it per call. */

@@ -597,8 +597,8 @@ int oilhip_gemm_bf16(const oilhip_weights* w, const uint16_t* d_x, float* d_y, i
 int oilhip_gemm_f32(const oilhip_weights* w, const float* d_x, float* d_y, int M, void* stream) {
     if (int rc = check_matmul_shape(w, d_x, d_y, M)) return rc;
     hipStream_t s = (hipStream_t)stream;
-    // plain OIL4, more than 256 tokens: the pre-pass of the prefill kernel rounds X on its way into fragment order
-    if (plain_oil4(*w) && M > 256 && (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0u) return launch_gemm_oil4_frag(*w, d_x, true, d_y, M, s);
+    // plain OIL4: the pre-pass of the prefill kernel rounds X on its way into fragment order
+    if (plain_oil4(*w) && (reinterpret_cast<uintptr_t>(d_x) & 15u) == 0u) return launch_gemm_oil4_frag(*w, d_x, true, d_y, M, s);
     uint16_t* xb = nullptr;
     if (int rc = launch_x_to_bf16(d_x, (uint64_t)M * w->cols, &xb, s)) return rc;
     return oilhip_gemm_bf16(w, xb, d_y, M, stream);

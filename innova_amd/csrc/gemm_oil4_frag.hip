@@ -1,4 +1,4 @@
-// gemm_oil4_frag.hip -- prefill GEMM over uniform OIL4 tensors for batches of more than 256 tokens:
+// gemm_oil4_frag.hip -- prefill GEMM over uniform OIL4 tensors (any batch size; 16-byte aligned activations):
 // Y[M][N] = X[M][K] . W^T, X in bf16 (or FP32, rounded once to bf16), W dequantized to bf16 on the fly,
 // v_mfma_f32_32x32x16_bf16 with FP32 accumulation, FP32 output.  Same contraction as the reference's FP32
 // prefill (Qwen35Engine::gemm with B up to 512, src/adapters/tools/qwen35_engine.cpp:47-85,630-753) over

@@ -52,10 +52,11 @@ def test_fragment_kernel_edges(rows, cols, M):
     assert np.all(np.isfinite(y))
 
 
-def test_fragment_kernel_takes_misaligned_activations_another_way():
+@pytest.mark.parametrize("M", [300, 64])
+def test_fragment_kernel_takes_misaligned_activations_another_way(M):
     """An activation pointer that is not 16-byte aligned cannot use the kernel's 16-byte loads: same result through
-    the older path."""
-    rows, cols, M = 256, 512, 300
+    the older paths (the pipelined kernel above 256 tokens, the 128 x 128 tiles below)."""
+    rows, cols = 256, 512
     w = gaussian_weights(rows * cols, 21)
     payload, blocks = ia.block_codec.quantize_tensor(w, ia.Format.OIL4)
     base = torch.randn(M * cols + 8, generator=torch.Generator().manual_seed(5)).to(torch.bfloat16).cuda()
