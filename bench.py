@@ -474,6 +474,10 @@ def bench_prefill(torch, ia, payload, blocks):
                     xf = x.float()
                     tf = time_calls(torch, lambda: d.gemm_f32(xf, out=y))
                     out["prefill_fp32_in_M512_N11008_us"] = round(tf * 1e6, 1)
+                    for Ms in (64, 128, 256):                                 # short prompts: chunks below the reference's cap of 512
+                        xs, ys = xf[:Ms].contiguous(), y[:Ms]
+                        ts = time_calls(torch, lambda: d.gemm_f32(xs, out=ys), min_ms=20.0)
+                        out[f"prefill_fp32_in_M{Ms}_N11008_us"] = round(ts * 1e6, 1)
     # a tensor that is not uniform OIL4 (here SPARK_Q0): decoded to bf16 slab by slab, then the same kernel over a dense operand
     ws = make_weights(11008, 4096, seed=12)
     ps, bs = ia.block_codec.quantize_tensor(ws, ia.Format.SPARK_Q0)
