@@ -112,6 +112,9 @@ struct BlockRef {
 // (src/adapters/tools/qwen35_engine.cpp:12,630-753).
 void set_prefill_min_batch(int min_batch);
 int prefill_min_batch();
+// DeviceTensor::gemm keeps the device buffers its host-pointer arguments pass through between calls (a pair per
+// thread that is inside gemm at once, grown on demand); this returns them to the driver.
+void release_staging();
 
 class DeviceTensor {
 public:

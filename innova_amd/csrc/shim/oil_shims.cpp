@@ -2,6 +2,8 @@
 #include "../../../include/oilhip_shims.hpp"
 
 #include <atomic>
+#include <mutex>
+#include <vector>
 #include <hip/hip_runtime.h>
 
 #include <cstring>
@@ -44,6 +46,50 @@ private:
 };
 
 size_t sz(long long v) { return v < 0 ? 0 : (size_t)v; }
+
+// Device staging for DeviceTensor::gemm: the reference hands over host pointers on every call (seven projections per
+// layer and token), so its activations and outputs pass through a pair of device buffers that are kept between
+// calls instead of a hipMalloc / hipFree pair per call (hipFree waits for the device).  A call leases a pair from a
+// small pool (one pair per thread that is inside gemm at the same moment); buffers grow, never shrink, and are
+// returned to the driver by release_staging().
+constexpr size_t kPinnedFloats = 64 * 1024;   // small transfers (a decode step's activations and outputs) go through pinned memory
+struct Stage { float* x = nullptr; size_t nx = 0; float* y = nullptr; size_t ny = 0; float* hx = nullptr; float* hy = nullptr; };
+std::mutex g_stage_mu;
+std::vector<Stage> g_stage_free;
+
+class StageLease {
+public:
+    StageLease(size_t nx, size_t ny) {
+        {
+            std::lock_guard<std::mutex> lk(g_stage_mu);
+            if (!g_stage_free.empty()) { s_ = g_stage_free.back(); g_stage_free.pop_back(); }
+        }
+        grow(s_.x, s_.nx, nx);
+        grow(s_.y, s_.ny, ny);
+        if (!s_.hx) {                                                  // pinned host memory is allocated, never registered
+            hip_ok(hipHostMalloc(reinterpret_cast<void**>(&s_.hx), kPinnedFloats * sizeof(float), hipHostMallocDefault), "hipHostMalloc");
+            hip_ok(hipHostMalloc(reinterpret_cast<void**>(&s_.hy), kPinnedFloats * sizeof(float), hipHostMallocDefault), "hipHostMalloc");
+        }
+    }
+    ~StageLease() {
+        std::lock_guard<std::mutex> lk(g_stage_mu);
+        g_stage_free.push_back(s_);
+    }
+    StageLease(const StageLease&) = delete;
+    StageLease& operator=(const StageLease&) = delete;
+    float* x() const { return s_.x; }
+    float* y() const { return s_.y; }
+    float* hx() const { return s_.hx; }
+    float* hy() const { return s_.hy; }
+private:
+    static void grow(float*& p, size_t& have, size_t want) {
+        if (want <= have) return;
+        if (p) { (void)hipFree(p); p = nullptr; have = 0; }
+        hip_ok(hipMalloc(&p, want * sizeof(float)), "hipMalloc");
+        have = want;
+    }
+    Stage s_;
+};
 
 }  // namespace
 
@@ -251,13 +297,40 @@ static std::atomic<int> g_prefill_min_batch{0};
 void set_prefill_min_batch(int min_batch) { g_prefill_min_batch.store(min_batch < 0 ? 0 : min_batch, std::memory_order_relaxed); }
 int prefill_min_batch() { return g_prefill_min_batch.load(std::memory_order_relaxed); }
 
+void release_staging() {
+    std::lock_guard<std::mutex> lk(g_stage_mu);
+    for (Stage& s : g_stage_free) {
+        if (s.x) (void)hipFree(s.x);
+        if (s.y) (void)hipFree(s.y);
+        if (s.hx) (void)hipHostFree(s.hx);
+        if (s.hy) (void)hipHostFree(s.hy);
+    }
+    g_stage_free.clear();
+}
+
 void DeviceTensor::gemm(const float* X, float* Y, int B) const {
     if (B <= 0) return;
-    Dev<float> x(X, (size_t)B * cols_), y(nullptr, (size_t)B * rows_);
+    const size_t nx = (size_t)B * cols_, ny = (size_t)B * rows_;
+    StageLease st(nx, ny);
+    // a decode step's few KB travel through pinned memory with asynchronous copies and one wait at the end; large
+    // batches are copied straight from and to the caller's memory
+    const bool small = nx <= kPinnedFloats && ny <= kPinnedFloats;
+    if (small) {
+        std::memcpy(st.hx(), X, nx * sizeof(float));
+        hip_ok(hipMemcpyAsync(st.x(), st.hx(), nx * sizeof(float), hipMemcpyHostToDevice, nullptr), "hipMemcpyAsync H2D");
+    } else {
+        hip_ok(hipMemcpy(st.x(), X, nx * sizeof(float), hipMemcpyHostToDevice), "hipMemcpy H2D");
+    }
     const int pmin = prefill_min_batch();
-    if (pmin > 0 && B >= pmin) ok(oilhip_gemm_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm (prefill)");
-    else ok(oilhip_gemv_f32(static_cast<oilhip_weights*>(handle_), x.get(), y.get(), B, nullptr), "gemm");
-    y.to_host(Y);
+    if (pmin > 0 && B >= pmin) ok(oilhip_gemm_f32(static_cast<oilhip_weights*>(handle_), st.x(), st.y(), B, nullptr), "gemm (prefill)");
+    else ok(oilhip_gemv_f32(static_cast<oilhip_weights*>(handle_), st.x(), st.y(), B, nullptr), "gemm");
+    if (small) {
+        hip_ok(hipMemcpyAsync(st.hy(), st.y(), ny * sizeof(float), hipMemcpyDeviceToHost, nullptr), "hipMemcpyAsync D2H");
+        hip_ok(hipStreamSynchronize(nullptr), "hipStreamSynchronize");
+        std::memcpy(Y, st.hy(), ny * sizeof(float));
+    } else {
+        hip_ok(hipMemcpy(Y, st.y(), ny * sizeof(float), hipMemcpyDeviceToHost), "hipMemcpy D2H");
+    }
 }
 
 void DeviceTensor::dequantize(float* out) const {

@@ -2,6 +2,7 @@
 // its kernels (tests/test_kernel.cpp:82-103, tests/test_quant_engines.cpp:229-263,
 // tests/test_block_codec.cpp), with results checked against brute-force double loops.
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -182,6 +183,17 @@ int main() {
         const double e2 = check(8, 1e-5, "gemm B=8 below the prefill threshold");
         CHECK(e1 > 1e-5, "B=512 with the threshold set should have run on the bf16 kernel (rel-L2 %.3g)", e1);
         std::printf("DeviceTensor::gemm 11008x4096: B=512 fp32 %.2g, B=512 prefill %.2g, B=8 %.2g\n", e0, e1, e2);
+        {   // host-pointer calls in a row, as the engine's decode loop makes them (the staging buffers are kept between calls)
+            std::vector<float> X(cols, 0.25f), Y(rows);
+            for (int i = 0; i < 5; ++i) t.gemm(X.data(), Y.data(), 1);
+            const auto t0 = std::chrono::steady_clock::now();
+            for (int i = 0; i < 200; ++i) t.gemm(X.data(), Y.data(), 1);
+            const double us = std::chrono::duration<double, std::micro>(std::chrono::steady_clock::now() - t0).count() / 200.0;
+            std::printf("DeviceTensor::gemm 11008x4096, B=1, host pointers: %.1f us per call\n", us);
+            gfx950::release_staging();
+            t.gemm(X.data(), Y.data(), 1);                        // allocates afresh after a release
+            CHECK(std::isfinite(Y[0]), "gemm after release_staging");
+        }
         gfx950::set_prefill_min_batch(0);
     }
     {   // OIL4KVCache: prefill + two decode appends; ranges are slices of the whole, the static pair round-trips
